@@ -1,0 +1,195 @@
+/*
+ * TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * CPU restatement of the arithmetic and index math of Fairring's K-way
+ * gradient-slice reduction. Only tests, the smoke check and the benchmark's
+ * CPU-baseline leg may link or call this file; the shipped library never does.
+ *
+ * What each function follows in the reference tree (paths relative to it):
+ *   orc_sum_f32 / orc_sum_bf16 / orc_max_*  -> fairring/device.cc:108-131
+ *       (doReduction: result = reduce over dim 0 of operand[K, n]); the order
+ *       of additions is the sequential at::add chain acc = x[0];
+ *       acc = acc + x[k] for k = 1..K-1, which is the contract this build is
+ *       held to (the reference delegates the arithmetic to ATen).
+ *   orc_compute_layout                       -> fairring/utils.h:288-327
+ *   orc_ceil_of_ratio / round helpers        -> fairring/utils.h:258-274
+ *   orc_num_slices / orc_slice_bounds        -> fairring/device.cc:315-326
+ *   orc_readme_layout                        -> README.md:61-62 (the
+ *       FAIRRING_TOTAL_MEMORY / FAIRRING_SLICE_SIZE pair)
+ *
+ * Pinned by (see tests/test_oracle.py): the installed ATen's add chain and
+ * sum(dim=0) (K <= 17) bit for bit, ATen's bf16 sum over dim 0, an exact
+ * rational-arithmetic brute force with explicit round-to-nearest-even on tiny
+ * inputs, the all-ones and arange known answers of
+ * benchmark/benchmark.cc:130-186, and hand-evaluated layout/slicing tables.
+ *
+ * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off, optional OpenMP).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <string.h>
+
+#define ORC_SCALE_NONE 0 /* out = acc */
+#define ORC_SCALE_MUL 1  /* out = acc * scale   (scale = 1/K, exact for K=2^p) */
+#define ORC_SCALE_DIV 2  /* out = acc / scale   (scale = K, at::div semantics) */
+
+static inline float apply_scale(float acc, int mode, float scale) {
+  if (mode == ORC_SCALE_MUL) return acc * scale;
+  if (mode == ORC_SCALE_DIV) return acc / scale;
+  return acc;
+}
+
+/* fp32: left fold in contribution order starting from x[0] (not from 0). */
+void orc_sum_f32(float* out, const float* const* in, int K, int64_t n,
+                 int scale_mode, float scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = in[0][i];
+    for (int k = 1; k < K; ++k) acc = acc + in[k][i];
+    out[i] = apply_scale(acc, scale_mode, scale);
+  }
+}
+
+/* Same chain, blocked over contributions the way a streaming CPU
+ * implementation would run it (acc = x0; acc += xk ...), used as the timed
+ * CPU baseline. Bit-identical to orc_sum_f32. */
+void orc_sum_f32_chain(float* out, const float* const* in, int K, int64_t n,
+                       int scale_mode, float scale) {
+#pragma omp parallel
+  {
+    const int64_t B = 4096;
+#pragma omp for schedule(static)
+    for (int64_t b = 0; b < (n + B - 1) / B; ++b) {
+      int64_t lo = b * B, hi = lo + B < n ? lo + B : n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = in[0][i];
+      for (int k = 1; k < K; ++k)
+        for (int64_t i = lo; i < hi; ++i) out[i] = out[i] + in[k][i];
+      if (scale_mode != ORC_SCALE_NONE)
+        for (int64_t i = lo; i < hi; ++i)
+          out[i] = apply_scale(out[i], scale_mode, scale);
+    }
+  }
+}
+
+static inline float bf16_to_f32(uint16_t b) {
+  uint32_t u = ((uint32_t)b) << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* Round-to-nearest-even fp32 -> bf16, NaN -> 0x7FC0. */
+static inline uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+  uint32_t bias = 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)((u + bias) >> 16);
+}
+
+/* bf16 storage: exact upcast, fp32 accumulation in contribution order, scale
+ * in fp32, one rounding on store. */
+void orc_sum_bf16(uint16_t* out, const uint16_t* const* in, int K, int64_t n,
+                  int scale_mode, float scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = bf16_to_f32(in[0][i]);
+    for (int k = 1; k < K; ++k) acc = acc + bf16_to_f32(in[k][i]);
+    out[i] = f32_to_bf16_rne(apply_scale(acc, scale_mode, scale));
+  }
+}
+
+/* MAX with NaN propagation (ATen amax): any NaN in a lane gives NaN. */
+static inline float max_nan(float a, float b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  return a > b ? a : b;
+}
+
+void orc_max_f32(float* out, const float* const* in, int K, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = in[0][i];
+    for (int k = 1; k < K; ++k) acc = max_nan(acc, in[k][i]);
+    out[i] = acc;
+  }
+}
+
+void orc_max_bf16(uint16_t* out, const uint16_t* const* in, int K, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = bf16_to_f32(in[0][i]);
+    for (int k = 1; k < K; ++k) acc = max_nan(acc, bf16_to_f32(in[k][i]));
+    out[i] = f32_to_bf16_rne(acc);
+  }
+}
+
+/* ---- integer helpers -------------------------------------------------- */
+
+int64_t orc_ceil_of_ratio(int64_t num, int64_t den) {
+  if (num == 0) return 0;
+  return (num - 1) / den + 1;
+}
+
+int64_t orc_round_down(int64_t val, int64_t factor) {
+  return (val / factor) * factor;
+}
+
+int64_t orc_round_up(int64_t val, int64_t factor) {
+  return orc_ceil_of_ratio(val, factor) * factor;
+}
+
+#define ORC_ALIGNMENT 8
+
+/* out4 = {slotSizeInBytes, sliceSizeInBytes, numPaddingSlots, numStagingSlots}.
+ * Returns 0, or 1/2 where the reference terminates (first/second check). */
+int orc_compute_layout(int64_t max_mem, int64_t max_pad, int64_t min_par,
+                       int64_t num_machines, int64_t devs_per_machine,
+                       int64_t* out4) {
+  int64_t one_pad = devs_per_machine * num_machines * ORC_ALIGNMENT;
+  int64_t num_pad_slots = max_pad / one_pad;
+  if (!(min_par <= num_pad_slots)) return 1;
+  int64_t slice = INT64_MAX, slot = 0, num_staging = 0;
+  if (devs_per_machine == 1) {
+    int64_t pad_mem = 2 * min_par * devs_per_machine * num_machines * ORC_ALIGNMENT;
+    if (!(pad_mem <= max_mem)) return 2;
+    slot = orc_round_down((max_mem - pad_mem) / min_par,
+                          devs_per_machine * num_machines * ORC_ALIGNMENT);
+    slice = slot * devs_per_machine;
+    num_staging = min_par;
+    num_pad_slots = min_par;
+  }
+  out4[0] = slot;
+  out4[1] = slice;
+  out4[2] = num_pad_slots;
+  out4[3] = num_staging;
+  return 0;
+}
+
+/* README regime: number of staging slots that TOTAL_MEMORY holds. */
+int64_t orc_readme_layout(int64_t total_memory, int64_t slice_size) {
+  return total_memory / slice_size;
+}
+
+int64_t orc_num_slices(int64_t numel, int64_t slice_bytes, int64_t elsize) {
+  int64_t max_elems = slice_bytes / elsize;
+  return orc_ceil_of_ratio(numel, max_elems);
+}
+
+/* bounds2 = {offsetInElems, sliceSizeInElems} of slice idx. */
+void orc_slice_bounds(int64_t numel, int64_t slice_bytes, int64_t elsize,
+                      int64_t idx, int64_t* bounds2) {
+  int64_t max_elems = slice_bytes / elsize;
+  int64_t off = idx * max_elems;
+  int64_t rem = numel - off;
+  bounds2[0] = off;
+  bounds2[1] = max_elems < rem ? max_elems : rem;
+}
+
+/* ---- thread control for the timed baseline ----------------------------- */
+#ifdef _OPENMP
+#include <omp.h>
+void orc_set_threads(int n) { omp_set_num_threads(n); }
+int orc_max_threads(void) { return omp_get_max_threads(); }
+#else
+void orc_set_threads(int n) { (void)n; }
+int orc_max_threads(void) { return 1; }
+#endif

@@ -1,0 +1,248 @@
+"""Pins the CPU oracle (test infrastructure) before anything is compared to it.
+
+Checks, none of which retypes the oracle's own formula:
+  * golden vectors written by the installed ATen (tests/golden/make_golden.py)
+  * live torch.add chain and torch.sum(dim=0) (K <= 17) from the installed torch
+  * ATen's bf16 sum over dim 0 (fp32 accumulate, one rounding)
+  * exact rational arithmetic + explicit round-to-nearest-even on tiny inputs
+  * the all-ones / arange known answers of benchmark/benchmark.cc:130-186
+  * closed forms for the layout and slicing (fairring/utils.h:258-327,
+    fairring/device.cc:315-326)
+"""
+import struct
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal
+
+F32_CASES = ["f32_k2", "f32_k3", "f32_k8", "f32_k17", "f32_k64"]
+BF16_CASES = ["bf16_k2", "bf16_k8", "bf16_k64"]
+
+
+@pytest.mark.parametrize("case", F32_CASES)
+def test_f32_matches_golden(golden, case):
+    x = golden[case + "_in"]
+    k = x.shape[0]
+    assert_bits_equal(oracle.sum_f32(list(x)), golden[case + "_sum"], case)
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_MUL, 1.0 / k),
+                      golden[case + "_mul"], case + " mul")
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k)),
+                      golden[case + "_div"], case + " div")
+    # the numpy restatement and the blocked multi-threaded chain agree too
+    assert_bits_equal(oracle.np_sum_f32(list(x)), golden[case + "_sum"], case + " np")
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k), chain=True, threads=4),
+                      golden[case + "_div"], case + " chain")
+
+
+@pytest.mark.parametrize("case", BF16_CASES)
+def test_bf16_matches_golden(golden, case):
+    x = golden[case + "_in"]
+    k = x.shape[0]
+    assert_bits_equal(oracle.sum_bf16(list(x)), golden[case + "_sum"], case)
+    assert_bits_equal(oracle.sum_bf16(list(x), oracle.SCALE_MUL, 1.0 / k),
+                      golden[case + "_mul"], case + " mul")
+    assert_bits_equal(oracle.sum_bf16(list(x), oracle.SCALE_DIV, float(k)),
+                      golden[case + "_div"], case + " div")
+    assert_bits_equal(oracle.np_sum_bf16(list(x), oracle.SCALE_MUL, 1.0 / k),
+                      golden[case + "_mul"], case + " np")
+
+
+@pytest.mark.parametrize("k", [2, 3, 8, 15, 16, 17, 32, 64])
+def test_f32_matches_live_torch_chain(k):
+    rng = np.random.default_rng(100 + k)
+    x = (rng.standard_normal((k, 20011)) * 0.01).astype(np.float32)
+    t = torch.from_numpy(x)
+    acc = t[0].clone()
+    for i in range(1, k):
+        acc = torch.add(acc, t[i])
+    assert_bits_equal(oracle.sum_f32(list(x)), acc.numpy(), "chain k=%d" % k)
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k)),
+                      torch.div(acc, float(k)).numpy(), "div k=%d" % k)
+    if k <= 17:
+        # ATen's CPU sum over dim 0 keeps the sequential order up to K = 17 in
+        # its vectorised body; the ragged tail lanes (numel % 64) go through a
+        # multi-accumulator scalar loop that regroups, so they are left out.
+        body = (x.shape[1] // 64) * 64
+        assert_bits_equal(oracle.sum_f32(list(x))[:body],
+                          torch.sum(t, dim=0).numpy()[:body], "sum_out k=%d" % k)
+
+
+@pytest.mark.parametrize("k", [2, 8, 64])
+def test_bf16_matches_aten_sum(k):
+    rng = np.random.default_rng(200 + k)
+    t = torch.from_numpy((rng.standard_normal((k, 10007)) * 0.01).astype(np.float32)).to(torch.bfloat16)
+    bits = t.view(torch.int16).numpy().view(np.uint16)
+    want = torch.sum(t, dim=0).view(torch.int16).numpy().view(np.uint16)
+    assert_bits_equal(oracle.sum_bf16(list(bits)), want, "bf16 sum k=%d" % k)
+
+
+def test_pow2_mul_equals_div_and_ddp_predivision():
+    # For K = 2^p and no subnormal results, acc*(1/K) == acc/K == sum of x/K.
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal((8, 50000)) * 0.01).astype(np.float32)
+    a = oracle.sum_f32(list(x), oracle.SCALE_MUL, 0.125)
+    b = oracle.sum_f32(list(x), oracle.SCALE_DIV, 8.0)
+    c = oracle.sum_f32(list(x / np.float32(8)))
+    assert_bits_equal(a, b)
+    assert_bits_equal(a, c)
+
+
+# ---- exact brute force ---------------------------------------------------------
+
+def _f32_from_fraction(q):
+    """Round an exact rational to binary32, round-to-nearest-even."""
+    if q == 0:
+        return 0.0
+    sign = -1 if q < 0 else 1
+    a = abs(q)
+    e = a.numerator.bit_length() - a.denominator.bit_length()
+    if Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, -126)
+    ulp = Fraction(2) ** (e - 23)
+    m = a / ulp
+    fl = m.numerator // m.denominator
+    rem = m - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and (fl & 1)):
+        fl += 1
+    val = fl * ulp
+    if val >= Fraction(2) ** 128:
+        return sign * float("inf")
+    return sign * float(val)
+
+
+def _exact_chain(col):
+    acc = Fraction(float(col[0]))
+    for v in col[1:]:
+        acc = Fraction(_f32_from_fraction(acc + Fraction(float(v))))
+    return _f32_from_fraction(acc)
+
+
+def test_f32_brute_force_exact_rationals():
+    rng = np.random.default_rng(3)
+    k, n = 9, 300
+    # wide exponent spread so that rounding happens at every step
+    x = (rng.standard_normal((k, n)) * np.exp(rng.uniform(-30, 30, (k, n)))).astype(np.float32)
+    x[:, 0] = np.float32(1e-45)
+    x[:, 1] = [np.float32(2.0 ** 24)] + [np.float32(1.0)] * (k - 1)
+    x[:, 2] = [np.float32(1.0)] * (k - 1) + [np.float32(2.0 ** 24)]
+    want = np.array([_exact_chain(x[:, i]) for i in range(n)], np.float32)
+    assert_bits_equal(oracle.sum_f32(list(x)), want, "brute force")
+
+
+def test_bf16_rounding_against_struct():
+    # every bf16 midpoint neighbourhood: compare the RNE pack with exact rationals
+    rng = np.random.default_rng(5)
+    vals = rng.standard_normal(2000).astype(np.float32)
+    vals[:6] = [1.00390625, 1.01171875, 1.0078125, -1.00390625, 3.3895314e38, 1e-40]
+    got = oracle.np_f32_to_bf16_rne(vals)
+    for v, g in zip(vals, got):
+        u = struct.unpack("<I", struct.pack("<f", float(v)))[0]
+        lo = u & 0xFFFF0000
+        hi = lo + 0x10000
+        flo = struct.unpack("<f", struct.pack("<I", lo))[0]
+        fhi = struct.unpack("<f", struct.pack("<I", hi & 0xFFFFFFFF))[0]
+        if np.isinf(fhi) or np.isnan(fhi):
+            # top binade: the next bf16 up is the infinity encoding, whose
+            # "value" for rounding purposes is 2^128
+            fhi_q = Fraction(2) ** 128 * (1 if v > 0 else -1)
+        else:
+            fhi_q = Fraction(fhi)
+        dlo = abs(Fraction(float(v)) - Fraction(flo))
+        dhi = abs(fhi_q - Fraction(float(v)))
+        if dlo < dhi:
+            want = lo >> 16
+        elif dhi < dlo:
+            want = (hi >> 16) & 0xFFFF
+        else:
+            want = (lo >> 16) if ((lo >> 16) & 1) == 0 else (hi >> 16) & 0xFFFF
+        assert int(g) == want, (v, hex(int(g)), hex(want))
+
+
+# ---- known answers from the reference's benchmark --------------------------------
+
+@pytest.mark.parametrize("k", [2, 8, 64])
+def test_all_ones_kat(k):
+    x = np.ones((k, 4097), np.float32)
+    assert (oracle.sum_f32(list(x)) == np.float32(k)).all()
+    ones_bf16 = np.full((k, 4097), 0x3F80, np.uint16)
+    assert (oracle.sum_bf16(list(ones_bf16)) == oracle.np_f32_to_bf16_rne(np.full(1, k, np.float32))[0]).all()
+
+
+def test_arange_kat():
+    k, n = 8, 100000  # n*k < 2^24 so every partial sum is exact
+    base = np.arange(n, dtype=np.float32)
+    got = oracle.sum_f32([base] * k)
+    assert_bits_equal(got, base * np.float32(k))
+
+
+def test_max_semantics():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((5, 1000)).astype(np.float32)
+    x[2, 3] = np.nan
+    x[:, 4] = [-0.0, 0.0, -0.0, 0.0, -0.0]
+    want = torch.amax(torch.from_numpy(x), dim=0).numpy()
+    got = oracle.max_f32(list(x))
+    assert np.isnan(got[3]) and np.isnan(want[3])
+    m = np.ones(1000, bool)
+    m[3] = m[4] = False  # sign of a zero maximum is not specified
+    assert_bits_equal(got[m], want[m])
+    assert got[4] == 0.0
+
+
+# ---- layout and slicing ---------------------------------------------------------------
+
+MiB = 1024 * 1024
+
+
+def test_compute_layout_known_answers():
+    assert oracle.compute_layout(50 * MiB, MiB, 16, 1, 1) == dict(
+        slot=3276784, slice=3276784, padding_slots=16, staging_slots=16)
+    assert oracle.compute_layout(50 * MiB, MiB, 16, 8, 1) == dict(
+        slot=3276672, slice=3276672, padding_slots=16, staging_slots=16)
+    assert oracle.compute_layout(50 * MiB, MiB, 2, 1, 1) == dict(
+        slot=26214384, slice=26214384, padding_slots=2, staging_slots=2)
+    lay = oracle.compute_layout(50 * MiB, MiB, 16, 4, 8)
+    assert lay == dict(slot=0, slice=2 ** 63 - 1, padding_slots=4096, staging_slots=0)
+    with pytest.raises(ValueError):
+        oracle.compute_layout(50 * MiB, 64, 16, 1, 1)   # 64/8 = 8 padding slots < 16
+    with pytest.raises(ValueError):
+        oracle.compute_layout(100, MiB, 16, 1, 1)        # padding alone exceeds the pool
+
+
+def test_compute_layout_hand_formula():
+    # independent evaluation of the D == 1 branch with Python integers
+    for total, par, m in [(50 * MiB, 16, 1), (123456789, 7, 3), (MiB, 1, 64)]:
+        unit = m * 8
+        slot = ((total - 2 * par * unit) // par) // unit * unit
+        lay = oracle.compute_layout(total, MiB, par, m, 1)
+        assert lay["slot"] == slot and lay["slice"] == slot
+        assert lay["staging_slots"] == par and lay["padding_slots"] == par
+
+
+def test_slicing_known_answers():
+    S = 25 * MiB
+    assert oracle.num_slices(1_370_000_000, S, 4) == 210
+    assert oracle.slice_bounds(1_370_000_000, S, 4, 209) == (209 * 6_553_600, 297_600)
+    assert oracle.num_slices(1_300_000_000, S, 2) == 100
+    assert oracle.slice_bounds(1_300_000_000, S, 2, 99) == (99 * 13_107_200, 2_387_200)
+    assert oracle.num_slices(0, S, 4) == 0
+    assert oracle.num_slices(6_553_600, S, 4) == 1
+    assert oracle.num_slices(6_553_601, S, 4) == 2
+    assert oracle.slice_bounds(6_553_601, S, 4, 1) == (6_553_600, 1)
+    assert oracle.lib().orc_readme_layout(50 * MiB, 25 * MiB) == 2
+
+
+def test_slices_tile_the_tensor():
+    for numel, sb, es in [(1000, 96, 4), (1001, 96, 4), (5, 8, 2), (12345, 1000, 2)]:
+        n = oracle.num_slices(numel, sb, es)
+        pos = 0
+        for i in range(n):
+            off, ln = oracle.slice_bounds(numel, sb, es, i)
+            assert off == pos and 0 < ln <= sb // es
+            pos += ln
+        assert pos == numel
