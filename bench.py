@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the K-way gradient-slice reduction on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (the configuration the metric is quoted on): K = 8 simulated rank
+contributions of a 1.37 G-element fp32 gradient, N(0, sigma = 0.01) from a
+fixed seed, reduced in contribution order with the divide-by-8 fused into the
+store, processed as 25 MiB slices (210 of them, the last 297,600 elements)
+into one output buffer. A step is one pass over the whole gradient; inputs are
+resident in HBM before the timed region starts. Bytes counted per step are the
+algorithmic ones: (K + 1) * numel * 4 = 49.32 GB.
+
+Prints one JSON line with the whole-job GB/s, the roofline of the reduction
+kernel (algorithmic bytes per launch / average launch duration from HIP events
+on the kernel's own stream) and a CPU baseline timed on this host's cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MiB = 1024 * 1024
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--numel", type=int, default=1_370_000_000)
+    ap.add_argument("--k", type=int, default=8)
+    ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
+    ap.add_argument("--total-memory", type=int, default=50 * MiB)
+    ap.add_argument("--streams", type=int, default=0, help="reduce streams (0 = library default)")
+    ap.add_argument("--blocks-per-cu", type=int, default=0)
+    ap.add_argument("--xcd-remap", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-slices", type=int, default=8)
+    return ap.parse_args()
+
+
+def check_parity(fa, oracle, np, torch, xs, out, numel, slice_elems, k):
+    """Bit-compare the first, a middle and the ragged last slice with the oracle
+    fed the very bytes the GPU read."""
+    n_slices = (numel + slice_elems - 1) // slice_elems
+    checked = []
+    for idx in sorted({0, n_slices // 2, n_slices - 1}):
+        lo = idx * slice_elems
+        hi = min(numel, lo + slice_elems)
+        host = [x[lo:hi].cpu().numpy() for x in xs]
+        want = oracle.sum_f32(host, oracle.SCALE_MUL, 1.0 / k, threads=os.cpu_count() or 1)
+        got = out[lo:hi].cpu().numpy()
+        if not (got.view(np.uint32) == want.view(np.uint32)).all():
+            raise SystemExit("parity FAILED on slice %d" % idx)
+        checked.append(idx)
+    return checked
+
+
+def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_slices_sample):
+    """The contract's reduction on this host's cores: torch's at::add chain
+    (acc = x0; acc += xk; acc /= K) over `n_slices_sample` distinct 25 MiB
+    slices copied back from the GPU; >= 3 warm-up and 10 timed passes, median.
+    The repository's C restatement (OpenMP) is timed beside it."""
+    host = [[x[i * slice_elems:(i + 1) * slice_elems].cpu() for x in xs]
+            for i in range(n_slices_sample)]
+    threads = torch.get_num_threads()
+    acc = torch.empty(slice_elems, dtype=torch.float32)
+
+    def one_pass():
+        for sl in host:
+            acc.copy_(sl[0])
+            for c in sl[1:]:
+                acc.add_(c)
+            acc.div_(float(k))
+
+    for _ in range(3):
+        one_pass()
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    algo_bytes = (k + 1) * slice_elems * 4 * n_slices_sample
+    torch_gbps = algo_bytes / med / 1e9
+
+    hnp = [[c.numpy() for c in sl] for sl in host]
+    cores = os.cpu_count() or 1
+    for sl in hnp[:2]:
+        oracle.sum_f32(sl, oracle.SCALE_DIV, float(k), chain=True, threads=cores)
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        for sl in hnp:
+            oracle.sum_f32(sl, oracle.SCALE_DIV, float(k), chain=True, threads=cores)
+        times.append(time.perf_counter() - t0)
+    c_gbps = algo_bytes / sorted(times)[len(times) // 2] / 1e9
+    return {
+        "value": round(torch_gbps, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "%d distinct 25 MiB slices x K=%d fp32, torch CPU at::add chain + div, "
+                  "median of 10 passes, %d torch threads of %d host cpus; same algorithmic-bytes "
+                  "formula" % (n_slices_sample, k, threads, cores),
+        "c_oracle_gbps": round(c_gbps, 2), "c_oracle_threads": cores,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import fairring_amd as fa
+    from fairring_amd import _capi
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    _capi.lib()  # fail now if the HIP library is missing
+    if args.blocks_per_cu or args.xcd_remap:
+        _capi.lib().frg_set_tuning(args.blocks_per_cu, args.xcd_remap)
+
+    k, numel = args.k, args.numel
+    slice_elems = args.slice_bytes // 4
+    n_slices = (numel + slice_elems - 1) // slice_elems
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams)
+
+    g = torch.Generator(device="cuda:0")
+    xs = []
+    for r in range(k):
+        g.manual_seed(20240 + r)
+        xs.append(torch.empty(numel, dtype=torch.float32, device="cuda:0")
+                  .normal_(0.0, 0.01, generator=g))
+    out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    torch.cuda.synchronize()
+
+    def step():
+        return dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+
+    for _ in range(args.warmup):
+        step().wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    w = None
+    for _ in range(args.steps):
+        w = step()
+    w.wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    step_bytes = (k + 1) * numel * 4
+    value = step_bytes * args.steps / elapsed / 1e9
+
+    # Roofline of the dominant kernel: the same steps again with a timing event
+    # before and after every launch, on the stream the launch goes to.
+    dev.set_profiling(True)
+    prof_steps = max(1, min(args.steps, 5))
+    for _ in range(prof_steps):
+        step()
+    times_ms = dev.kernel_times_ms()
+    dev.set_profiling(False)
+    assert len(times_ms) == prof_steps * n_slices, (len(times_ms), n_slices)
+    # full 25 MiB slices only: the ragged last launch of each step is left out
+    full = [t for i, t in enumerate(times_ms) if (i % n_slices) != n_slices - 1 or
+            numel % slice_elems == 0]
+    avg_ms = sum(full) / len(full)
+    launch_bytes = (k + 1) * slice_elems * 4
+    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+
+    checked = check_parity(fa, __import__("oracle"), np, torch, xs, out, numel, slice_elems, k)
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_traffic.json")
+    if os.path.exists(tpath) and k == 8 and args.slice_bytes == 25 * MiB:
+        with open(tpath) as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+
+    result = {
+        "metric": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic: N(0, sigma=0.01) per contribution from fixed seeds, resident in HBM",
+        "config": {
+            "workload": "K=%d contributions x %d fp32 elements, %d slices of %d B, fused x1/%d, "
+                        "one output buffer (BASELINE configs[1])" % (k, numel, n_slices,
+                                                                      args.slice_bytes, k),
+            "k": k, "numel": numel, "slice_bytes": args.slice_bytes,
+            "staging_total_bytes": args.total_memory, "layout": dev.layout,
+            "reduce_streams": args.streams or "default",
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "parity": "bit-exact vs CPU oracle on slices %s" % checked,
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "kernel": "ksumKernel<F32Vec, SUM, K=8>", "launch_bytes": launch_bytes,
+            "avg_launch_us": round(avg_ms * 1e3, 3), "launches_timed": len(full),
+        },
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        result["cpu_baseline"] = cpu_baseline(oracle, np, torch, xs, slice_elems, k,
+                                              min(args.cpu_slices, max(1, n_slices - 1)))
+    dev.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,94 @@
+"""ctypes binding of the C ABI in include/fairring_hip.h.
+
+Loading fails loudly when libfairring_hip.so has not been built: there is no
+CPU or eager fallback behind this module.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libfairring_hip.so")
+
+OK, ERR_INVALID, ERR_HIP, ERR_LAYOUT, ERR_UNSUPPORTED, ERR_NOT_READY = range(6)
+F32, BF16 = 0, 1
+SUM, MAX = 0, 1
+SCALE_NONE, SCALE_MUL, SCALE_DIV = 0, 1, 2
+
+# every symbol include/fairring_hip.h declares
+EXPORTS = (
+    "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_reduce_slice",
+    "frg_create", "frg_destroy", "frg_get_layout", "frg_allreduce", "frg_allreduce_host",
+    "frg_work_wait", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
+    "frg_synchronize", "frg_set_profiling", "frg_kernel_times", "frg_set_tuning",
+    "frg_last_error", "frg_version",
+)
+
+
+class FairringError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("fairring error %d: %s" % (code, message))
+        self.code = code
+
+
+class Layout(ctypes.Structure):
+    _fields_ = [("slot_size_in_bytes", ctypes.c_int64),
+                ("slice_size_in_bytes", ctypes.c_int64),
+                ("num_padding_slots", ctypes.c_int64),
+                ("num_staging_slots", ctypes.c_int64)]
+
+
+class Options(ctypes.Structure):
+    _fields_ = [("max_memory_allocated_in_bytes", ctypes.c_int64),
+                ("max_padding_allocated_in_bytes", ctypes.c_int64),
+                ("min_parallelism", ctypes.c_int64),
+                ("slice_size_in_bytes", ctypes.c_int64),
+                ("num_machines", ctypes.c_int64),
+                ("num_reduce_streams", ctypes.c_int32),
+                ("reserved", ctypes.c_int32)]
+
+
+DONE_FN = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p)
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python -m fairring_amd.build` "
+            "(there is no fallback implementation)" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+    pvp = ctypes.POINTER(ctypes.c_void_p)
+    L.frg_compute_layout.argtypes = [i64, i64, i64, i64, i64, ctypes.POINTER(Layout)]
+    L.frg_num_slices.argtypes = [i64, i64, i64]
+    L.frg_num_slices.restype = i64
+    L.frg_slice_bounds.argtypes = [i64, i64, i64, i64, ctypes.POINTER(i64), ctypes.POINTER(i64)]
+    L.frg_reduce_slice.argtypes = [vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp]
+    L.frg_create.argtypes = [i32, ctypes.POINTER(Options), pvp]
+    L.frg_destroy.argtypes = [vp]
+    L.frg_get_layout.argtypes = [vp, ctypes.POINTER(Layout)]
+    for fn in (L.frg_allreduce, L.frg_allreduce_host):
+        fn.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize):
+        fn.argtypes = [vp]
+    L.frg_work_block_stream.argtypes = [vp, vp]
+    L.frg_set_profiling.argtypes = [vp, i32]
+    L.frg_kernel_times.argtypes = [vp, ctypes.POINTER(ctypes.c_float), i32, ctypes.POINTER(i32)]
+    L.frg_set_tuning.argtypes = [i32, i32]
+    L.frg_last_error.restype = ctypes.c_char_p
+    L.frg_version.restype = ctypes.c_char_p
+    _lib = L
+    return L
+
+
+def check(rc):
+    if rc != OK:
+        raise FairringError(rc, lib().frg_last_error().decode("utf-8", "replace"))
+
+
+def ptr_table(ptrs):
+    return (ctypes.c_void_p * len(ptrs))(*ptrs)

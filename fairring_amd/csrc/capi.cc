@@ -1,0 +1,221 @@
+// The C ABI declared in include/fairring_hip.h: argument checks, error strings
+// and nothing else; the work is in pipeline.cc and ksum_kernels.hip.
+#include <string>
+
+#include "../../include/fairring_hip.h"
+#include "ksum_kernels.h"
+#include "layout.h"
+#include "pipeline.h"
+
+using frg::Context;
+using frg::Work;
+
+namespace {
+
+int fail(int code, const std::string& msg) {
+  frg::setLastError(msg);
+  return code;
+}
+
+Context* asCtx(frg_ctx* c) { return reinterpret_cast<Context*>(c); }
+Work* asWork(frg_work* w) { return reinterpret_cast<Work*>(w); }
+
+int submitCommon(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
+                 int dtype, int op, int scale_mode, float scale, void* producer_stream,
+                 frg_done_fn done, void* user, frg_work** work, bool fromHost) {
+  if (work) *work = nullptr;
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  if (contribs == nullptr || K < 1) {
+    return fail(FRG_ERR_INVALID, "at least one contribution is required");
+  }
+  Context::Request r;
+  r.out = out;
+  r.contribs.assign(contribs, contribs + K);
+  r.numel = numel;
+  r.dtype = dtype;
+  r.op = op;
+  r.scaleMode = scale_mode;
+  r.scale = scale;
+  r.fromHost = fromHost;
+  r.producerStream = static_cast<hipStream_t>(producer_stream);
+  r.done = done;
+  r.user = user;
+  std::string err;
+  Work* w = nullptr;
+  const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  if (work) *work = reinterpret_cast<frg_work*>(w);
+  return FRG_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int frg_compute_layout(int64_t max_memory_allocated_in_bytes,
+                       int64_t max_padding_allocated_in_bytes, int64_t min_parallelism,
+                       int64_t num_machines, int64_t num_devices_per_machine, frg_layout* out) {
+  if (out == nullptr) return fail(FRG_ERR_INVALID, "null layout output");
+  if (num_machines < 1 || num_devices_per_machine < 1 || min_parallelism < 1) {
+    return fail(FRG_ERR_INVALID, "machines, devices per machine and parallelism must be >= 1");
+  }
+  frg::Layout l;
+  const int rc = frg::computeLayout(max_memory_allocated_in_bytes,
+                                    max_padding_allocated_in_bytes, min_parallelism,
+                                    num_machines, num_devices_per_machine, &l);
+  if (rc == 1) {
+    return fail(FRG_ERR_LAYOUT, "min_parallelism exceeds the number of padding slots");
+  }
+  if (rc == 2) return fail(FRG_ERR_LAYOUT, "padding memory exceeds the total staging memory");
+  out->slot_size_in_bytes = l.slotSizeInBytes;
+  out->slice_size_in_bytes = l.sliceSizeInBytes;
+  out->num_padding_slots = l.numPaddingSlots;
+  out->num_staging_slots = l.numStagingSlots;
+  return FRG_OK;
+}
+
+int64_t frg_num_slices(int64_t numel, int64_t slice_size_in_bytes, int64_t element_size) {
+  if (numel < 0 || element_size < 1 || slice_size_in_bytes < element_size) return -1;
+  return frg::numSlices(numel, slice_size_in_bytes, element_size);
+}
+
+int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes, int64_t element_size,
+                     int64_t idx, int64_t* offset_in_elems, int64_t* size_in_elems) {
+  if (numel < 0 || element_size < 1 || slice_size_in_bytes < element_size ||
+      offset_in_elems == nullptr || size_in_elems == nullptr) {
+    return fail(FRG_ERR_INVALID, "bad slicing arguments");
+  }
+  if (idx < 0 || idx >= frg::numSlices(numel, slice_size_in_bytes, element_size)) {
+    return fail(FRG_ERR_INVALID, "slice index out of range");
+  }
+  frg::sliceBounds(numel, slice_size_in_bytes, element_size, idx, offset_in_elems,
+                   size_in_elems);
+  return FRG_OK;
+}
+
+int frg_reduce_slice(void* out, const void* const* contribs, int K, int64_t n, int dtype,
+                     int op, int scale_mode, float scale, int carry, void* stream) {
+  frg::ReduceArgs a;
+  a.out = out;
+  a.contribs = contribs;
+  a.K = K;
+  a.n = n;
+  a.dtype = dtype;
+  a.op = op;
+  a.scale_mode = scale_mode;
+  a.scale = scale;
+  a.carry = carry != 0;
+  std::string err;
+  const int rc = frg::launchReduce(a, static_cast<hipStream_t>(stream), &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_create(int device, const frg_options* opts, frg_ctx** out) {
+  if (out == nullptr) return fail(FRG_ERR_INVALID, "null context output");
+  *out = nullptr;
+  frg_options o = {};
+  if (opts) o = *opts;
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count < 1) {
+    (void)hipGetLastError();
+    return fail(FRG_ERR_HIP, "no HIP device available");
+  }
+  if (device < 0 || device >= count) return fail(FRG_ERR_INVALID, "device index out of range");
+  Context* c = nullptr;
+  std::string err;
+  const int rc = Context::create(device, o, &c, &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  *out = reinterpret_cast<frg_ctx*>(c);
+  return FRG_OK;
+}
+
+int frg_destroy(frg_ctx* ctx) {
+  if (ctx == nullptr) return FRG_OK;
+  delete asCtx(ctx);
+  return FRG_OK;
+}
+
+int frg_get_layout(frg_ctx* ctx, frg_layout* out) {
+  if (ctx == nullptr || out == nullptr) return fail(FRG_ERR_INVALID, "null argument");
+  const frg::Layout& l = asCtx(ctx)->layout();
+  out->slot_size_in_bytes = l.slotSizeInBytes;
+  out->slice_size_in_bytes = l.sliceSizeInBytes;
+  out->num_padding_slots = l.numPaddingSlots;
+  out->num_staging_slots = l.numStagingSlots;
+  return FRG_OK;
+}
+
+int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
+                  int dtype, int op, int scale_mode, float scale, void* producer_stream,
+                  frg_done_fn done, void* user, frg_work** work) {
+  return submitCommon(ctx, out, contribs, K, numel, dtype, op, scale_mode, scale,
+                      producer_stream, done, user, work, /*fromHost=*/false);
+}
+
+int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs, int K,
+                       int64_t numel, int dtype, int op, int scale_mode, float scale,
+                       void* producer_stream, frg_done_fn done, void* user, frg_work** work) {
+  return submitCommon(ctx, out, host_contribs, K, numel, dtype, op, scale_mode, scale,
+                      producer_stream, done, user, work, /*fromHost=*/true);
+}
+
+int frg_work_wait(frg_work* work) {
+  if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
+  std::string err;
+  const int rc = Context::waitWork(asWork(work), &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_work_is_completed(frg_work* work) {
+  if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
+  return Context::workEnqueued(asWork(work)) ? FRG_OK : FRG_ERR_NOT_READY;
+}
+
+int frg_work_block_stream(frg_work* work, void* stream) {
+  if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
+  std::string err;
+  const int rc = Context::blockStream(asWork(work), static_cast<hipStream_t>(stream), &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_work_release(frg_work* work) {
+  if (work == nullptr) return FRG_OK;
+  Context::releaseWork(asWork(work));
+  return FRG_OK;
+}
+
+int frg_synchronize(frg_ctx* ctx) {
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  std::string err;
+  const int rc = asCtx(ctx)->synchronize(&err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_set_profiling(frg_ctx* ctx, int on) {
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  asCtx(ctx)->setProfiling(on != 0);
+  return FRG_OK;
+}
+
+int frg_kernel_times(frg_ctx* ctx, float* ms, int capacity, int* count) {
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  std::string err;
+  const int rc = asCtx(ctx)->kernelTimes(ms, capacity, count, &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_set_tuning(int blocks_per_cu, int xcd_remap) {
+  frg::setTuning(blocks_per_cu, xcd_remap);
+  return FRG_OK;
+}
+
+const char* frg_last_error(void) { return frg::lastError(); }
+
+const char* frg_version(void) { return "0.1"; }
+
+}  // extern "C"

@@ -1,0 +1,33 @@
+// Internal launcher of the K-way slice reduction kernels (gfx950).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+namespace frg {
+
+constexpr int kMaxContribsPerLaunch = 64;
+
+struct ReduceArgs {
+  void* out = nullptr;
+  const void* const* contribs = nullptr;  // host array of K device pointers
+  int K = 0;
+  int64_t n = 0;  // elements
+  int dtype = 0;  // FRG_F32 / FRG_BF16
+  int op = 0;     // FRG_SUM / FRG_MAX
+  int scale_mode = 0;
+  float scale = 1.0f;
+  bool carry = false;  // out is read first and takes part as term "-1"
+};
+
+// Validates the arguments, picks the kernel variant that fits K and the
+// pointers' alignment, and enqueues one launch on `stream`. Returns an FRG_*
+// status; on failure `err` says why. Never synchronises.
+int launchReduce(const ReduceArgs& args, hipStream_t stream, std::string* err);
+
+// Launch-shape knobs (process-wide); 0 keeps the default.
+void setTuning(int blocksPerCu, int xcdRemap);
+
+}  // namespace frg

@@ -1,0 +1,441 @@
+// K-way elementwise reduction of gradient slices for MI355X (gfx950, CDNA4).
+//
+// Stands in for the two places where the reference reduces a slice:
+//   * doReduction, fairring/device.cc:108-131: at::sum_out / at::amax_out over
+//     dim 0 of operand[K, n] (server-side accumulation of per-machine shards);
+//   * the arithmetic inside ncclReduceScatter, fairring/device.cc:33-70 (the
+//     local reduction over the devices of a machine).
+//
+// The work is HBM-bound (K reads + 1 write per element, K-1 adds), so the
+// kernel is a pure streaming design: every lane owns one 16-byte vector per
+// contribution, all K loads are issued before the first add so K x 16 B per
+// lane are in flight, the adds run strictly in contribution order in fp32
+// registers, the optional post-scale and the bf16 rounding are fused into the
+// store, and nothing goes through LDS. Addresses are a uniform 64-bit base
+// (SGPRs) plus a 32-bit lane offset, so a wave's load covers 1 KiB of
+// consecutive bytes. Loads and stores are non-temporal: no byte is reused.
+//
+// Bit-exactness rules: no FMA contraction, no reassociation, no packed-fp32
+// instructions (build flags), IEEE division for FRG_SCALE_DIV, fp32 denormals
+// kept.
+
+#include "ksum_kernels.h"
+
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+
+#include "../../include/fairring_hip.h"
+
+#ifndef FRG_BLOCK
+#define FRG_BLOCK 256
+#endif
+#ifndef FRG_UNROLL
+#define FRG_UNROLL 1
+#endif
+#ifndef FRG_NONTEMPORAL
+#define FRG_NONTEMPORAL 1
+#endif
+#ifndef FRG_BLOCKS_PER_CU
+#define FRG_BLOCKS_PER_CU 8
+#endif
+
+namespace frg {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = FRG_BLOCK;
+constexpr int kUnroll = FRG_UNROLL;
+constexpr int kChunk = 8;  // contributions loaded together in the runtime-K path
+
+template <typename V>
+__device__ __forceinline__ V ldStream(const V* p) {
+#if FRG_NONTEMPORAL
+  return __builtin_nontemporal_load(p);
+#else
+  return *p;
+#endif
+}
+
+template <typename V>
+__device__ __forceinline__ void stStream(V v, V* p) {
+#if FRG_NONTEMPORAL
+  __builtin_nontemporal_store(v, p);
+#else
+  *p = v;
+#endif
+}
+
+__device__ __forceinline__ float bitsToFloat(unsigned int u) {
+  return __builtin_bit_cast(float, u);
+}
+
+// fp32 -> bf16 bits, round to nearest even, NaN -> 0x7FC0.
+__device__ __forceinline__ unsigned int f32ToBf16Rne(float f) {
+  unsigned int u = __builtin_bit_cast(unsigned int, f);
+  unsigned int r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? 0x7FC0u : r;
+}
+
+// ---- storage traits: how a "vector" of elements is loaded and unpacked ------
+
+struct F32Vec {
+  using elem_t = float;
+  using vec_t = f32x4;
+  static constexpr int kLanes = 4;
+  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+    f[0] = v[0]; f[1] = v[1]; f[2] = v[2]; f[3] = v[3];
+  }
+  __device__ static vec_t pack(const float (&f)[kLanes]) {
+    vec_t v;
+    v[0] = f[0]; v[1] = f[1]; v[2] = f[2]; v[3] = f[3];
+    return v;
+  }
+};
+
+struct F32Scalar {
+  using elem_t = float;
+  using vec_t = float;
+  static constexpr int kLanes = 1;
+  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) { f[0] = v; }
+  __device__ static vec_t pack(const float (&f)[kLanes]) { return f[0]; }
+};
+
+struct Bf16Vec {  // 8 bf16 in 16 bytes
+  using elem_t = unsigned short;
+  using vec_t = u32x4;
+  static constexpr int kLanes = 8;
+  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[2 * j] = bitsToFloat(v[j] << 16);
+      f[2 * j + 1] = bitsToFloat(v[j] & 0xFFFF0000u);
+    }
+  }
+  __device__ static vec_t pack(const float (&f)[kLanes]) {
+    vec_t v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      v[j] = f32ToBf16Rne(f[2 * j]) | (f32ToBf16Rne(f[2 * j + 1]) << 16);
+    }
+    return v;
+  }
+};
+
+struct Bf16Scalar {
+  using elem_t = unsigned short;
+  using vec_t = unsigned short;
+  static constexpr int kLanes = 1;
+  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+    f[0] = bitsToFloat(static_cast<unsigned int>(v) << 16);
+  }
+  __device__ static vec_t pack(const float (&f)[kLanes]) {
+    return static_cast<unsigned short>(f32ToBf16Rne(f[0]));
+  }
+};
+
+template <int OP>
+__device__ __forceinline__ float combine(float a, float b) {
+  if (OP == FRG_SUM) {
+    return a + b;
+  } else {
+    // maximum with NaN propagation, as at::amax
+    return (a != a) ? a : ((b != b) ? b : (a > b ? a : b));
+  }
+}
+
+// Pointer table passed by value in the kernel arguments: no dependent load
+// sits between the launch and the first data load.
+template <int KT>
+struct Ptrs {
+  const void* p[KT > 0 ? KT : kMaxContribsPerLaunch];
+};
+
+// Loads N contributions [k0, k0+N) at (base + lane), then folds them into acc
+// in index order. `first` makes contribution k0 initialise acc instead.
+template <typename TR, int OP, int N, typename PT>
+__device__ __forceinline__ void foldChunk(float (&acc)[TR::kLanes], const PT& in,
+                                          int k0, int64_t elemBase,
+                                          unsigned int laneBytes, bool first) {
+  using vec_t = typename TR::vec_t;
+  using elem_t = typename TR::elem_t;
+  vec_t v[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    // uniform 64-bit base + 32-bit byte offset of the lane
+    const char* b = reinterpret_cast<const char*>(
+        static_cast<const elem_t*>(in.p[k0 + k]) + elemBase);
+    v[k] = ldStream(reinterpret_cast<const vec_t*>(b + laneBytes));
+  }
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    float f[TR::kLanes];
+    TR::unpack(v[k], f);
+    if (k == 0 && first) {
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = f[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = combine<OP>(acc[j], f[j]);
+    }
+  }
+}
+
+// One vector of the output: out = scale(carry? (+) in[0] (+) ... (+) in[K-1]).
+template <typename TR, int OP, int KT>
+__device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
+                                          const Ptrs<KT>& in, int K, bool carry,
+                                          int scaleMode, float scale,
+                                          int64_t elemBase, unsigned int lane) {
+  using vec_t = typename TR::vec_t;
+  const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
+  vec_t* o = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(out + elemBase) + laneBytes);
+  float acc[TR::kLanes];
+  bool first = true;
+  vec_t c;
+  if (carry) c = *o;  // issued before the contribution loads, consumed first
+  if (KT > 0) {
+    if (carry) {
+      TR::unpack(c, acc);
+      first = false;
+    }
+    foldChunk<TR, OP, (KT > 0 ? KT : 1)>(acc, in, 0, elemBase, laneBytes, first);
+  } else {
+    if (carry) {
+      TR::unpack(c, acc);
+      first = false;
+    }
+    int k = 0;
+    for (; k + kChunk <= K; k += kChunk) {
+      foldChunk<TR, OP, kChunk>(acc, in, k, elemBase, laneBytes, first);
+      first = false;
+    }
+    const int rem = K - k;
+    if (rem & 4) {
+      foldChunk<TR, OP, 4>(acc, in, k, elemBase, laneBytes, first);
+      first = false;
+      k += 4;
+    }
+    if (rem & 2) {
+      foldChunk<TR, OP, 2>(acc, in, k, elemBase, laneBytes, first);
+      first = false;
+      k += 2;
+    }
+    if (rem & 1) {
+      foldChunk<TR, OP, 1>(acc, in, k, elemBase, laneBytes, first);
+    }
+  }
+  if (OP == FRG_SUM) {
+    if (scaleMode == FRG_SCALE_MUL) {
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] * scale;
+    } else if (scaleMode == FRG_SCALE_DIV) {
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] / scale;
+    }
+  }
+  stStream(TR::pack(acc), o);
+}
+
+// Body kernel. The slice is [head scalars][nvec vectors][tail scalars], where
+// `head` brings every pointer to a 16-byte boundary. Tiles of kBlock*kUnroll
+// vectors are dealt to the blocks round-robin; with xcdRemap each of the 8 XCDs
+// (hardware deals consecutive blocks to consecutive XCDs) walks its own
+// contiguous eighth of the slice.
+template <typename TRV, typename TRS, int OP, int KT>
+__global__ void __launch_bounds__(kBlock)
+    ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K, int carry,
+               int scaleMode, float scale, int64_t head, int64_t nvec,
+               int64_t tail, int xcdRemap) {
+  constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
+  const int64_t ntiles = (nvec + kTile - 1) / kTile;
+  const int64_t perXcd = ntiles >> 3;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int64_t tile = xcdRemap ? ((t & 7) * perXcd + (t >> 3)) : t;
+    const int64_t v0 = tile * kTile;
+    const int64_t elemBase = head + v0 * TRV::kLanes;
+    if (v0 + kTile <= nvec) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale, elemBase,
+                               threadIdx.x + u * kBlock);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const unsigned int lane = threadIdx.x + u * kBlock;
+        if (v0 + lane < nvec) {
+          reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale,
+                                 elemBase, lane);
+        }
+      }
+    }
+  }
+  // ragged edges: at most kLanes-1 scalars on each side, done by block 0
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const int64_t e = threadIdx.x < head
+                          ? static_cast<int64_t>(threadIdx.x)
+                          : head + nvec * TRV::kLanes + (threadIdx.x - head);
+    reduceOne<TRS, OP, KT>(out, in, K, carry != 0, scaleMode, scale, e, 0u);
+  }
+}
+
+struct DeviceInfo {
+  int numCus = 0;
+};
+
+DeviceInfo& deviceInfo(int device) {
+  static std::mutex mu;
+  static DeviceInfo infos[64];
+  std::lock_guard<std::mutex> g(mu);
+  DeviceInfo& d = infos[device & 63];
+  if (d.numCus == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount,
+                              device) != hipSuccess ||
+        cus <= 0) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    d.numCus = cus;
+  }
+  return d;
+}
+
+int gBlocksPerCu = FRG_BLOCKS_PER_CU;
+int gXcdRemap = 0;
+
+template <typename TRV, typename TRS, int OP, int KT>
+hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
+                         int64_t tail, int numCus, hipStream_t stream) {
+  Ptrs<KT> tab;
+  for (int k = 0; k < a.K; ++k) tab.p[k] = a.contribs[k];
+  for (int k = a.K; k < (KT > 0 ? KT : kMaxContribsPerLaunch); ++k) {
+    tab.p[k] = a.contribs[0];
+  }
+  constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
+  const int64_t ntiles = (nvec + kTile - 1) / kTile;
+  int64_t cap = static_cast<int64_t>(numCus) * gBlocksPerCu;
+  int64_t grid = ntiles < cap ? ntiles : cap;
+  if (grid < 1) grid = 1;
+  int remap = 0;
+  if (gXcdRemap && (ntiles % 8 == 0) && (grid % 8 == 0)) remap = 1;
+  hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT>), dim3(static_cast<unsigned>(grid)),
+                     dim3(kBlock), 0, stream,
+                     static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
+                     a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail,
+                     remap);
+  return hipGetLastError();
+}
+
+template <typename TRV, typename TRS>
+hipError_t dispatchK(const ReduceArgs& a, int64_t head, int64_t nvec,
+                     int64_t tail, int numCus, hipStream_t stream) {
+  if (a.op == FRG_MAX) {
+    return launchVariant<TRV, TRS, FRG_MAX, 0>(a, head, nvec, tail, numCus, stream);
+  }
+  switch (a.K) {
+    case 2:
+      return launchVariant<TRV, TRS, FRG_SUM, 2>(a, head, nvec, tail, numCus, stream);
+    case 4:
+      return launchVariant<TRV, TRS, FRG_SUM, 4>(a, head, nvec, tail, numCus, stream);
+    case 8:
+      return launchVariant<TRV, TRS, FRG_SUM, 8>(a, head, nvec, tail, numCus, stream);
+    default:
+      return launchVariant<TRV, TRS, FRG_SUM, 0>(a, head, nvec, tail, numCus, stream);
+  }
+}
+
+}  // namespace
+
+void setTuning(int blocksPerCu, int xcdRemap) {
+  gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : FRG_BLOCKS_PER_CU;
+  gXcdRemap = xcdRemap > 0 ? 1 : 0;
+}
+
+int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
+  auto fail = [&](int code, const std::string& msg) {
+    if (err) *err = msg;
+    return code;
+  };
+  if (a.dtype != FRG_F32 && a.dtype != FRG_BF16) {
+    return fail(FRG_ERR_UNSUPPORTED, "unsupported dtype " + std::to_string(a.dtype));
+  }
+  if (a.op != FRG_SUM && a.op != FRG_MAX) {
+    return fail(FRG_ERR_UNSUPPORTED,
+                "unsupported reduce op " + std::to_string(a.op) + " (only SUM and MAX)");
+  }
+  if (a.K < 1 || a.K > kMaxContribsPerLaunch) {
+    return fail(FRG_ERR_INVALID, "K must be in [1, 64] per launch, got " + std::to_string(a.K));
+  }
+  if (a.n < 0) return fail(FRG_ERR_INVALID, "negative element count");
+  if (a.scale_mode < FRG_SCALE_NONE || a.scale_mode > FRG_SCALE_DIV) {
+    return fail(FRG_ERR_INVALID, "bad scale mode");
+  }
+  if (a.op == FRG_MAX && a.scale_mode != FRG_SCALE_NONE) {
+    return fail(FRG_ERR_INVALID, "MAX takes no post-scale");
+  }
+  if (a.contribs == nullptr) return fail(FRG_ERR_INVALID, "null contribution table");
+  if (a.n == 0) return FRG_OK;  // device.cc:120-122
+  if (a.out == nullptr) return fail(FRG_ERR_INVALID, "null output");
+
+  const int64_t elsize = a.dtype == FRG_F32 ? 4 : 2;
+  const int lanes = static_cast<int>(16 / elsize);
+  const uintptr_t o = reinterpret_cast<uintptr_t>(a.out);
+  const uintptr_t bytes = static_cast<uintptr_t>(a.n) * elsize;
+  if (o % elsize != 0) return fail(FRG_ERR_INVALID, "output not element-aligned");
+  bool congruent = true;
+  for (int k = 0; k < a.K; ++k) {
+    const uintptr_t p = reinterpret_cast<uintptr_t>(a.contribs[k]);
+    if (p == 0) return fail(FRG_ERR_INVALID, "null contribution " + std::to_string(k));
+    if (p % elsize != 0) {
+      return fail(FRG_ERR_INVALID, "contribution " + std::to_string(k) + " not element-aligned");
+    }
+    if (p != o && p < o + bytes && o < p + bytes) {
+      return fail(FRG_ERR_INVALID,
+                  "output partially overlaps contribution " + std::to_string(k));
+    }
+    if ((p & 15) != (o & 15)) congruent = false;
+  }
+
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    return fail(FRG_ERR_HIP, "hipGetDevice failed");
+  }
+  const int numCus = deviceInfo(device).numCus;
+
+  int64_t head = 0, nvec = 0, tail = 0;
+  if (congruent) {
+    head = static_cast<int64_t>(((16 - (o & 15)) & 15) / elsize);
+    if (head > a.n) head = a.n;
+    nvec = (a.n - head) / lanes;
+    tail = a.n - head - nvec * lanes;
+  }
+  hipError_t e;
+  if (nvec > 0) {
+    e = a.dtype == FRG_F32
+            ? dispatchK<F32Vec, F32Scalar>(a, head, nvec, tail, numCus, stream)
+            : dispatchK<Bf16Vec, Bf16Scalar>(a, head, nvec, tail, numCus, stream);
+  } else {
+    // Pointers disagree modulo 16 (or the slice is shorter than a vector):
+    // element-wise variant, still coalesced, one element per lane.
+    ReduceArgs s = a;
+    if (a.dtype == FRG_F32) {
+      e = a.op == FRG_MAX
+              ? launchVariant<F32Scalar, F32Scalar, FRG_MAX, 0>(s, 0, a.n, 0, numCus, stream)
+              : launchVariant<F32Scalar, F32Scalar, FRG_SUM, 0>(s, 0, a.n, 0, numCus, stream);
+    } else {
+      e = a.op == FRG_MAX
+              ? launchVariant<Bf16Scalar, Bf16Scalar, FRG_MAX, 0>(s, 0, a.n, 0, numCus, stream)
+              : launchVariant<Bf16Scalar, Bf16Scalar, FRG_SUM, 0>(s, 0, a.n, 0, numCus, stream);
+    }
+  }
+  if (e != hipSuccess) {
+    return fail(FRG_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString(e));
+  }
+  return FRG_OK;
+}
+
+}  // namespace frg

@@ -1,0 +1,77 @@
+// Integer layout and slicing rules of the staging pool (host only, no GPU).
+//
+// computeLayout follows fairring/utils.h:288-327, the helpers follow
+// fairring/utils.h:258-279, the slicing follows fairring/device.cc:315-326.
+#pragma once
+
+#include <stdint.h>
+
+#include <limits>
+
+namespace frg {
+
+// Every slot and slice holds a whole number of elements of any supported type;
+// 8 bytes (a double) is the widest (fairring/utils.h:276-279).
+constexpr int64_t kAlignment = 8;
+
+constexpr int64_t kDefaultTotalMemory = 50ll * 1024 * 1024;   // fairring/__init__.py:26
+constexpr int64_t kDefaultPaddingMemory = 1024ll * 1024;      // fairring/__init__.py:30
+constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init__.py:34
+
+inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {
+  return num == 0 ? 0 : (num - 1) / den + 1;
+}
+
+inline constexpr int64_t roundDownToNearestMultiple(int64_t val, int64_t factor) {
+  return (val / factor) * factor;
+}
+
+inline constexpr int64_t roundUpToNearestMultiple(int64_t val, int64_t factor) {
+  return ceilOfRatio(val, factor) * factor;
+}
+
+struct Layout {
+  int64_t slotSizeInBytes = 0;
+  int64_t sliceSizeInBytes = 0;
+  int64_t numPaddingSlots = 0;
+  int64_t numStagingSlots = 0;
+};
+
+// Returns 0 on success; 1 / 2 name the precondition the reference would
+// terminate on (too little padding memory for the parallelism asked for /
+// padding alone exceeding the pool).
+inline int computeLayout(int64_t maxMemoryAllocatedInBytes,
+                         int64_t maxPaddingAllocatedInBytes,
+                         int64_t minParallelism, int64_t numMachines,
+                         int64_t numDevicesPerMachine, Layout* out) {
+  const int64_t unit = numDevicesPerMachine * numMachines * kAlignment;
+  Layout l;
+  l.numPaddingSlots = maxPaddingAllocatedInBytes / unit;
+  if (minParallelism > l.numPaddingSlots) return 1;
+  l.sliceSizeInBytes = std::numeric_limits<int64_t>::max();
+  if (numDevicesPerMachine == 1) {
+    const int64_t reserved = 2 * minParallelism * unit;
+    if (reserved > maxMemoryAllocatedInBytes) return 2;
+    l.slotSizeInBytes = roundDownToNearestMultiple(
+        (maxMemoryAllocatedInBytes - reserved) / minParallelism, unit);
+    l.sliceSizeInBytes = l.slotSizeInBytes * numDevicesPerMachine;
+    l.numStagingSlots = minParallelism;
+    l.numPaddingSlots = minParallelism;
+  }
+  *out = l;
+  return 0;
+}
+
+inline int64_t numSlices(int64_t numel, int64_t sliceSizeInBytes, int64_t elsize) {
+  return ceilOfRatio(numel, sliceSizeInBytes / elsize);
+}
+
+inline void sliceBounds(int64_t numel, int64_t sliceSizeInBytes, int64_t elsize,
+                        int64_t idx, int64_t* offset, int64_t* size) {
+  const int64_t maxElems = sliceSizeInBytes / elsize;
+  *offset = idx * maxElems;
+  const int64_t left = numel - *offset;
+  *size = left < maxElems ? left : maxElems;
+}
+
+}  // namespace frg

@@ -1,0 +1,577 @@
+#include "pipeline.h"
+
+#include <cstdio>
+#include <stdexcept>
+
+#include "ksum_kernels.h"
+
+namespace frg {
+
+namespace {
+
+thread_local std::string tlsError;
+
+struct HipFailure : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+struct ContractFailure : std::runtime_error {
+  int code;
+  ContractFailure(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+
+// Throws on failure, like the reference's CUDA_CHECK (fairring/utils.h:35-45).
+#define FRG_HIP_CHECK(op)                                                        \
+  do {                                                                           \
+    hipError_t res_ = (op);                                                      \
+    if (res_ != hipSuccess) {                                                    \
+      (void)hipGetLastError();                                                   \
+      throw HipFailure(std::string("HIP error at ") + __FILE__ + ":" +           \
+                       std::to_string(__LINE__) + ": " + hipGetErrorString(res_)); \
+    }                                                                            \
+  } while (0)
+
+// Makes `device` current for the scope and restores the caller's device.
+class DeviceGuard {
+ public:
+  explicit DeviceGuard(int device) {
+    FRG_HIP_CHECK(hipGetDevice(&prev_));
+    if (prev_ != device) {
+      FRG_HIP_CHECK(hipSetDevice(device));
+      changed_ = true;
+    }
+  }
+  ~DeviceGuard() {
+    if (changed_) (void)hipSetDevice(prev_);
+  }
+
+ private:
+  int prev_ = 0;
+  bool changed_ = false;
+};
+
+int64_t elementSize(int dtype) { return dtype == FRG_F32 ? 4 : 2; }
+
+}  // namespace
+
+void setLastError(const std::string& msg) { tlsError = msg; }
+const char* lastError() { return tlsError.c_str(); }
+
+void CommandQueue::enqueue(std::function<void()> fn) {
+  std::unique_lock<std::mutex> lock(mutex_);
+  fns_.push_back(std::move(fn));
+  cv_.notify_one();
+}
+
+std::function<void()> CommandQueue::dequeue() {
+  std::unique_lock<std::mutex> lock(mutex_);
+  cv_.wait(lock, [&] { return !fns_.empty(); });
+  std::function<void()> fn = std::move(fns_.front());
+  fns_.pop_front();
+  return fn;
+}
+
+int Context::create(int device, const frg_options& o, Context** out, std::string* err) {
+  const int64_t total = o.max_memory_allocated_in_bytes > 0 ? o.max_memory_allocated_in_bytes
+                                                             : kDefaultTotalMemory;
+  const int64_t padding = o.max_padding_allocated_in_bytes > 0
+                              ? o.max_padding_allocated_in_bytes
+                              : kDefaultPaddingMemory;
+  const int64_t parallelism = o.min_parallelism > 0 ? o.min_parallelism : kDefaultParallelism;
+  const int64_t machines = o.num_machines > 0 ? o.num_machines : 1;
+
+  Layout layout;
+  if (o.slice_size_in_bytes > 0) {
+    // README regime: the pool holds TOTAL / SLICE slots of one slice each.
+    if (o.slice_size_in_bytes % kAlignment != 0) {
+      *err = "slice size must be a multiple of 8 bytes";
+      return FRG_ERR_LAYOUT;
+    }
+    layout.sliceSizeInBytes = o.slice_size_in_bytes;
+    layout.slotSizeInBytes = o.slice_size_in_bytes;
+    layout.numStagingSlots = total / o.slice_size_in_bytes;
+    layout.numPaddingSlots = layout.numStagingSlots;
+    if (layout.numStagingSlots < 1) {
+      *err = "FAIRRING_TOTAL_MEMORY holds less than one slice";
+      return FRG_ERR_LAYOUT;
+    }
+  } else {
+    const int rc = computeLayout(total, padding, parallelism, machines, 1, &layout);
+    if (rc != 0) {
+      *err = rc == 1 ? "min_parallelism exceeds the padding slots the padding memory allows"
+                     : "padding memory alone exceeds the total staging memory";
+      return FRG_ERR_LAYOUT;
+    }
+    if (layout.slotSizeInBytes < kAlignment) {
+      *err = "staging memory too small for the requested parallelism";
+      return FRG_ERR_LAYOUT;
+    }
+  }
+
+  Context* c = new Context();
+  c->device_ = device;
+  c->layout_ = layout;
+  c->numSlots_ = layout.numStagingSlots;
+  c->slotBytes_ = layout.slotSizeInBytes;
+  try {
+    DeviceGuard g(device);
+    int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams
+                                            : static_cast<int>(c->numSlots_ < 2 ? c->numSlots_ : 2);
+    if (nStreams > c->numSlots_) nStreams = static_cast<int>(c->numSlots_);
+    if (nStreams < 1) nStreams = 1;
+    // Default priority on purpose: all streams of the pipeline share one level.
+    for (int i = 0; i < nStreams; ++i) {
+      hipStream_t s;
+      FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+      c->reduceStreams_.push_back(s);
+    }
+    FRG_HIP_CHECK(hipStreamCreateWithFlags(&c->copyStream_, hipStreamNonBlocking));
+    FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->stagingPool_),
+                            static_cast<size_t>(c->numSlots_ * c->slotBytes_)));
+    for (int64_t i = 0; i < c->numSlots_; ++i) {
+      hipEvent_t a, b;
+      FRG_HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
+      FRG_HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
+      c->slotFreeEvents_.push_back(a);
+      c->slotFilledEvents_.push_back(b);
+    }
+    c->slotUsed_.assign(static_cast<size_t>(c->numSlots_), 0);
+  } catch (const std::exception& e) {
+    *err = e.what();
+    // partially built: release what exists, without a command thread to join
+    if (c->stagingPool_) (void)hipFree(c->stagingPool_);
+    delete c;
+    return FRG_ERR_HIP;
+  }
+
+  c->thread_ = std::thread([c] {
+    (void)hipSetDevice(c->device_);
+    while (true) {
+      std::function<void()> fn = c->queue_.dequeue();
+      if (!fn) return;
+      fn();
+    }
+  });
+  *out = c;
+  return FRG_OK;
+}
+
+Context::~Context() {
+  if (thread_.joinable()) {
+    queue_.enqueue(nullptr);
+    thread_.join();
+  }
+  // Everything submitted has been enqueued; let it finish before the pool goes.
+  int prev = 0;
+  (void)hipGetDevice(&prev);
+  (void)hipSetDevice(device_);
+  for (hipStream_t s : reduceStreams_) (void)hipStreamSynchronize(s);
+  if (copyStream_) (void)hipStreamSynchronize(copyStream_);
+  if (stagingPool_) (void)hipFree(stagingPool_);
+  for (hipEvent_t e : slotFreeEvents_) (void)hipEventDestroy(e);
+  for (hipEvent_t e : slotFilledEvents_) (void)hipEventDestroy(e);
+  for (hipEvent_t e : freeEvents_) (void)hipEventDestroy(e);
+  for (auto& p : profEvents_) {
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
+  }
+  // The streams are not destroyed: a consumer may still hold an event that
+  // orders its own stream after one of them (fairring/machine.cc:162-175).
+  (void)hipSetDevice(prev);
+}
+
+hipEvent_t Context::takeEvent() {
+  {
+    std::lock_guard<std::mutex> g(eventMu_);
+    if (!freeEvents_.empty()) {
+      hipEvent_t e = freeEvents_.back();
+      freeEvents_.pop_back();
+      return e;
+    }
+  }
+  hipEvent_t e;
+  FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  return e;
+}
+
+void Context::giveEvent(hipEvent_t e) {
+  std::lock_guard<std::mutex> g(eventMu_);
+  freeEvents_.push_back(e);
+}
+
+void Context::releaseWork(Work* w) {
+  if (w->refs.fetch_sub(1) == 1) {
+    if (w->doneEvent) (void)hipEventDestroy(w->doneEvent);
+    delete w;
+  }
+}
+
+bool Context::workEnqueued(Work* w) {
+  std::lock_guard<std::mutex> g(w->mu);
+  return w->enqueued;
+}
+
+int Context::waitWork(Work* w, std::string* err) {
+  {
+    std::unique_lock<std::mutex> lock(w->mu);
+    w->cv.wait(lock, [&] { return w->enqueued; });
+    if (w->status != FRG_OK) {
+      *err = w->error;
+      return w->status;
+    }
+  }
+  try {
+    DeviceGuard g(w->device);
+    FRG_HIP_CHECK(hipEventSynchronize(w->doneEvent));
+  } catch (const std::exception& e) {
+    *err = e.what();
+    return FRG_ERR_HIP;
+  }
+  return FRG_OK;
+}
+
+int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
+  {
+    std::unique_lock<std::mutex> lock(w->mu);
+    w->cv.wait(lock, [&] { return w->enqueued; });
+    if (w->status != FRG_OK) {
+      *err = w->error;
+      return w->status;
+    }
+  }
+  try {
+    DeviceGuard g(w->device);
+    FRG_HIP_CHECK(hipStreamWaitEvent(stream, w->doneEvent, 0));
+  } catch (const std::exception& e) {
+    *err = e.what();
+    return FRG_ERR_HIP;
+  }
+  return FRG_OK;
+}
+
+int Context::submit(Request req, Work** workOut, std::string* err) {
+  // Contract checks made on the caller's thread, before anything is queued.
+  if (req.dtype != FRG_F32 && req.dtype != FRG_BF16) {
+    *err = "unsupported dtype";
+    return FRG_ERR_UNSUPPORTED;
+  }
+  if (req.op != FRG_SUM && req.op != FRG_MAX) {  // fairring/machine.cc:181
+    *err = "unsupported reduce op (only SUM and MAX)";
+    return FRG_ERR_UNSUPPORTED;
+  }
+  if (req.contribs.empty()) {
+    *err = "at least one contribution is required";
+    return FRG_ERR_INVALID;
+  }
+  if (req.numel < 0) {
+    *err = "negative element count";
+    return FRG_ERR_INVALID;
+  }
+  if (req.op == FRG_MAX && req.scaleMode != FRG_SCALE_NONE) {
+    *err = "MAX takes no post-scale";
+    return FRG_ERR_INVALID;
+  }
+  if (req.scaleMode < FRG_SCALE_NONE || req.scaleMode > FRG_SCALE_DIV) {
+    *err = "bad scale mode";
+    return FRG_ERR_INVALID;
+  }
+  if (kAlignment % elementSize(req.dtype) != 0) {  // fairring/device.cc:316
+    *err = "element size must divide 8";
+    return FRG_ERR_INVALID;
+  }
+  if (req.numel > 0) {
+    if (req.out == nullptr) {
+      *err = "null output";
+      return FRG_ERR_INVALID;
+    }
+    for (const void* p : req.contribs) {
+      if (p == nullptr) {
+        *err = "null contribution";
+        return FRG_ERR_INVALID;
+      }
+    }
+  }
+
+  Work* work = new Work();
+  work->device = device_;
+  hipEvent_t initial = nullptr;
+  try {
+    DeviceGuard g(device_);
+    FRG_HIP_CHECK(hipEventCreateWithFlags(&work->doneEvent, hipEventDisableTiming));
+    // Orders the pipeline after whatever produced the inputs
+    // (fairring/device.cc:294-295).
+    initial = takeEvent();
+    FRG_HIP_CHECK(hipEventRecord(initial, req.producerStream));
+  } catch (const std::exception& e) {
+    *err = e.what();
+    if (initial) giveEvent(initial);
+    releaseWork(work);
+    return FRG_ERR_HIP;
+  }
+  if (workOut) {
+    work->refs.fetch_add(1);
+    *workOut = work;
+  }
+  queue_.enqueue([this, req = std::move(req), initial, work]() { run(req, initial, work); });
+  return FRG_OK;
+}
+
+void Context::launch(const ReduceArgs& args, hipStream_t stream) {
+  hipEvent_t t0 = nullptr, t1 = nullptr;
+  const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
+  if (prof) {
+    FRG_HIP_CHECK(hipEventCreate(&t0));
+    FRG_HIP_CHECK(hipEventCreate(&t1));
+    FRG_HIP_CHECK(hipEventRecord(t0, stream));
+  }
+  std::string err;
+  const int rc = launchReduce(args, stream, &err);
+  if (rc == FRG_ERR_HIP) throw HipFailure(err);
+  if (rc != FRG_OK) throw ContractFailure(rc, err);
+  if (prof) {
+    FRG_HIP_CHECK(hipEventRecord(t1, stream));
+    std::lock_guard<std::mutex> g(profMu_);
+    profEvents_.emplace_back(t0, t1);
+  }
+}
+
+// Device-resident contributions: one reduction launch per slice, slices
+// rotating over the reduce streams so that the tail of one launch overlaps
+// the head of the next (the slicing of fairring/device.cc:315-326).
+void Context::runResident(const Request& req, hipEvent_t initialEvent, hipStream_t* last) {
+  const int64_t elsize = elementSize(req.dtype);
+  const int64_t nSlices = numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
+  const size_t nStreams = reduceStreams_.size();
+  std::vector<char> waited(nStreams, 0);
+  std::vector<const void*> ptrs(req.contribs.size());
+  size_t lastIdx = 0;
+  for (int64_t i = 0; i < nSlices; ++i) {
+    int64_t off, len;
+    sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &off, &len);
+    const int64_t slot = (nextStagingSlot_++) % numSlots_;
+    const size_t si = static_cast<size_t>(slot) % nStreams;
+    hipStream_t s = reduceStreams_[si];
+    if (!waited[si]) {
+      // Only the first slice on a stream needs the producer's event; later
+      // ones follow it in stream order (fairring/device.cc:334-336,507-509).
+      FRG_HIP_CHECK(hipStreamWaitEvent(s, initialEvent, 0));
+      waited[si] = 1;
+    }
+    for (size_t k = 0; k < ptrs.size(); ++k) {
+      ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * elsize;
+    }
+    // More contributions than one launch takes: chain launches, carrying the
+    // partial result in `out`; the post-scale goes on the last one only.
+    const int total = static_cast<int>(ptrs.size());
+    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
+      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
+      const bool lastLaunch = k0 + kn == total;
+      ReduceArgs a;
+      a.out = static_cast<char*>(req.out) + off * elsize;
+      a.contribs = ptrs.data() + k0;
+      a.K = kn;
+      a.n = len;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = lastLaunch ? req.scaleMode : FRG_SCALE_NONE;
+      a.scale = req.scale;
+      a.carry = k0 > 0;
+      launch(a, s);
+    }
+    lastIdx = si;
+  }
+  // Join: the stream of the last slice waits for the others that took part.
+  hipStream_t ls = reduceStreams_[lastIdx];
+  if (nSlices == 0) {
+    FRG_HIP_CHECK(hipStreamWaitEvent(ls, initialEvent, 0));
+  }
+  for (size_t si = 0; si < nStreams; ++si) {
+    if (si == lastIdx || !waited[si]) continue;
+    hipEvent_t j = takeEvent();
+    FRG_HIP_CHECK(hipEventRecord(j, reduceStreams_[si]));
+    FRG_HIP_CHECK(hipStreamWaitEvent(ls, j, 0));
+    giveEvent(j);
+  }
+  *last = ls;
+}
+
+// Contributions in pinned host memory (server-side accumulation): contribution
+// 0 lands directly in `out`; each later one is copied into the next staging
+// slot on the copy stream as soon as the reduction that last read that slot
+// has finished, and folded into `out` on the reduce stream in index order
+// (slot rule of fairring/device.cc:543-545,587-589; cursor of :482). With four
+// or more slots, half the pool is folded per launch so that copies into the
+// other half overlap it.
+void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStream_t* last) {
+  const int64_t elsize = elementSize(req.dtype);
+  // A staged slice must fit a slot as well as the slice size.
+  const int64_t sliceBytes =
+      layout_.sliceSizeInBytes < slotBytes_ ? layout_.sliceSizeInBytes : slotBytes_;
+  const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
+  const int K = static_cast<int>(req.contribs.size());
+  hipStream_t s = reduceStreams_[0];
+  FRG_HIP_CHECK(hipStreamWaitEvent(s, initialEvent, 0));
+  FRG_HIP_CHECK(hipStreamWaitEvent(copyStream_, initialEvent, 0));
+  int64_t batch = numSlots_ / 2;
+  if (batch < 1) batch = 1;
+  if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
+
+  for (int64_t i = 0; i < nSlices; ++i) {
+    int64_t off, len;
+    sliceBounds(req.numel, sliceBytes, elsize, i, &off, &len);
+    const size_t bytes = static_cast<size_t>(len * elsize);
+    char* outp = static_cast<char*>(req.out) + off * elsize;
+
+    FRG_HIP_CHECK(hipMemcpyAsync(outp, static_cast<const char*>(req.contribs[0]) + off * elsize,
+                                 bytes, hipMemcpyHostToDevice, copyStream_));
+    hipEvent_t first = takeEvent();
+    FRG_HIP_CHECK(hipEventRecord(first, copyStream_));
+    FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
+    giveEvent(first);
+
+    if (K == 1 && req.scaleMode != FRG_SCALE_NONE) {
+      const void* self = outp;
+      ReduceArgs a;
+      a.out = outp;
+      a.contribs = &self;
+      a.K = 1;
+      a.n = len;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = req.scaleMode;
+      a.scale = req.scale;
+      launch(a, s);
+    }
+
+    std::vector<const void*> staged;
+    std::vector<int64_t> slots;
+    for (int k = 1; k < K;) {
+      staged.clear();
+      slots.clear();
+      for (; k < K && static_cast<int64_t>(staged.size()) < batch; ++k) {
+        const int64_t slot = (nextStagingSlot_++) % numSlots_;
+        if (slotUsed_[slot]) {
+          FRG_HIP_CHECK(hipStreamWaitEvent(copyStream_, slotFreeEvents_[slot], 0));
+        }
+        char* dst = stagingPool_ + slot * slotBytes_;
+        FRG_HIP_CHECK(hipMemcpyAsync(dst,
+                                     static_cast<const char*>(req.contribs[k]) + off * elsize,
+                                     bytes, hipMemcpyHostToDevice, copyStream_));
+        FRG_HIP_CHECK(hipEventRecord(slotFilledEvents_[slot], copyStream_));
+        staged.push_back(dst);
+        slots.push_back(slot);
+      }
+      // The copy stream is in order: the last slot's event covers the batch.
+      FRG_HIP_CHECK(hipStreamWaitEvent(s, slotFilledEvents_[slots.back()], 0));
+      ReduceArgs a;
+      a.out = outp;
+      a.contribs = staged.data();
+      a.K = static_cast<int>(staged.size());
+      a.n = len;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = k == K ? req.scaleMode : FRG_SCALE_NONE;
+      a.scale = req.scale;
+      a.carry = true;
+      launch(a, s);
+      for (int64_t slot : slots) {
+        FRG_HIP_CHECK(hipEventRecord(slotFreeEvents_[slot], s));
+        slotUsed_[slot] = 1;
+      }
+    }
+    // The next slice's first copy overwrites nothing this slice still reads
+    // (it targets another range of `out`), so no extra wait is needed here.
+  }
+  *last = s;
+}
+
+void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
+  const int64_t seq = nextSeq_++;
+  int status = FRG_OK;
+  std::string error;
+  hipStream_t lastStream = reduceStreams_[0];
+  try {
+    if (req.fromHost) {
+      runHostStaged(req, initialEvent, &lastStream);
+    } else {
+      runResident(req, initialEvent, &lastStream);
+    }
+    FRG_HIP_CHECK(hipEventRecord(work->doneEvent, lastStream));
+  } catch (const ContractFailure& e) {
+    status = e.code;
+    error = e.what();
+  } catch (const std::exception& e) {
+    status = FRG_ERR_HIP;
+    error = e.what();
+  }
+  if (status != FRG_OK) {
+    std::fprintf(stderr, "[fairring] operation #%lld failed: %s\n",
+                 static_cast<long long>(seq), error.c_str());
+  }
+  giveEvent(initialEvent);
+  {
+    std::lock_guard<std::mutex> g(work->mu);
+    work->status = status;
+    work->error = error;
+    work->lastStream = lastStream;
+    work->enqueued = true;
+  }
+  work->cv.notify_all();
+  if (req.done) req.done(req.user, status, lastStream);
+  releaseWork(work);
+}
+
+int Context::synchronize(std::string* err) {
+  // A marker through the queue: everything submitted before it is enqueued
+  // once it runs.
+  std::mutex mu;
+  std::condition_variable cv;
+  bool reached = false;
+  queue_.enqueue([&] {
+    std::lock_guard<std::mutex> g(mu);
+    reached = true;
+    cv.notify_all();
+  });
+  {
+    std::unique_lock<std::mutex> lock(mu);
+    cv.wait(lock, [&] { return reached; });
+  }
+  try {
+    DeviceGuard g(device_);
+    for (hipStream_t s : reduceStreams_) FRG_HIP_CHECK(hipStreamSynchronize(s));
+    FRG_HIP_CHECK(hipStreamSynchronize(copyStream_));
+  } catch (const std::exception& e) {
+    *err = e.what();
+    return FRG_ERR_HIP;
+  }
+  return FRG_OK;
+}
+
+void Context::setProfiling(bool on) { profiling_.store(on); }
+
+int Context::kernelTimes(float* ms, int capacity, int* count, std::string* err) {
+  const int rc = synchronize(err);
+  if (rc != FRG_OK) return rc;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> evs;
+  {
+    std::lock_guard<std::mutex> g(profMu_);
+    evs.swap(profEvents_);
+  }
+  int n = 0;
+  int status = FRG_OK;
+  for (auto& p : evs) {
+    float t = 0.f;
+    const hipError_t e = hipEventElapsedTime(&t, p.first, p.second);
+    if (e != hipSuccess && status == FRG_OK) {
+      status = FRG_ERR_HIP;
+      *err = std::string("hipEventElapsedTime: ") + hipGetErrorString(e);
+    }
+    if (n < capacity && ms) ms[n] = t;
+    ++n;
+    (void)hipEventDestroy(p.first);
+    (void)hipEventDestroy(p.second);
+  }
+  if (count) *count = n;
+  return status;
+}
+
+}  // namespace frg

@@ -1,0 +1,126 @@
+// The per-GPU slice pipeline: streams, events, the fixed staging pool and the
+// command thread (the role of DeviceFairring, fairring/device.h:22-117).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <atomic>
+#include <condition_variable>
+#include <deque>
+#include <functional>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <utility>
+#include <vector>
+
+#include "../../include/fairring_hip.h"
+#include "layout.h"
+
+namespace frg {
+
+// Unbounded FIFO of closures drained by one thread; an empty function is the
+// shutdown token (fairring/utils.h:329-351, fairring/device.cc:275-283).
+class CommandQueue {
+ public:
+  void enqueue(std::function<void()> fn);
+  std::function<void()> dequeue();
+
+ private:
+  std::mutex mutex_;
+  std::condition_variable cv_;
+  std::deque<std::function<void()>> fns_;
+};
+
+// Completion state of one submitted operation (what the reference keeps in an
+// ivalue::Future, fairring/device.cc:303-307,337-348).
+struct Work {
+  std::mutex mu;
+  std::condition_variable cv;
+  bool enqueued = false;  // the command thread is done with it
+  int status = FRG_OK;
+  std::string error;
+  hipEvent_t doneEvent = nullptr;  // recorded on lastStream after the last slice
+  hipStream_t lastStream = nullptr;
+  int device = 0;
+  std::atomic<int> refs{1};
+};
+
+class Context {
+ public:
+  static int create(int device, const frg_options& opts, Context** out, std::string* err);
+  ~Context();
+
+  const Layout& layout() const { return layout_; }
+  int device() const { return device_; }
+
+  struct Request {
+    void* out = nullptr;
+    std::vector<const void*> contribs;
+    int64_t numel = 0;
+    int dtype = FRG_F32;
+    int op = FRG_SUM;
+    int scaleMode = FRG_SCALE_NONE;
+    float scale = 1.0f;
+    bool fromHost = false;
+    hipStream_t producerStream = nullptr;
+    frg_done_fn done = nullptr;
+    void* user = nullptr;
+  };
+
+  // Validates, records the initial event on the producer stream, hands the
+  // request to the command thread and returns. `*work` may be null.
+  int submit(Request req, Work** work, std::string* err);
+
+  int synchronize(std::string* err);
+  void setProfiling(bool on);
+  int kernelTimes(float* ms, int capacity, int* count, std::string* err);
+
+  static void releaseWork(Work* w);
+  // Host blocks until the operation is enqueued and its GPU work is done.
+  static int waitWork(Work* w, std::string* err);
+  // `stream` waits for the operation; the host only waits for the enqueue.
+  static int blockStream(Work* w, hipStream_t stream, std::string* err);
+  static bool workEnqueued(Work* w);
+
+ private:
+  Context() = default;
+
+  void run(const Request& req, hipEvent_t initialEvent, Work* work);
+  void runResident(const Request& req, hipEvent_t initialEvent, hipStream_t* last);
+  void runHostStaged(const Request& req, hipEvent_t initialEvent, hipStream_t* last);
+  void launch(const struct ReduceArgs& args, hipStream_t stream);
+  hipEvent_t takeEvent();
+  void giveEvent(hipEvent_t e);
+
+  int device_ = 0;
+  Layout layout_;
+  int64_t numSlots_ = 0;
+  int64_t slotBytes_ = 0;
+
+  std::vector<hipStream_t> reduceStreams_;
+  hipStream_t copyStream_ = nullptr;
+
+  char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
+  std::vector<hipEvent_t> slotFreeEvents_;    // recorded after a slot's last consumer
+  std::vector<hipEvent_t> slotFilledEvents_;  // recorded after the copy into a slot
+  std::vector<char> slotUsed_;
+  int64_t nextStagingSlot_ = 0;  // round-robin cursor (fairring/device.cc:482)
+  int64_t nextSeq_ = 0;          // operation counter for log lines
+
+  std::mutex eventMu_;
+  std::vector<hipEvent_t> freeEvents_;
+
+  std::atomic<bool> profiling_{false};
+  std::mutex profMu_;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> profEvents_;
+
+  CommandQueue queue_;
+  std::thread thread_;
+};
+
+void setLastError(const std::string& msg);
+const char* lastError();
+
+}  // namespace frg

@@ -1,0 +1,210 @@
+"""Host-side mirror of the reference's per-GPU object on top of the C ABI.
+
+``DeviceFairring`` plays the role of fairring/device.h:22-117 for one MI355X:
+it owns a pipeline context (streams, staging pool, command thread) and turns
+``allreduce`` calls on torch tensors into asynchronous slice reductions.
+PyTorch is used here for device memory and the current stream only.
+"""
+import ctypes
+import os
+import sys
+
+from . import _capi
+from ._capi import (BF16, F32, MAX, SCALE_DIV, SCALE_MUL, SCALE_NONE, SUM,
+                    FairringError)
+
+MiB = 1024 * 1024
+
+
+def options_from_env(environ=None, stderr=None):
+    """Staging options from the environment, as fairring/__init__.py:17-34 reads
+    them, plus the FAIRRING_SLICE_SIZE of README.md:62."""
+    env = os.environ if environ is None else environ
+    err = sys.stderr if stderr is None else stderr
+    opts = {}
+    try:
+        opts["max_memory_allocated_in_bytes"] = int(env["FAIRRING_TOTAL_MEMORY"])
+    except KeyError:
+        err.write(
+            "The Fairring process group will allocate up to 50 MiB of staging memory "
+            "on each GPU. This can be tuned by setting the FAIRRING_TOTAL_MEMORY "
+            "environment variable (to an amount of bytes).\n")
+        opts["max_memory_allocated_in_bytes"] = 50 * MiB
+    try:
+        opts["max_padding_allocated_in_bytes"] = int(env["FAIRRING_PADDING_MEMORY"])
+    except KeyError:
+        opts["max_padding_allocated_in_bytes"] = MiB
+    try:
+        opts["min_parallelism"] = int(env["FAIRRING_PARALLELISM"])
+    except KeyError:
+        opts["min_parallelism"] = 16
+    if "FAIRRING_SLICE_SIZE" in env:
+        opts["slice_size_in_bytes"] = int(env["FAIRRING_SLICE_SIZE"])
+    return opts
+
+
+def compute_layout(max_memory, max_padding, min_parallelism, num_machines, devices_per_machine):
+    out = _capi.Layout()
+    _capi.check(_capi.lib().frg_compute_layout(max_memory, max_padding, min_parallelism,
+                                               num_machines, devices_per_machine,
+                                               ctypes.byref(out)))
+    return dict(slot=out.slot_size_in_bytes, slice=out.slice_size_in_bytes,
+                padding_slots=out.num_padding_slots, staging_slots=out.num_staging_slots)
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise FairringError(_capi.ERR_UNSUPPORTED, "unsupported dtype %s" % t.dtype)
+
+
+def is_non_overlapping_and_dense(t):
+    """True when the tensor's elements fill one contiguous range of memory in
+    some dimension order (what viewAsFlat requires, fairring/utils.h:353-361)."""
+    dims = sorted((st, sz) for sz, st in zip(t.shape, t.stride()) if sz != 1)
+    expect = 1
+    for st, sz in dims:
+        if sz == 0:
+            return True
+        if st != expect:
+            return False
+        expect *= sz
+    return True
+
+
+def _check_dense(t, what, device=True):
+    import torch
+    if t.layout != torch.strided:
+        raise FairringError(_capi.ERR_INVALID, "%s must be strided" % what)
+    if device and not t.is_cuda:
+        raise FairringError(_capi.ERR_INVALID, "%s must be a GPU tensor" % what)
+    if not is_non_overlapping_and_dense(t):
+        raise FairringError(_capi.ERR_INVALID, "%s must be non-overlapping and dense" % what)
+
+
+def reduce_slice(out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, carry=False,
+                 stream=None):
+    """One reduction launch (doReduction, fairring/device.cc:108-131) on torch
+    GPU tensors, on `stream` (default: torch's current stream)."""
+    import torch
+    stream = torch.cuda.current_stream(out.device) if stream is None else stream
+    tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+    for c in contribs:
+        if c.numel() != out.numel() or c.dtype != out.dtype:
+            raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+    _capi.check(_capi.lib().frg_reduce_slice(
+        out.data_ptr(), tab, len(contribs), out.numel(), _dtype_code(out), op, scale_mode,
+        scale, 1 if carry else 0, stream.cuda_stream))
+
+
+class Work:
+    """Handle on a submitted operation (WorkFairring, process_group.cc:35-75)."""
+
+    def __init__(self, handle, keepalive):
+        self._h = handle
+        self._keep = keepalive
+
+    def is_completed(self):
+        return _capi.lib().frg_work_is_completed(self._h) == _capi.OK
+
+    def wait(self, timeout=None):  # the timeout is ignored, as in the reference
+        _capi.check(_capi.lib().frg_work_wait(self._h))
+        return True
+
+    def block_stream(self, stream=None):
+        import torch
+        stream = torch.cuda.current_stream() if stream is None else stream
+        _capi.check(_capi.lib().frg_work_block_stream(self._h, stream.cuda_stream))
+
+    def result(self):
+        self.wait()
+        return [self._keep[0]]
+
+    def __del__(self):
+        h, self._h = self._h, None
+        if h is not None:
+            try:
+                _capi.lib().frg_work_release(h)
+            except Exception:
+                pass
+
+
+class DeviceFairring:
+    def __init__(self, device=0, max_memory_allocated_in_bytes=50 * MiB,
+                 max_padding_allocated_in_bytes=MiB, min_parallelism=16,
+                 slice_size_in_bytes=0, num_machines=1, num_reduce_streams=0):
+        o = _capi.Options(max_memory_allocated_in_bytes, max_padding_allocated_in_bytes,
+                          min_parallelism, slice_size_in_bytes, num_machines,
+                          num_reduce_streams, 0)
+        h = ctypes.c_void_p()
+        self._h = None
+        _capi.check(_capi.lib().frg_create(int(device), ctypes.byref(o), ctypes.byref(h)))
+        self._h = h
+        self.device = int(device)
+
+    @property
+    def layout(self):
+        out = _capi.Layout()
+        _capi.check(_capi.lib().frg_get_layout(self._h, ctypes.byref(out)))
+        return dict(slot=out.slot_size_in_bytes, slice=out.slice_size_in_bytes,
+                    padding_slots=out.num_padding_slots,
+                    staging_slots=out.num_staging_slots)
+
+    def _submit(self, fn, out, contribs, op, scale_mode, scale, stream):
+        import torch
+        _check_dense(out, "output")
+        for c in contribs:
+            if c.numel() != out.numel() or c.dtype != out.dtype:
+                raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+        stream = torch.cuda.current_stream(out.device) if stream is None else stream
+        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        wh = ctypes.c_void_p()
+        _capi.check(fn(self._h, out.data_ptr(), tab, len(contribs), out.numel(),
+                       _dtype_code(out), op, scale_mode, scale, stream.cuda_stream,
+                       _capi.DONE_FN(), None, ctypes.byref(wh)))
+        return Work(wh, (out, list(contribs)))
+
+    def allreduce(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+        """DeviceFairring::allReduce (fairring/device.cc:291-353) with the peers'
+        contributions given as GPU tensors. Returns at once."""
+        for c in contribs:
+            _check_dense(c, "contribution")
+        return self._submit(_capi.lib().frg_allreduce, out, contribs, op, scale_mode, scale,
+                            stream)
+
+    def allreduce_host(self, out, host_contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0,
+                       stream=None):
+        """Server-side accumulation of contributions held in pinned host memory."""
+        for c in host_contribs:
+            _check_dense(c, "contribution", device=False)
+            if c.is_cuda or not c.is_pinned():
+                raise FairringError(_capi.ERR_INVALID,
+                                    "host contributions must be pinned CPU tensors")
+        return self._submit(_capi.lib().frg_allreduce_host, out, host_contribs, op,
+                            scale_mode, scale, stream)
+
+    def synchronize(self):
+        _capi.check(_capi.lib().frg_synchronize(self._h))
+
+    def set_profiling(self, on):
+        _capi.check(_capi.lib().frg_set_profiling(self._h, 1 if on else 0))
+
+    def kernel_times_ms(self, capacity=1 << 16):
+        buf = (ctypes.c_float * capacity)()
+        n = ctypes.c_int()
+        _capi.check(_capi.lib().frg_kernel_times(self._h, buf, capacity, ctypes.byref(n)))
+        return list(buf[:min(n.value, capacity)])
+
+    def close(self):
+        h, self._h = self._h, None
+        if h is not None:
+            _capi.lib().frg_destroy(h)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

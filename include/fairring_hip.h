@@ -1,0 +1,191 @@
+/*
+ * fairring_hip.h - C ABI of the MI355X (gfx950) K-way gradient-slice reduction.
+ *
+ * This is the boundary a host program binds to (the c10d backend in
+ * fairring_amd/csrc/torch_ext, Python ctypes, a C benchmark). Plain pointers,
+ * sizes and opaque handles only; every function returns an int status
+ * (FRG_OK == 0) and leaves a message for frg_last_error() on failure; no C++
+ * exception or type crosses it. Device pointers are HIP device pointers on the
+ * context's device; streams and events are passed as void* (hipStream_t).
+ *
+ * Each entry point cites the part of the reference (facebookresearch/fairring,
+ * paths relative to its root) that it stands in for.
+ */
+#ifndef FAIRRING_HIP_H_
+#define FAIRRING_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FRG_API __attribute__((visibility("default")))
+
+/* ---- status codes ---------------------------------------------------- */
+enum {
+  FRG_OK = 0,
+  FRG_ERR_INVALID = 1,     /* contract violation (the reference's MY_CHECK, utils.h:29-33) */
+  FRG_ERR_HIP = 2,         /* a HIP runtime call failed (the reference's CUDA_CHECK, utils.h:35-45) */
+  FRG_ERR_LAYOUT = 3,      /* computeLayout precondition failed (utils.h:297,305) */
+  FRG_ERR_UNSUPPORTED = 4, /* dtype / op outside the supported set (machine.cc:181) */
+  FRG_ERR_NOT_READY = 5    /* non-blocking query: work not finished yet */
+};
+
+/* element types of a slice (storage type; accumulation is fp32 for both) */
+enum { FRG_F32 = 0, FRG_BF16 = 1 };
+
+/* reduction ops accepted by MachineFairring::allReduce (machine.cc:181) */
+enum { FRG_SUM = 0, FRG_MAX = 1 };
+
+/* fused post-scale applied once to the accumulated value before the store */
+enum {
+  FRG_SCALE_NONE = 0, /* out = acc                                     */
+  FRG_SCALE_MUL = 1,  /* out = acc * scale  (scale = 1/K; exact for K = 2^p) */
+  FRG_SCALE_DIV = 2   /* out = acc / scale  (scale = K; IEEE division, at::div) */
+};
+
+/* ---- layout and slicing (pure integer functions, no GPU) ---------------- */
+
+/* Layout: fairring/utils.h:281-286 */
+typedef struct frg_layout {
+  int64_t slot_size_in_bytes;
+  int64_t slice_size_in_bytes;
+  int64_t num_padding_slots;
+  int64_t num_staging_slots;
+} frg_layout;
+
+/* computeLayout: fairring/utils.h:288-327. FRG_ERR_LAYOUT where the reference
+ * terminates. */
+FRG_API int frg_compute_layout(int64_t max_memory_allocated_in_bytes,
+                               int64_t max_padding_allocated_in_bytes,
+                               int64_t min_parallelism, int64_t num_machines,
+                               int64_t num_devices_per_machine, frg_layout* out);
+
+/* numSlices = ceilOfRatio(numel, sliceBytes / elsize): fairring/device.cc:315-319 */
+FRG_API int64_t frg_num_slices(int64_t numel, int64_t slice_size_in_bytes,
+                               int64_t element_size);
+
+/* slice idx -> (offset, length) in elements: fairring/device.cc:321-326 */
+FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
+                             int64_t element_size, int64_t idx,
+                             int64_t* offset_in_elems, int64_t* size_in_elems);
+
+/* ---- one reduction launch (no pipeline) -------------------------------- */
+
+/* doReduction: fairring/device.cc:108-131 (at::sum_out / at::amax_out over
+ * dim 0 of operand[K, n]) and the arithmetic of doReduceScatter
+ * (device.cc:33-70), as one kernel launch on `stream`.
+ *
+ *   out[i] = scale( (carry ? out[i] : nothing) (+) in[0][i] (+) ... (+) in[K-1][i] )
+ *
+ * folded left to right in fp32 in exactly that order. `out` may be the same
+ * pointer as one of the contributions (in-place, as the reference reduces into
+ * the caller's own shard); partial overlaps are rejected. 1 <= K <= 64 per
+ * launch; chain launches with carry = 1 for more. n == 0 is a no-op
+ * (device.cc:120-122). Asynchronous: returns after enqueueing. */
+FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
+                             int64_t n, int dtype, int op, int scale_mode,
+                             float scale, int carry, void* stream);
+
+/* ---- the per-GPU slice pipeline ----------------------------------------- */
+
+typedef struct frg_ctx frg_ctx;   /* DeviceFairring: fairring/device.h:22-117 */
+typedef struct frg_work frg_work; /* the ivalue::Future behind WorkFairring: process_group.cc:35-75 */
+
+/* Options: OptionsFairring (fairring/process_group.h:52-77) plus the README's
+ * FAIRRING_SLICE_SIZE (README.md:62). Zero-initialise, then set fields. */
+typedef struct frg_options {
+  int64_t max_memory_allocated_in_bytes;  /* FAIRRING_TOTAL_MEMORY, default 50 MiB (__init__.py:18-26) */
+  int64_t max_padding_allocated_in_bytes; /* FAIRRING_PADDING_MEMORY, default 1 MiB (__init__.py:27-30) */
+  int64_t min_parallelism;                /* FAIRRING_PARALLELISM, default 16 (__init__.py:31-34) */
+  int64_t slice_size_in_bytes;            /* FAIRRING_SLICE_SIZE; 0 = derive with computeLayout */
+  int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
+  int32_t num_reduce_streams;             /* 0 = default (min(slots, 2)) */
+  int32_t reserved;
+} frg_options;
+
+/* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,
+ * per-slot events, command thread). No padding pool: ragged tails are handled
+ * inside the kernel. */
+FRG_API int frg_create(int device, const frg_options* opts, frg_ctx** out);
+
+/* DeviceFairring dtor: fairring/device.cc:286-289 (drain the command queue,
+ * join the thread). Streams are deliberately leaked, as machine.cc:162-175
+ * requires for streams that consumers may still hold events on. */
+FRG_API int frg_destroy(frg_ctx* ctx);
+
+/* The layout in force (slice size, number of staging slots). */
+FRG_API int frg_get_layout(frg_ctx* ctx, frg_layout* out);
+
+/* Called on the command thread once the last slice of an operation has been
+ * enqueued (status FRG_OK) or enqueueing failed; `last_stream` is the stream
+ * on which completion is ordered (device.cc:337-340 marks the future under a
+ * guard of that stream). */
+typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
+
+/* DeviceFairring::allReduce: fairring/device.cc:291-353, with the
+ * contributions that peers would have delivered passed in explicitly.
+ * Device-resident contributions: `contribs[k]` are device pointers to `numel`
+ * elements each; the tensor is cut into slices of the layout's slice size and
+ * each slice is reduced by one kernel launch, slices rotating over the
+ * reduce streams / staging slots. `producer_stream` is the stream the caller's
+ * producer work was enqueued on (the reference records its initial event on
+ * the current stream, device.cc:294-295). Returns immediately; `*work`
+ * (optional) receives a handle to wait on. */
+FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
+                          int K, int64_t numel, int dtype, int op,
+                          int scale_mode, float scale, void* producer_stream,
+                          frg_done_fn done, void* user, frg_work** work);
+
+/* Server-side accumulation with contributions in pinned host memory
+ * (device.cc:543-589: collect into a staging slot, then reduce): contribution
+ * k is copied with hipMemcpyAsync on the copy stream into staging slot
+ * (next++) % numSlots once the event recorded after that slot's previous
+ * consumer has fired, and accumulated into `out` on the reduce stream in
+ * contribution order. `contribs[k]` are host pointers (hipHostMalloc'd). */
+FRG_API int frg_allreduce_host(frg_ctx* ctx, void* out,
+                               const void* const* host_contribs, int K,
+                               int64_t numel, int dtype, int op, int scale_mode,
+                               float scale, void* producer_stream,
+                               frg_done_fn done, void* user, frg_work** work);
+
+/* WorkFairring::wait / synchronize (process_group.cc:60-68): block the host
+ * until the operation has been enqueued and its GPU work has finished. */
+FRG_API int frg_work_wait(frg_work* work);
+
+/* WorkFairring::isCompleted (process_group.cc:43-45): FRG_OK once the command
+ * thread has enqueued the whole operation, FRG_ERR_NOT_READY before. */
+FRG_API int frg_work_is_completed(frg_work* work);
+
+/* What waiting on the reference's device-aware future does for a consumer
+ * stream: make `stream` wait for the operation without blocking the host
+ * longer than the enqueue takes. */
+FRG_API int frg_work_block_stream(frg_work* work, void* stream);
+
+FRG_API int frg_work_release(frg_work* work);
+
+/* Block until every operation submitted so far has been enqueued and finished. */
+FRG_API int frg_synchronize(frg_ctx* ctx);
+
+/* ---- measurement hooks -------------------------------------------------- */
+
+/* When on, every reduction launch is bracketed by timing events on its own
+ * stream; frg_kernel_times() returns the durations (milliseconds) recorded
+ * since the last call, after synchronising. */
+FRG_API int frg_set_profiling(frg_ctx* ctx, int on);
+FRG_API int frg_kernel_times(frg_ctx* ctx, float* ms, int capacity, int* count);
+
+/* Launch-shape knobs of the reduction kernel (0 keeps the built-in default). */
+FRG_API int frg_set_tuning(int blocks_per_cu, int xcd_remap);
+
+/* Message of the last failure on the calling thread (or of the failed work). */
+FRG_API const char* frg_last_error(void);
+
+/* "major.minor" of this ABI. */
+FRG_API const char* frg_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAIRRING_HIP_H_ */

@@ -1,0 +1,346 @@
+"""GPU parity: the HIP kernels and the slice pipeline, called through the C ABI,
+against the CPU oracle and the committed golden vectors. Bit-exact for fp32 and
+for bf16 (the contract allows 1 bf16 ulp; the kernel meets 0).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+fa = pytest.importorskip("fairring_amd")
+
+DEV = "cuda:0"
+MiB = 1024 * 1024
+
+
+def _print_case(*a):
+    print("[case]", *a, flush=True)
+
+
+def to_gpu_f32(x):
+    return [torch.from_numpy(np.ascontiguousarray(r)).to(DEV) for r in x]
+
+
+def to_gpu_bf16(bits):
+    return [torch.from_numpy(np.ascontiguousarray(r).view(np.int16)).to(DEV).view(torch.bfloat16)
+            for r in bits]
+
+
+def bf16_bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+F32_CASES = ["f32_k2", "f32_k3", "f32_k8", "f32_k17", "f32_k64"]
+BF16_CASES = ["bf16_k2", "bf16_k8", "bf16_k64"]
+MODES = [("sum", fa.SCALE_NONE, None), ("mul", fa.SCALE_MUL, "inv"), ("div", fa.SCALE_DIV, "k")]
+
+
+@pytest.mark.parametrize("case", F32_CASES)
+def test_kernel_f32_golden(golden, case):
+    x = golden[case + "_in"]
+    k = x.shape[0]
+    xs = to_gpu_f32(x)
+    for name, mode, s in MODES:
+        _print_case("golden", case, name)
+        scale = 1.0 if s is None else (1.0 / k if s == "inv" else float(k))
+        out = torch.empty_like(xs[0])
+        fa.reduce_slice(out, xs, scale_mode=mode, scale=scale)
+        torch.cuda.synchronize()
+        assert_bits_equal(out.cpu().numpy(), golden[case + "_" + name], case + " " + name)
+
+
+@pytest.mark.parametrize("case", BF16_CASES)
+def test_kernel_bf16_golden(golden, case):
+    x = golden[case + "_in"]
+    k = x.shape[0]
+    xs = to_gpu_bf16(x)
+    for name, mode, s in MODES:
+        _print_case("golden", case, name)
+        scale = 1.0 if s is None else (1.0 / k if s == "inv" else float(k))
+        out = torch.empty_like(xs[0])
+        fa.reduce_slice(out, xs, scale_mode=mode, scale=scale)
+        torch.cuda.synchronize()
+        assert_bits_equal(bf16_bits(out), golden[case + "_" + name], case + " " + name)
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 33, 64])
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 1024, 4099, 262147])
+def test_kernel_f32_vs_oracle_sizes(k, n):
+    _print_case("f32 sizes", k, n)
+    rng = np.random.default_rng(1000 * k + n)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    xs = to_gpu_f32(x)
+    out = torch.empty_like(xs[0])
+    fa.reduce_slice(out, xs, scale_mode=fa.SCALE_DIV, scale=float(k))
+    torch.cuda.synchronize()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k)))
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 8, 13, 64])
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 1023, 131075])
+def test_kernel_bf16_vs_oracle_sizes(k, n):
+    _print_case("bf16 sizes", k, n)
+    rng = np.random.default_rng(2000 * k + n)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    bits = oracle.np_f32_to_bf16_rne(x)
+    xs = to_gpu_bf16(bits)
+    out = torch.empty_like(xs[0])
+    fa.reduce_slice(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+    torch.cuda.synchronize()
+    assert_bits_equal(bf16_bits(out), oracle.sum_bf16(list(bits), oracle.SCALE_MUL, 1.0 / k))
+
+
+@pytest.mark.parametrize("head", [0, 1, 2, 3])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_kernel_unaligned_congruent(head, dtype):
+    # every pointer shifted by the same number of elements off a 16-byte boundary
+    _print_case("unaligned congruent", head, dtype)
+    k, n = 8, 10007
+    rng = np.random.default_rng(77 + head)
+    x = (rng.standard_normal((k, n + head)) * 0.01).astype(np.float32)
+    if dtype == "f32":
+        big = to_gpu_f32(x)
+        outb = torch.zeros(n + head, dtype=torch.float32, device=DEV)
+        fa.reduce_slice(outb[head:], [b[head:] for b in big])
+        torch.cuda.synchronize()
+        assert_bits_equal(outb[head:].cpu().numpy(), oracle.sum_f32(list(x[:, head:])))
+        assert (outb[:head] == 0).all()
+    else:
+        bits = oracle.np_f32_to_bf16_rne(x)
+        big = to_gpu_bf16(bits)
+        outb = torch.zeros(n + head, dtype=torch.bfloat16, device=DEV)
+        fa.reduce_slice(outb[head:], [b[head:] for b in big])
+        torch.cuda.synchronize()
+        assert_bits_equal(bf16_bits(outb[head:]), oracle.sum_bf16(list(bits[:, head:])))
+        assert (outb[:head] == 0).all()
+
+
+def test_kernel_mismatched_alignment_falls_back():
+    _print_case("mismatched alignment")
+    k, n = 5, 5003
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((k, n + 4)) * 0.01).astype(np.float32)
+    big = to_gpu_f32(x)
+    views = [b[(i % 4):(i % 4) + n] for i, b in enumerate(big)]
+    out = torch.empty(n, dtype=torch.float32, device=DEV)
+    fa.reduce_slice(out, views)
+    torch.cuda.synchronize()
+    want = oracle.sum_f32([x[i, (i % 4):(i % 4) + n] for i in range(k)])
+    assert_bits_equal(out.cpu().numpy(), want)
+
+
+def test_kernel_in_place_and_carry():
+    _print_case("in place / carry")
+    k, n = 8, 70001
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    xs = to_gpu_f32(x)
+    want = oracle.sum_f32(list(x), oracle.SCALE_MUL, 0.125)
+    # in place into contribution 3's buffer (the reference reduces into its own shard)
+    fa.reduce_slice(xs[3], xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+    torch.cuda.synchronize()
+    assert_bits_equal(xs[3].cpu().numpy(), want)
+    # chained launches with carry reproduce the single-launch order
+    xs = to_gpu_f32(x)
+    out = torch.empty_like(xs[0])
+    fa.reduce_slice(out, xs[:3])
+    fa.reduce_slice(out, xs[3:5], carry=True)
+    fa.reduce_slice(out, xs[5:], carry=True, scale_mode=fa.SCALE_MUL, scale=0.125)
+    torch.cuda.synchronize()
+    assert_bits_equal(out.cpu().numpy(), want)
+
+
+def test_kernel_max():
+    _print_case("max")
+    k, n = 6, 40003
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((k, n)).astype(np.float32)
+    x[2, 5] = np.nan
+    xs = to_gpu_f32(x)
+    out = torch.empty_like(xs[0])
+    fa.reduce_slice(out, xs, op=fa.MAX)
+    torch.cuda.synchronize()
+    assert_bits_equal(out.cpu().numpy(), oracle.max_f32(list(x)))
+    bits = oracle.np_f32_to_bf16_rne(x)
+    xb = to_gpu_bf16(bits)
+    outb = torch.empty_like(xb[0])
+    fa.reduce_slice(outb, xb, op=fa.MAX)
+    torch.cuda.synchronize()
+    assert_bits_equal(bf16_bits(outb), oracle.max_bf16(list(bits)))
+
+
+@pytest.mark.parametrize("k", [2, 8, 64])
+def test_reference_known_answers(k):
+    # benchmark/benchmark.cc:130-186: all ones -> world size; arange -> arange * world
+    _print_case("KAT", k)
+    n = 6_553_600 if k <= 8 else 262_144
+    ones = torch.ones(n, device=DEV)
+    out = torch.empty_like(ones)
+    fa.reduce_slice(out, [ones] * k)
+    torch.cuda.synchronize()
+    assert bool((out == float(k)).all())
+    m = min(n, (1 << 24) // k)
+    ar = torch.arange(m, dtype=torch.float32, device=DEV)
+    out = torch.empty_like(ar)
+    fa.reduce_slice(out, [ar] * k)
+    torch.cuda.synchronize()
+    assert bool((out == ar * k).all())
+
+
+def test_error_paths():
+    _print_case("errors")
+    a = torch.zeros(1000, device=DEV)
+    with pytest.raises(fa.FairringError):  # partial overlap of output and input
+        fa.reduce_slice(a[0:600], [a[100:700], a[0:600]])
+    with pytest.raises(fa.FairringError):  # unsupported dtype
+        fa.reduce_slice(a.double(), [a.double()])
+    with pytest.raises(fa.FairringError):  # K beyond one launch
+        fa.reduce_slice(a, [a] * 65)
+    with pytest.raises(fa.FairringError):  # MAX with a scale
+        fa.reduce_slice(a, [a, a], op=fa.MAX, scale_mode=fa.SCALE_MUL, scale=0.5)
+    empty = torch.zeros(0, device=DEV)
+    fa.reduce_slice(empty, [empty, empty])  # empty is a no-op, not an error
+    torch.cuda.synchronize()
+
+
+# ---- pipeline -----------------------------------------------------------------------
+
+@pytest.mark.parametrize("slice_bytes,total,streams", [
+    (4096, 8192, 0), (40000, 400000, 3), (25 * MiB, 50 * MiB, 0), (0, 50 * MiB, 0)])
+def test_pipeline_resident_independent_of_slicing(slice_bytes, total, streams):
+    _print_case("pipeline resident", slice_bytes, total, streams)
+    k, n = 8, 300_007
+    rng = np.random.default_rng(31)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    xs = to_gpu_f32(x)
+    out = torch.empty_like(xs[0])
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=total,
+                            slice_size_in_bytes=slice_bytes, num_reduce_streams=streams)
+    w = dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+    assert w.wait() is True and w.is_completed()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_MUL, 0.125))
+    # stream-ordered consumption without a host wait
+    out2 = torch.empty_like(xs[0])
+    w2 = dev.allreduce(out2, xs)
+    w2.block_stream()
+    doubled = out2 * 2
+    torch.cuda.synchronize()
+    want = oracle.sum_f32(list(x))
+    assert_bits_equal(doubled.cpu().numpy(), want * np.float32(2))
+    dev.close()
+
+
+def test_pipeline_more_than_64_contributions():
+    _print_case("pipeline K=100")
+    k, n = 100, 50_003
+    rng = np.random.default_rng(32)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    xs = to_gpu_f32(x)
+    out = torch.empty_like(xs[0])
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=64 * 1024, max_memory_allocated_in_bytes=MiB)
+    dev.allreduce(out, xs, scale_mode=fa.SCALE_DIV, scale=float(k)).wait()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k)))
+    dev.close()
+
+
+def test_pipeline_waits_for_producer_stream():
+    _print_case("pipeline producer stream")
+    n = 4_000_000
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=MiB, max_memory_allocated_in_bytes=4 * MiB)
+    side = torch.cuda.Stream()
+    a = torch.zeros(n, device=DEV)
+    b = torch.zeros(n, device=DEV)
+    out = torch.empty(n, device=DEV)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(20):  # a long tail of producer work on a side stream
+            a.add_(1.0)
+            b.add_(2.0)
+        w = dev.allreduce(out, [a, b])
+    w.wait()
+    assert bool((out == 60.0).all())
+    dev.close()
+
+
+@pytest.mark.parametrize("k,slots", [(1, 2), (2, 2), (5, 1), (9, 2), (9, 3), (12, 8), (64, 2)])
+def test_pipeline_host_staged(k, slots):
+    _print_case("pipeline host staged", k, slots)
+    n = 100_003
+    slot = 160_000  # bytes: the tensor needs 3 staged slices per contribution
+    rng = np.random.default_rng(40 + k)
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    hs = [torch.from_numpy(np.ascontiguousarray(r)).pin_memory() for r in x]
+    out = torch.empty(n, dtype=torch.float32, device=DEV)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=slot, max_memory_allocated_in_bytes=slot * slots)
+    dev.allreduce_host(out, hs, scale_mode=fa.SCALE_DIV, scale=float(k)).wait()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_DIV, float(k)))
+    # second operation reuses the slots: the slot-free events must hold
+    dev.allreduce_host(out, hs[::-1]).wait()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x[::-1])))
+    dev.close()
+
+
+def test_pipeline_host_staged_bf16_default_layout():
+    _print_case("pipeline host staged bf16")
+    k, n = 8, 2_000_003
+    rng = np.random.default_rng(50)
+    bits = oracle.np_f32_to_bf16_rne((rng.standard_normal((k, n)) * 0.01).astype(np.float32))
+    hs = [torch.from_numpy(np.ascontiguousarray(r).view(np.int16)).view(torch.bfloat16).pin_memory()
+          for r in bits]
+    out = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    dev = fa.DeviceFairring(0)  # 50 MiB, parallelism 16 -> 16 slots of 3,276,784 B
+    assert dev.layout == dict(slot=3276784, slice=3276784, padding_slots=16, staging_slots=16)
+    dev.allreduce_host(out, hs, scale_mode=fa.SCALE_MUL, scale=0.125).wait()
+    assert_bits_equal(bf16_bits(out), oracle.sum_bf16(list(bits), oracle.SCALE_MUL, 0.125))
+    dev.close()
+
+
+def test_pipeline_many_small_operations_in_order():
+    _print_case("pipeline many ops")
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=64 * 1024, max_memory_allocated_in_bytes=256 * 1024)
+    rng = np.random.default_rng(60)
+    works, wants, outs = [], [], []
+    for i in range(40):
+        n = int(rng.integers(1, 60000))
+        k = int(rng.integers(1, 10))
+        x = (rng.standard_normal((k, n))).astype(np.float32)
+        xs = to_gpu_f32(x)
+        out = torch.empty(n, device=DEV)
+        works.append(dev.allreduce(out, xs))
+        outs.append(out)
+        wants.append(oracle.sum_f32(list(x)))
+    for w, o, want in zip(works, outs, wants):
+        w.wait()
+        assert_bits_equal(o.cpu().numpy(), want)
+    dev.synchronize()
+    dev.close()
+
+
+def test_pipeline_empty_tensor_and_layout_errors():
+    _print_case("pipeline empty / layout errors")
+    dev = fa.DeviceFairring(0)
+    e = torch.zeros(0, device=DEV)
+    assert dev.allreduce(e, [e, e]).wait() is True
+    dev.close()
+    with pytest.raises(fa.FairringError):
+        fa.DeviceFairring(0, max_padding_allocated_in_bytes=64)   # 8 padding slots < 16
+    with pytest.raises(fa.FairringError):
+        fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=MiB)
+
+
+def test_full_slice_parity_k8_25mib():
+    # one real 25 MiB slice, K = 8, fused /8: the headline shape
+    _print_case("full slice K=8 25MiB")
+    k, n = 8, 6_553_600
+    g = torch.Generator(device=DEV)
+    g.manual_seed(1234)
+    xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    out = torch.empty(n, device=DEV)
+    fa.reduce_slice(out, xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+    torch.cuda.synchronize()
+    host = [t.cpu().numpy() for t in xs]
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(host, oracle.SCALE_MUL, 0.125, threads=8))
