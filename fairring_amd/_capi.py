@@ -56,11 +56,16 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("FAIRRING_HIP_LIBRARY", LIB_PATH)
+    if not os.path.exists(path):
         raise ImportError(
             "%s is missing: build it with `python -m fairring_amd.build` "
-            "(there is no fallback implementation)" % LIB_PATH)
-    L = ctypes.CDLL(LIB_PATH)
+            "(there is no fallback implementation)" % path)
+    # PyTorch ships its own copy of the HIP runtime. Load it first so that this
+    # library binds to the runtime that owns torch's tensors and streams; two
+    # runtimes in one process do not see each other's devices.
+    import torch  # noqa: F401
+    L = ctypes.CDLL(path)
     i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
     pvp = ctypes.POINTER(ctypes.c_void_p)
     L.frg_compute_layout.argtypes = [i64, i64, i64, i64, i64, ctypes.POINTER(Layout)]

@@ -20,6 +20,10 @@ struct ReduceArgs {
   int scale_mode = 0;
   float scale = 1.0f;
   bool carry = false;  // out is read first and takes part as term "-1"
+  // Optional timing events (created with timing enabled) that receive the
+  // begin and end timestamps of this launch.
+  hipEvent_t startEvent = nullptr;
+  hipEvent_t stopEvent = nullptr;
 };
 
 // Validates the arguments, picks the kernel variant that fits K and the

@@ -316,22 +316,25 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
 }
 
 void Context::launch(const ReduceArgs& args, hipStream_t stream) {
-  hipEvent_t t0 = nullptr, t1 = nullptr;
+  ReduceArgs a = args;
   const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
   if (prof) {
-    FRG_HIP_CHECK(hipEventCreate(&t0));
-    FRG_HIP_CHECK(hipEventCreate(&t1));
-    FRG_HIP_CHECK(hipEventRecord(t0, stream));
+    FRG_HIP_CHECK(hipEventCreate(&a.startEvent));
+    FRG_HIP_CHECK(hipEventCreate(&a.stopEvent));
   }
   std::string err;
-  const int rc = launchReduce(args, stream, &err);
+  const int rc = launchReduce(a, stream, &err);
+  if (prof) {
+    if (rc == FRG_OK) {
+      std::lock_guard<std::mutex> g(profMu_);
+      profEvents_.emplace_back(a.startEvent, a.stopEvent);
+    } else {
+      (void)hipEventDestroy(a.startEvent);
+      (void)hipEventDestroy(a.stopEvent);
+    }
+  }
   if (rc == FRG_ERR_HIP) throw HipFailure(err);
   if (rc != FRG_OK) throw ContractFailure(rc, err);
-  if (prof) {
-    FRG_HIP_CHECK(hipEventRecord(t1, stream));
-    std::lock_guard<std::mutex> g(profMu_);
-    profEvents_.emplace_back(t0, t1);
-  }
 }
 
 // Device-resident contributions: one reduction launch per slice, slices
