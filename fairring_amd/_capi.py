@@ -17,7 +17,7 @@ SCALE_NONE, SCALE_MUL, SCALE_DIV = 0, 1, 2
 # every symbol include/fairring_hip.h declares
 EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_reduce_slice",
-    "frg_create", "frg_destroy", "frg_get_layout", "frg_allreduce", "frg_allreduce_host",
+    "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_set_profiling", "frg_kernel_times", "frg_set_tuning",
     "frg_last_error", "frg_version",
@@ -76,8 +76,10 @@ def lib():
     L.frg_create.argtypes = [i32, ctypes.POINTER(Options), pvp]
     L.frg_destroy.argtypes = [vp]
     L.frg_get_layout.argtypes = [vp, ctypes.POINTER(Layout)]
-    for fn in (L.frg_allreduce, L.frg_allreduce_host):
-        fn.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    L.frg_get_streams.argtypes = [vp, pvp, i32, ctypes.POINTER(i32)]
+    L.frg_allreduce.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    L.frg_allreduce_host.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp,
+                                     DONE_FN, vp, pvp]
     for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize):
         fn.argtypes = [vp]
     L.frg_work_block_stream.argtypes = [vp, vp]

@@ -22,15 +22,16 @@ Work* asWork(frg_work* w) { return reinterpret_cast<Work*>(w); }
 
 int submitCommon(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
                  int dtype, int op, int scale_mode, float scale, void* producer_stream,
-                 frg_done_fn done, void* user, frg_work** work, bool fromHost) {
+                 frg_done_fn done, void* user, frg_work** work, bool fromHost, bool carry) {
   if (work) *work = nullptr;
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  if (contribs == nullptr || K < 1) {
+  if (K < 0 || (K > 0 && contribs == nullptr) || (K == 0 && !carry)) {
     return fail(FRG_ERR_INVALID, "at least one contribution is required");
   }
   Context::Request r;
   r.out = out;
-  r.contribs.assign(contribs, contribs + K);
+  if (K > 0) r.contribs.assign(contribs, contribs + K);
+  r.carry = carry;
   r.numel = numel;
   r.dtype = dtype;
   r.op = op;
@@ -146,18 +147,26 @@ int frg_get_layout(frg_ctx* ctx, frg_layout* out) {
   return FRG_OK;
 }
 
+int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count) {
+  if (ctx == nullptr || count == nullptr) return fail(FRG_ERR_INVALID, "null argument");
+  const std::vector<hipStream_t> v = asCtx(ctx)->streams();
+  *count = static_cast<int>(v.size());
+  for (int i = 0; i < *count && i < capacity && streams != nullptr; ++i) streams[i] = v[i];
+  return FRG_OK;
+}
+
 int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
                   int dtype, int op, int scale_mode, float scale, void* producer_stream,
                   frg_done_fn done, void* user, frg_work** work) {
   return submitCommon(ctx, out, contribs, K, numel, dtype, op, scale_mode, scale,
-                      producer_stream, done, user, work, /*fromHost=*/false);
+                      producer_stream, done, user, work, /*fromHost=*/false, /*carry=*/false);
 }
 
 int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs, int K,
-                       int64_t numel, int dtype, int op, int scale_mode, float scale,
+                       int64_t numel, int dtype, int op, int scale_mode, float scale, int carry,
                        void* producer_stream, frg_done_fn done, void* user, frg_work** work) {
   return submitCommon(ctx, out, host_contribs, K, numel, dtype, op, scale_mode, scale,
-                      producer_stream, done, user, work, /*fromHost=*/true);
+                      producer_stream, done, user, work, /*fromHost=*/true, carry != 0);
 }
 
 int frg_work_wait(frg_work* work) {

@@ -258,7 +258,7 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     *err = "unsupported reduce op (only SUM and MAX)";
     return FRG_ERR_UNSUPPORTED;
   }
-  if (req.contribs.empty()) {
+  if (req.contribs.empty() && !(req.fromHost && req.carry)) {
     *err = "at least one contribution is required";
     return FRG_ERR_INVALID;
   }
@@ -365,6 +365,13 @@ void Context::runResident(const Request& req, hipEvent_t initialEvent, hipStream
     // More contributions than one launch takes: chain launches, carrying the
     // partial result in `out`; the post-scale goes on the last one only.
     const int total = static_cast<int>(ptrs.size());
+    if (total == 1 && ptrs[0] == static_cast<char*>(req.out) + off * elsize &&
+        req.scaleMode == FRG_SCALE_NONE) {
+      // A lone contribution reduced in place is the identity (what the
+      // reference does for one machine and one device: device.cc:523,569).
+      lastIdx = si;
+      continue;
+    }
     for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
       const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
       const bool lastLaunch = k0 + kn == total;
@@ -424,14 +431,21 @@ void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStre
     const size_t bytes = static_cast<size_t>(len * elsize);
     char* outp = static_cast<char*>(req.out) + off * elsize;
 
-    FRG_HIP_CHECK(hipMemcpyAsync(outp, static_cast<const char*>(req.contribs[0]) + off * elsize,
-                                 bytes, hipMemcpyHostToDevice, copyStream_));
-    hipEvent_t first = takeEvent();
-    FRG_HIP_CHECK(hipEventRecord(first, copyStream_));
-    FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
-    giveEvent(first);
+    int firstStaged = 0;
+    if (!req.carry) {
+      // contribution 0 needs no staging: it lands in `out` directly
+      FRG_HIP_CHECK(hipMemcpyAsync(outp,
+                                   static_cast<const char*>(req.contribs[0]) + off * elsize,
+                                   bytes, hipMemcpyHostToDevice, copyStream_));
+      hipEvent_t first = takeEvent();
+      FRG_HIP_CHECK(hipEventRecord(first, copyStream_));
+      FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
+      giveEvent(first);
+      firstStaged = 1;
+    }
 
-    if (K == 1 && req.scaleMode != FRG_SCALE_NONE) {
+    if (K == firstStaged && req.scaleMode != FRG_SCALE_NONE) {
+      // nothing left to fold, but the post-scale is still owed
       const void* self = outp;
       ReduceArgs a;
       a.out = outp;
@@ -447,7 +461,7 @@ void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStre
 
     std::vector<const void*> staged;
     std::vector<int64_t> slots;
-    for (int k = 1; k < K;) {
+    for (int k = firstStaged; k < K;) {
       staged.clear();
       slots.clear();
       for (; k < K && static_cast<int64_t>(staged.size()) < batch; ++k) {

@@ -54,6 +54,11 @@ class Context {
 
   const Layout& layout() const { return layout_; }
   int device() const { return device_; }
+  std::vector<hipStream_t> streams() const {
+    std::vector<hipStream_t> v = reduceStreams_;
+    v.push_back(copyStream_);
+    return v;
+  }
 
   struct Request {
     void* out = nullptr;
@@ -64,6 +69,7 @@ class Context {
     int scaleMode = FRG_SCALE_NONE;
     float scale = 1.0f;
     bool fromHost = false;
+    bool carry = false;  // host-staged only: `out` already holds the first term
     hipStream_t producerStream = nullptr;
     frg_done_fn done = nullptr;
     void* user = nullptr;

@@ -1,0 +1,284 @@
+#include "process_group.h"
+
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/core/StreamGuard.h>
+
+#include <cstdio>
+#include <exception>
+
+namespace fairring {
+
+namespace {
+
+// Contract violations end the process, as the reference's MY_CHECK does
+// (fairring/utils.h:29-33); the message goes to stderr first.
+#define FRG_CHECK(cond)                                                        \
+  if (!(cond)) {                                                               \
+    std::fprintf(stderr, "[fairring] Condition %s is false (%s:%d)\n", #cond,  \
+                 __FILE__, __LINE__);                                          \
+    std::terminate();                                                          \
+  }
+
+// Flat 1-D view over the same storage, valid for any dense permutation
+// (fairring/utils.h:353-361).
+at::Tensor viewAsFlat(const at::Tensor& t) {
+  FRG_CHECK(t.layout() == at::kStrided);
+  FRG_CHECK(t.is_non_overlapping_and_dense());
+  return at::as_strided(t, {t.numel()}, {1}, t.storage_offset());
+}
+
+int dtypeCode(const at::Tensor& t) {
+  switch (t.scalar_type()) {
+    case at::kFloat:
+      return FRG_F32;
+    case at::kBFloat16:
+      return FRG_BF16;
+    default:
+      return -1;
+  }
+}
+
+// What travels through the C ABI's completion callback.
+struct Pending {
+  c10::intrusive_ptr<c10::ivalue::Future> future;
+  at::Tensor tensor;               // the caller's tensor: result and keep-alive
+  std::vector<at::Tensor> peers;   // keep-alive
+  c10::DeviceIndex device;
+};
+
+// Runs on the pipeline's command thread once the last slice is enqueued:
+// completes the future under a guard of the last stream, so that consumers
+// are ordered after it on the GPU without a host wait
+// (fairring/device.cc:337-348).
+void onDone(void* user, int status, void* lastStream) {
+  std::unique_ptr<Pending> p(static_cast<Pending*>(user));
+  c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
+      static_cast<hipStream_t>(lastStream), p->device);
+  c10::StreamGuard g(s);
+  if (status == FRG_OK) {
+    p->future->markCompleted(std::vector<at::Tensor>{std::move(p->tensor)});
+  } else {
+    p->future->setError(std::make_exception_ptr(
+        std::runtime_error("fairring: allreduce failed with status " + std::to_string(status))));
+  }
+}
+
+}  // namespace
+
+// ---- WorkFairring ---------------------------------------------------------
+
+ProcessGroupFairring::WorkFairring::WorkFairring(
+    c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future)
+    : c10d::Work(/*rank=*/-1, opType), future_(std::move(future)) {}
+
+ProcessGroupFairring::WorkFairring::~WorkFairring() = default;
+
+bool ProcessGroupFairring::WorkFairring::isCompleted() { return future_->completed(); }
+
+bool ProcessGroupFairring::WorkFairring::isSuccess() const { return future_->hasValue(); }
+
+std::exception_ptr ProcessGroupFairring::WorkFairring::exception() const {
+  return future_->exception_ptr();
+}
+
+std::vector<at::Tensor> ProcessGroupFairring::WorkFairring::result() {
+  future_->wait();
+  return future_->value().toTensorVector();
+}
+
+void ProcessGroupFairring::WorkFairring::synchronize() { future_->wait(); }
+
+// The timeout is ignored, as in the reference (process_group.cc:64-68).
+bool ProcessGroupFairring::WorkFairring::wait(std::chrono::milliseconds /*timeout*/) {
+  future_->wait();
+  return true;
+}
+
+void ProcessGroupFairring::WorkFairring::abort() {}
+
+c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupFairring::WorkFairring::getFuture() {
+  return future_;
+}
+
+// ---- OptionsFairring -------------------------------------------------------
+
+ProcessGroupFairring::OptionsFairring::OptionsFairring(
+    int64_t maxMemory, int64_t maxPadding, int64_t minPar, bool highPriority,
+    std::chrono::milliseconds timeout, int64_t sliceSize)
+    : c10d::Backend::Options(kPgName, timeout),
+      maxMemoryAllocatedInBytes(maxMemory),
+      maxPaddingAllocatedInBytes(maxPadding),
+      minParallelism(minPar),
+      isHighPriorityStream(highPriority),
+      sliceSizeInBytes(sliceSize) {}
+
+ProcessGroupFairring::OptionsFairring::~OptionsFairring() = default;
+
+c10::intrusive_ptr<ProcessGroupFairring::OptionsFairring>
+ProcessGroupFairring::OptionsFairring::create(int64_t maxMemory, int64_t maxPadding,
+                                              int64_t minPar, bool highPriority,
+                                              std::chrono::milliseconds timeout,
+                                              int64_t sliceSize) {
+  return c10::make_intrusive<OptionsFairring>(maxMemory, maxPadding, minPar, highPriority,
+                                              timeout, sliceSize);
+}
+
+// ---- ProcessGroupFairring --------------------------------------------------
+
+ProcessGroupFairring::ProcessGroupFairring(const c10::intrusive_ptr<c10d::Store>& store,
+                                           int rank, int size,
+                                           c10::intrusive_ptr<OptionsFairring> options)
+    : c10d::Backend(rank, size), store_(store), options_(std::move(options)) {
+  TORCH_CHECK(0 <= rank && rank < size, "fairring: rank ", rank, " outside group of ", size);
+}
+
+ProcessGroupFairring::~ProcessGroupFairring() {
+  for (auto& kv : contexts_) frg_destroy(kv.second);
+}
+
+const std::string ProcessGroupFairring::getBackendName() const { return kPgName; }
+
+frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
+  auto it = contexts_.find(device);
+  if (it != contexts_.end()) return it->second;
+  frg_options o = {};
+  o.max_memory_allocated_in_bytes = options_->maxMemoryAllocatedInBytes;
+  o.max_padding_allocated_in_bytes = options_->maxPaddingAllocatedInBytes;
+  o.min_parallelism = options_->minParallelism;
+  o.slice_size_in_bytes = options_->sliceSizeInBytes;
+  o.num_machines = getSize();  // every simulated peer counts as a machine with one device
+  frg_ctx* ctx = nullptr;
+  const int rc = frg_create(device, &o, &ctx);
+  if (rc == FRG_ERR_LAYOUT) {
+    // the reference terminates inside computeLayout (fairring/utils.h:297,305)
+    std::fprintf(stderr, "[fairring] %s\n", frg_last_error());
+    std::terminate();
+  }
+  TORCH_CHECK(rc == FRG_OK, "fairring: ", frg_last_error());
+  contexts_.emplace(device, ctx);
+  return ctx;
+}
+
+void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor> peers) {
+  std::lock_guard<std::mutex> g(mutex_);
+  peers_ = std::move(peers);
+}
+
+void ProcessGroupFairring::setFusedDivide(bool on) {
+  std::lock_guard<std::mutex> g(mutex_);
+  fusedDivide_ = on;
+}
+
+std::vector<int64_t> ProcessGroupFairring::layout() {
+  std::lock_guard<std::mutex> g(mutex_);
+  TORCH_CHECK(!contexts_.empty(), "fairring: no device initialised yet");
+  frg_layout l;
+  TORCH_CHECK(frg_get_layout(contexts_.begin()->second, &l) == FRG_OK, frg_last_error());
+  return {l.slot_size_in_bytes, l.slice_size_in_bytes, l.num_padding_slots,
+          l.num_staging_slots};
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduce(
+    std::vector<at::Tensor>& data, const c10d::AllreduceOptions& opts) {
+  // One tensor per local device (fairring/machine.cc:183); one device here.
+  FRG_CHECK(data.size() == 1);
+  at::Tensor& t = data[0];
+  FRG_CHECK(t.layout() == at::kStrided);
+  FRG_CHECK(t.is_cuda());
+  FRG_CHECK(t.is_non_overlapping_and_dense());
+  t = viewAsFlat(t);
+
+  // fairring/machine.cc:181: SUM and MAX only
+  const c10d::ReduceOp::RedOpType op = opts.reduceOp.op_;
+  FRG_CHECK(op == c10d::ReduceOp::SUM || op == c10d::ReduceOp::MAX);
+  // fairring/device.cc:316
+  FRG_CHECK(8 % t.element_size() == 0);
+  const int dtype = dtypeCode(t);
+  TORCH_CHECK(dtype >= 0, "fairring: unsupported dtype ", t.scalar_type(),
+              " (float32 and bfloat16 are implemented)");
+
+  std::lock_guard<std::mutex> g(mutex_);
+  const c10::DeviceIndex device = t.device().index();
+  frg_ctx* ctx = contextFor(device);
+
+  const int size = getSize();
+  const int rank = getRank();
+  std::vector<at::Tensor> peers = peers_;
+  TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
+              "fairring: this build runs on one GPU without a transport; a group of size ",
+              size, " needs ", size - 1, " simulated peer contributions, got ", peers.size());
+  bool fromHost = false;
+  for (size_t i = 0; i < peers.size(); ++i) {
+    at::Tensor& p = peers[i];
+    TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense(),
+                "fairring: peer contribution must be dense");
+    TORCH_CHECK(p.scalar_type() == t.scalar_type() && p.numel() == t.numel(),
+                "fairring: peer contribution must match the tensor's dtype and size");
+    p = viewAsFlat(p);
+    if (i == 0) fromHost = !p.is_cuda();
+    TORCH_CHECK(fromHost == !p.is_cuda(), "fairring: peers must be all on the GPU or all pinned");
+    if (fromHost) {
+      TORCH_CHECK(p.is_pinned(), "fairring: host-side peer contributions must be pinned");
+    } else {
+      TORCH_CHECK(p.device() == t.device(), "fairring: peer contribution on another device");
+    }
+  }
+
+  // Contribution table in rank order, this rank's own tensor at its index.
+  std::vector<const void*> table;
+  table.reserve(size);
+  for (int r = 0, pi = 0; r < size; ++r) {
+    table.push_back(r == rank ? t.data_ptr() : peers[pi++].data_ptr());
+  }
+
+  // Tell the caching allocator which streams will touch these buffers
+  // (fairring/device.cc:297-301).
+  void* streams[16];
+  int nStreams = 0;
+  TORCH_CHECK(frg_get_streams(ctx, streams, 16, &nStreams) == FRG_OK, frg_last_error());
+  for (int i = 0; i < nStreams && i < 16; ++i) {
+    c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
+        static_cast<hipStream_t>(streams[i]), device);
+    t.record_stream(s);
+    if (!fromHost) {
+      for (at::Tensor& p : peers) p.record_stream(s);
+    }
+  }
+
+  auto future = c10::make_intrusive<c10::ivalue::Future>(
+      c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
+
+  const bool divide = fusedDivide_ && op == c10d::ReduceOp::SUM && size > 1;
+  const bool pow2 = (size & (size - 1)) == 0;
+  const int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
+  const float scale = !divide ? 1.0f : (pow2 ? 1.0f / static_cast<float>(size)
+                                              : static_cast<float>(size));
+
+  hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
+  auto* pending = new Pending{future, t, std::move(peers), device};
+  int rc;
+  const int frgOp = op == c10d::ReduceOp::SUM ? FRG_SUM : FRG_MAX;
+  if (fromHost) {
+    // Server-side accumulation: this rank's own shard is already in the
+    // tensor, the peers' are staged from pinned memory and folded into it in
+    // rank order. The fixed order needs the resident contribution to be first.
+    if (rank != 0) {
+      delete pending;
+      TORCH_CHECK(false, "fairring: pinned peer contributions are folded after the resident "
+                         "tensor, which must therefore be rank 0 (got rank ", rank, ")");
+    }
+    rc = frg_allreduce_host(ctx, t.data_ptr(), table.data() + 1, size - 1, t.numel(), dtype,
+                            frgOp, scaleMode, scale, /*carry=*/1, current, &onDone, pending,
+                            nullptr);
+  } else {
+    rc = frg_allreduce(ctx, t.data_ptr(), table.data(), size, t.numel(), dtype, frgOp,
+                       scaleMode, scale, current, &onDone, pending, nullptr);
+  }
+  if (rc != FRG_OK) {
+    delete pending;
+    TORCH_CHECK(false, "fairring: ", frg_last_error());
+  }
+  return c10::make_intrusive<WorkFairring>(c10d::OpType::ALLREDUCE, std::move(future));
+}
+
+}  // namespace fairring

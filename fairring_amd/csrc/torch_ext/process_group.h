@@ -1,0 +1,106 @@
+// c10d backend "fairring" for PyTorch-ROCm on MI355X: the allreduce entry point
+// of the reference's ProcessGroupFairring (fairring/process_group.h:22-189),
+// re-targeted at the c10d::Backend / c10d::Work interfaces of current PyTorch
+// and driven through the C ABI of include/fairring_hip.h.
+//
+// One GPU, no transport: the contributions that peers would deliver are handed
+// in through setSimulatedPeerContributions() (not part of the reference), and
+// an allreduce on a group of size > 1 without them fails loudly.
+#pragma once
+
+#include <torch/csrc/distributed/c10d/Backend.hpp>
+#include <torch/csrc/distributed/c10d/Store.hpp>
+#include <torch/csrc/distributed/c10d/Work.hpp>
+#include <torch/torch.h>
+
+#include <map>
+#include <mutex>
+
+#include "../../../include/fairring_hip.h"
+
+namespace fairring {
+
+constexpr const char* kPgName = "fairring";
+
+class ProcessGroupFairring : public c10d::Backend {
+ public:
+  // fairring/process_group.h:24-50, fairring/process_group.cc:35-75
+  class WorkFairring : public c10d::Work {
+   public:
+    WorkFairring(c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future);
+    ~WorkFairring() override;
+
+    bool isCompleted() override;
+    bool isSuccess() const override;
+    std::exception_ptr exception() const override;
+    std::vector<at::Tensor> result() override;
+    void synchronize() override;
+    bool wait(std::chrono::milliseconds timeout = kNoTimeout) override;
+    void abort() override;
+    c10::intrusive_ptr<c10::ivalue::Future> getFuture() override;
+
+   private:
+    const c10::intrusive_ptr<c10::ivalue::Future> future_;
+  };
+
+  // fairring/process_group.h:52-77, plus the README's slice size
+  class OptionsFairring : public c10d::Backend::Options {
+   public:
+    explicit OptionsFairring(int64_t maxMemoryAllocatedInBytes,
+                             int64_t maxPaddingAllocatedInBytes, int64_t minParallelism,
+                             bool isHighPriorityStream = false,
+                             std::chrono::milliseconds timeout = kBackendDefaultTimeout,
+                             int64_t sliceSizeInBytes = 0);
+    ~OptionsFairring() override;
+
+    static c10::intrusive_ptr<OptionsFairring> create(
+        int64_t maxMemoryAllocatedInBytes, int64_t maxPaddingAllocatedInBytes,
+        int64_t minParallelism, bool isHighPriorityStream = false,
+        std::chrono::milliseconds timeout = kBackendDefaultTimeout,
+        int64_t sliceSizeInBytes = 0);
+
+    const int64_t maxMemoryAllocatedInBytes;
+    const int64_t maxPaddingAllocatedInBytes;
+    const int64_t minParallelism;
+    // Accepted for compatibility; every stream of the pipeline is created at
+    // the default priority.
+    const bool isHighPriorityStream;
+    const int64_t sliceSizeInBytes;
+  };
+
+  ProcessGroupFairring(const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
+                       c10::intrusive_ptr<OptionsFairring> options);
+  ~ProcessGroupFairring() override;
+
+  const std::string getBackendName() const override;
+
+  // fairring/process_group.cc:131-155
+  c10::intrusive_ptr<c10d::Work> allreduce(
+      std::vector<at::Tensor>& data,
+      const c10d::AllreduceOptions& opts = c10d::AllreduceOptions()) override;
+
+  // Not in the reference. The contributions of the other size-1 ranks, in rank
+  // order with this rank left out; GPU tensors on the caller's device or
+  // pinned CPU tensors (then they are staged through the pool). Used by every
+  // allreduce until replaced; an empty list clears them.
+  void setSimulatedPeerContributions(std::vector<at::Tensor> peers);
+
+  // Not in the reference. When on, SUM results are divided by the group size
+  // inside the reduction (DDP otherwise pre-divides each gradient).
+  void setFusedDivide(bool on);
+
+  // {slot size, slice size, padding slots, staging slots} once initialised.
+  std::vector<int64_t> layout();
+
+ private:
+  frg_ctx* contextFor(c10::DeviceIndex device);
+
+  c10::intrusive_ptr<c10d::Store> store_;
+  c10::intrusive_ptr<OptionsFairring> options_;
+  std::mutex mutex_;
+  std::map<c10::DeviceIndex, frg_ctx*> contexts_;  // built lazily (process_group.cc:140-152)
+  std::vector<at::Tensor> peers_;
+  bool fusedDivide_ = false;
+};
+
+}  // namespace fairring

@@ -153,7 +153,7 @@ class DeviceFairring:
                     padding_slots=out.num_padding_slots,
                     staging_slots=out.num_staging_slots)
 
-    def _submit(self, fn, out, contribs, op, scale_mode, scale, stream):
+    def _submit(self, out, contribs, op, scale_mode, scale, stream, host, carry=False):
         import torch
         _check_dense(out, "output")
         for c in contribs:
@@ -162,9 +162,14 @@ class DeviceFairring:
         stream = torch.cuda.current_stream(out.device) if stream is None else stream
         tab = _capi.ptr_table([c.data_ptr() for c in contribs])
         wh = ctypes.c_void_p()
-        _capi.check(fn(self._h, out.data_ptr(), tab, len(contribs), out.numel(),
-                       _dtype_code(out), op, scale_mode, scale, stream.cuda_stream,
-                       _capi.DONE_FN(), None, ctypes.byref(wh)))
+        L = _capi.lib()
+        head = (self._h, out.data_ptr(), tab, len(contribs), out.numel(), _dtype_code(out), op,
+                scale_mode, scale)
+        tail = (stream.cuda_stream, _capi.DONE_FN(), None, ctypes.byref(wh))
+        if host:
+            _capi.check(L.frg_allreduce_host(*head, 1 if carry else 0, *tail))
+        else:
+            _capi.check(L.frg_allreduce(*head, *tail))
         return Work(wh, (out, list(contribs)))
 
     def allreduce(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
@@ -172,19 +177,19 @@ class DeviceFairring:
         contributions given as GPU tensors. Returns at once."""
         for c in contribs:
             _check_dense(c, "contribution")
-        return self._submit(_capi.lib().frg_allreduce, out, contribs, op, scale_mode, scale,
-                            stream)
+        return self._submit(out, contribs, op, scale_mode, scale, stream, host=False)
 
     def allreduce_host(self, out, host_contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0,
-                       stream=None):
-        """Server-side accumulation of contributions held in pinned host memory."""
+                       carry=False, stream=None):
+        """Server-side accumulation of contributions held in pinned host memory;
+        with carry=True `out` already holds the first term of the sum."""
         for c in host_contribs:
             _check_dense(c, "contribution", device=False)
             if c.is_cuda or not c.is_pinned():
                 raise FairringError(_capi.ERR_INVALID,
                                     "host contributions must be pinned CPU tensors")
-        return self._submit(_capi.lib().frg_allreduce_host, out, host_contribs, op,
-                            scale_mode, scale, stream)
+        return self._submit(out, host_contribs, op, scale_mode, scale, stream, host=True,
+                            carry=carry)
 
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))

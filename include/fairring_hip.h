@@ -118,6 +118,11 @@ FRG_API int frg_destroy(frg_ctx* ctx);
 /* The layout in force (slice size, number of staging slots). */
 FRG_API int frg_get_layout(frg_ctx* ctx, frg_layout* out);
 
+/* The streams the pipeline launches on (reduce streams first, the copy stream
+ * last), for callers that must tell an allocator which streams touch a buffer
+ * (the reference calls record_stream on its five streams, device.cc:297-301). */
+FRG_API int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count);
+
 /* Called on the command thread once the last slice of an operation has been
  * enqueued (status FRG_OK) or enqueueing failed; `last_stream` is the stream
  * on which completion is ordered (device.cc:337-340 marks the future under a
@@ -142,12 +147,17 @@ FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
  * (device.cc:543-589: collect into a staging slot, then reduce): contribution
  * k is copied with hipMemcpyAsync on the copy stream into staging slot
  * (next++) % numSlots once the event recorded after that slot's previous
- * consumer has fired, and accumulated into `out` on the reduce stream in
- * contribution order. `contribs[k]` are host pointers (hipHostMalloc'd). */
+ * consumer has fired, and folded into `out` on the reduce stream in
+ * contribution order. `host_contribs[k]` are host pointers (hipHostMalloc'd).
+ * carry = 0: the K host contributions are all there is (the first one is
+ * copied straight into `out`). carry = 1: `out` already holds the device's own
+ * contribution, which comes first in the order (the reference reduces the
+ * staged shards into its own shard of the caller's tensor, device.cc:570-575);
+ * K may then be 0. */
 FRG_API int frg_allreduce_host(frg_ctx* ctx, void* out,
                                const void* const* host_contribs, int K,
                                int64_t numel, int dtype, int op, int scale_mode,
-                               float scale, void* producer_stream,
+                               float scale, int carry, void* producer_stream,
                                frg_done_fn done, void* user, frg_work** work);
 
 /* WorkFairring::wait / synchronize (process_group.cc:60-68): block the host
