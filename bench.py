@@ -1,15 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the K-way gradient-slice reduction on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
 
-Workload (the configuration the metric is quoted on): K = 8 simulated rank
-contributions of a 1.37 G-element fp32 gradient, N(0, sigma = 0.01) from a
-fixed seed, reduced in contribution order with the divide-by-8 fused into the
-store, processed as 25 MiB slices (210 of them, the last 297,600 elements)
-into one output buffer. A step is one pass over the whole gradient; inputs are
-resident in HBM before the timed region starts. Bytes counted per step are the
-algorithmic ones: (K + 1) * numel * 4 = 49.32 GB.
+Default workload c2 (the configuration the metric is quoted on): K = 8
+simulated rank contributions of a 1.37 G-element fp32 gradient, N(0, sigma =
+0.01) from fixed seeds, reduced in contribution order with the divide-by-8
+fused into the store, processed as 25 MiB slices (210 of them, the last
+297,600 elements) into one output buffer. A step is one pass over the whole
+gradient; inputs are resident in HBM before the timed region starts. Bytes
+counted are the algorithmic ones: (K + 1) * numel * elsize per step.
+
+Other workloads (the remaining BASELINE configurations, for the record):
+  c4    bf16, K = 8 x 1.3 G elements, fp32 accumulate, RNE store, fused /8
+  c3    K = 64 contributions of one 25 MiB fp32 slice staged from pinned host
+        memory with hipMemcpyAsync, overlapped with the accumulate kernel
+  c5    DDP backward stream: the 1.37 G gradient as 25 MiB buckets (first one
+        1 MiB) released in reverse order, one allreduce call per bucket
+  copy  K = 1 (a plain copy of known size), the calibration for HBM counters
 
 Prints one JSON line with the whole-job GB/s, the roofline of the reduction
 kernel (algorithmic bytes per launch / average launch duration from HIP events
@@ -34,8 +42,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--numel", type=int, default=1_370_000_000)
-    ap.add_argument("--k", type=int, default=8)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy"])
+    ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
+    ap.add_argument("--k", type=int, default=0, help="override the number of contributions")
     ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
     ap.add_argument("--total-memory", type=int, default=50 * MiB)
     ap.add_argument("--streams", type=int, default=0, help="reduce streams (0 = library default)")
@@ -46,7 +55,22 @@ def parse_args():
     return ap.parse_args()
 
 
-def check_parity(fa, oracle, np, torch, xs, out, numel, slice_elems, k):
+def oracle_slice(oracle, host, dtype, k, scale):
+    cores = os.cpu_count() or 1
+    if dtype == "f32":
+        mode = oracle.SCALE_MUL if scale else oracle.SCALE_NONE
+        return oracle.sum_f32(host, mode, 1.0 / k if scale else 1.0, threads=cores)
+    mode = oracle.SCALE_MUL if scale else oracle.SCALE_NONE
+    return oracle.sum_bf16(host, mode, 1.0 / k if scale else 1.0, threads=cores)
+
+
+def to_host(np, torch, t):
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.cpu().numpy()
+
+
+def check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale):
     """Bit-compare the first, a middle and the ragged last slice with the oracle
     fed the very bytes the GPU read."""
     n_slices = (numel + slice_elems - 1) // slice_elems
@@ -54,24 +78,30 @@ def check_parity(fa, oracle, np, torch, xs, out, numel, slice_elems, k):
     for idx in sorted({0, n_slices // 2, n_slices - 1}):
         lo = idx * slice_elems
         hi = min(numel, lo + slice_elems)
-        host = [x[lo:hi].cpu().numpy() for x in xs]
-        want = oracle.sum_f32(host, oracle.SCALE_MUL, 1.0 / k, threads=os.cpu_count() or 1)
-        got = out[lo:hi].cpu().numpy()
-        if not (got.view(np.uint32) == want.view(np.uint32)).all():
+        host = [to_host(np, torch, x[lo:hi]) for x in xs]
+        want = oracle_slice(oracle, host, dtype, k, scale)
+        got = to_host(np, torch, out[lo:hi])
+        if dtype == "f32":
+            ok = (got.view(np.uint32) == want.view(np.uint32)).all()
+        else:
+            ok = (got == want).all()
+        if not ok:
             raise SystemExit("parity FAILED on slice %d" % idx)
         checked.append(idx)
     return checked
 
 
-def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_slices_sample):
+def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
     """The contract's reduction on this host's cores: torch's at::add chain
-    (acc = x0; acc += xk; acc /= K) over `n_slices_sample` distinct 25 MiB
-    slices copied back from the GPU; >= 3 warm-up and 10 timed passes, median.
-    The repository's C restatement (OpenMP) is timed beside it."""
+    (acc = x0; acc += xk; acc /= K; bf16: fp32 accumulator, one final cast) over
+    `n_sample` distinct 25 MiB slices copied back from the GPU; 3 warm-up and 10
+    timed passes, median. The repository's C restatement (OpenMP) is timed
+    beside it. GB/s uses the same algorithmic-bytes formula as the GPU figure."""
     host = [[x[i * slice_elems:(i + 1) * slice_elems].cpu() for x in xs]
-            for i in range(n_slices_sample)]
+            for i in range(n_sample)]
     threads = torch.get_num_threads()
     acc = torch.empty(slice_elems, dtype=torch.float32)
+    res = torch.empty(slice_elems, dtype=xs[0].dtype)
 
     def one_pass():
         for sl in host:
@@ -79,6 +109,8 @@ def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_slices_sample):
             for c in sl[1:]:
                 acc.add_(c)
             acc.div_(float(k))
+            if dtype != "f32":
+                res.copy_(acc)
 
     for _ in range(3):
         one_pass()
@@ -88,27 +120,241 @@ def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_slices_sample):
         one_pass()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    algo_bytes = (k + 1) * slice_elems * 4 * n_slices_sample
+    elsize = 4 if dtype == "f32" else 2
+    algo_bytes = (k + 1) * slice_elems * elsize * n_sample
     torch_gbps = algo_bytes / med / 1e9
 
-    hnp = [[c.numpy() for c in sl] for sl in host]
     cores = os.cpu_count() or 1
+    hnp = [[to_host(np, torch, c) for c in sl] for sl in host]
+    fn = oracle.sum_f32 if dtype == "f32" else oracle.sum_bf16
+    kw = dict(chain=True) if dtype == "f32" else {}
     for sl in hnp[:2]:
-        oracle.sum_f32(sl, oracle.SCALE_DIV, float(k), chain=True, threads=cores)
+        fn(sl, oracle.SCALE_DIV, float(k), threads=cores, **kw)
     times = []
     for _ in range(5):
         t0 = time.perf_counter()
         for sl in hnp:
-            oracle.sum_f32(sl, oracle.SCALE_DIV, float(k), chain=True, threads=cores)
+            fn(sl, oracle.SCALE_DIV, float(k), threads=cores, **kw)
         times.append(time.perf_counter() - t0)
     c_gbps = algo_bytes / sorted(times)[len(times) // 2] / 1e9
     return {
         "value": round(torch_gbps, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-        "sample": "%d distinct 25 MiB slices x K=%d fp32, torch CPU at::add chain + div, "
-                  "median of 10 passes, %d torch threads of %d host cpus; same algorithmic-bytes "
-                  "formula" % (n_slices_sample, k, threads, cores),
+        "sample": "%d distinct 25 MiB slices x K=%d %s, torch CPU at::add chain + div, median of "
+                  "10 passes, %d torch threads of %d host cpus" % (n_sample, k, dtype, threads,
+                                                                    cores),
         "c_oracle_gbps": round(c_gbps, 2), "c_oracle_threads": cores,
     }
+
+
+def synth(torch, numel, k, dtype, seed0):
+    g = torch.Generator(device="cuda:0")
+    xs = []
+    for r in range(k):
+        g.manual_seed(seed0 + r)
+        t = torch.empty(numel, dtype=torch.float32, device="cuda:0").normal_(0.0, 0.01,
+                                                                             generator=g)
+        xs.append(t if dtype == "f32" else t.to(torch.bfloat16))
+        del t
+    return xs
+
+
+def kernel_roofline(fa, args, run_steps, n_launch_per_step, launch_bytes, keep):
+    """Average duration of the reduction launches on ONE reduce stream (launches
+    back to back, never overlapping, so a launch's duration is its own), each
+    bracketed by HIP events that take the dispatch's begin and end timestamps on
+    that stream. `keep(i)` selects the full-size launches of a step."""
+    dev1 = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                             slice_size_in_bytes=args.slice_bytes, num_reduce_streams=1)
+    dev1.set_profiling(True)
+    prof_steps = max(1, min(args.steps, 5))
+    for _ in range(prof_steps):
+        run_steps(dev1)
+    times_ms = dev1.kernel_times_ms()
+    dev1.set_profiling(False)
+    dev1.close()
+    assert len(times_ms) == prof_steps * n_launch_per_step, (len(times_ms), n_launch_per_step)
+    full = [t for i, t in enumerate(times_ms) if keep(i % n_launch_per_step)]
+    avg_ms = sum(full) / len(full)
+    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+    return {
+        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "launch_bytes": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 3),
+        "launches_timed": len(full),
+        "how": "HIP events on the launch's own stream, one reduce stream (no overlap)",
+    }
+
+
+def timed(torch, dev, steps, warmup, step):
+    for _ in range(warmup):
+        step(dev).wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    w = None
+    for _ in range(steps):
+        w = step(dev)
+    w.wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def run_resident(args, np, torch, fa, oracle, dtype):
+    """c2 / c4 / copy: device-resident contributions, one allreduce per step."""
+    elsize = 4 if dtype == "f32" else 2
+    if args.workload == "copy":
+        k, numel, scale = args.k or 1, args.numel or 1_370_000_000, False
+    elif dtype == "f32":
+        k, numel, scale = args.k or 8, args.numel or 1_370_000_000, True
+    else:
+        k, numel, scale = args.k or 8, args.numel or 1_300_000_000, True
+    slice_elems = args.slice_bytes // elsize
+    n_slices = (numel + slice_elems - 1) // slice_elems
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams)
+    xs = synth(torch, numel, k, dtype, 20240)
+    out = torch.empty(numel, dtype=xs[0].dtype, device="cuda:0")
+    torch.cuda.synchronize()
+    mode = fa.SCALE_MUL if scale else fa.SCALE_NONE
+
+    def step(d):
+        return d.allreduce(out, xs, scale_mode=mode, scale=1.0 / k)
+
+    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    step_bytes = (k + 1) * numel * elsize
+    value = step_bytes * args.steps / elapsed / 1e9
+    ragged = numel % slice_elems != 0
+    roof = kernel_roofline(fa, args, step, n_slices, (k + 1) * slice_elems * elsize,
+                           lambda i: not (ragged and i == n_slices - 1))
+    roof["kernel"] = "ksumKernel<%s, SUM, K=%d>" % ("F32Vec" if dtype == "f32" else "Bf16Vec", k)
+    step(dev).wait()
+    checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale)
+    layout = dev.layout
+    dev.close()
+    name = {"c2": "BASELINE configs[1]", "c4": "BASELINE configs[3]",
+            "copy": "calibration copy"}[args.workload]
+    cfg = {
+        "workload": "K=%d contributions x %d %s elements, %d slices of %d B, %s, one output "
+                    "buffer (%s)" % (k, numel, dtype, n_slices, args.slice_bytes,
+                                     "fused x1/%d" % k if scale else "no scale", name),
+        "k": k, "numel": numel, "slice_bytes": args.slice_bytes,
+        "staging_total_bytes": args.total_memory, "layout": layout,
+        "reduce_streams": args.streams or "default",
+    }
+    base = None
+    if not args.no_cpu_baseline and args.workload != "copy":
+        base = cpu_baseline(oracle, np, torch, xs, slice_elems, k,
+                            min(args.cpu_slices, max(1, n_slices - 1)), dtype)
+    return value, elapsed, cfg, roof, checked, base, dtype
+
+
+def run_c3(args, np, torch, fa, oracle):
+    """Server-side accumulation: K = 64 contributions of one 25 MiB fp32 slice in
+    pinned host memory, staged through the pool and folded in order."""
+    k, numel = args.k or 64, args.numel or 6_553_600
+    rng = np.random.default_rng(33)
+    hs = []
+    for r in range(k):
+        t = torch.empty(numel, dtype=torch.float32).pin_memory()
+        t.copy_(torch.from_numpy((rng.standard_normal(numel) * 0.01).astype(np.float32)))
+        hs.append(t)
+    out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams)
+
+    def step(d):
+        return d.allreduce_host(out, hs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+
+    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    step_bytes = (k + 1) * numel * 4
+    value = step_bytes * args.steps / elapsed / 1e9
+    link = k * numel * 4 * args.steps / elapsed / 1e9
+    slots = dev.layout["staging_slots"]
+    batch = max(1, slots // 2)
+    n_launch = -(-(k - 1) // batch)
+    # the accumulate kernel of a batch reads `batch` staged slots and `out`, writes `out`
+    roof = kernel_roofline(fa, args, step, n_launch, (batch + 2) * numel * 4,
+                           lambda i: (i + 1) * batch <= k - 1)
+    roof["kernel"] = "ksumKernel<F32Vec, SUM, carry, K=%d>" % batch
+    step(dev).wait()
+    want = oracle.sum_f32([h.numpy() for h in hs], oracle.SCALE_MUL, 1.0 / k,
+                          threads=os.cpu_count() or 1)
+    got = out.cpu().numpy()
+    if not (got.view(np.uint32) == want.view(np.uint32)).all():
+        raise SystemExit("parity FAILED (c3)")
+    layout = dev.layout
+    dev.close()
+    cfg = {
+        "workload": "K=%d pinned-host contributions of one %d-element fp32 slice, staged with "
+                    "hipMemcpyAsync through %d slots, fused x1/%d (BASELINE configs[2])" % (
+                        k, numel, slots, k),
+        "k": k, "numel": numel, "layout": layout, "host_link_GBps": round(link, 2),
+        "bound": "host link (PCIe): every contribution crosses it once",
+    }
+    return value, elapsed, cfg, roof, ["whole slice"], None, "f32"
+
+
+def ddp_buckets(numel, bucket_elems, first_elems):
+    """Buckets in the order DDP releases them: reverse parameter order, so from
+    the end of the flat gradient towards its start; the first one is small."""
+    spans = []
+    hi = numel
+    size = first_elems
+    while hi > 0:
+        lo = max(0, hi - size)
+        spans.append((lo, hi))
+        hi = lo
+        size = bucket_elems
+    return spans
+
+
+def run_c5(args, np, torch, fa, oracle):
+    k, numel = args.k or 8, args.numel or 1_370_000_000
+    slice_elems = args.slice_bytes // 4
+    spans = ddp_buckets(numel, slice_elems, MiB // 4)
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams)
+    xs = synth(torch, numel, k, "f32", 20240)
+    out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    views = [(out[lo:hi], [x[lo:hi] for x in xs]) for lo, hi in spans]
+    torch.cuda.synchronize()
+
+    class Last:
+        def __init__(self, works):
+            self.works = works
+
+        def wait(self):
+            for w in self.works:
+                w.wait()
+
+    def step(d):
+        return Last([d.allreduce(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+                     for o, cs in views])
+
+    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    step_bytes = (k + 1) * numel * 4
+    value = step_bytes * args.steps / elapsed / 1e9
+    full = [i for i, (lo, hi) in enumerate(spans) if hi - lo == slice_elems]
+    roof = kernel_roofline(fa, args, step, len(spans), (k + 1) * slice_elems * 4,
+                           lambda i: i in set(full))
+    roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
+    step(dev).wait()
+    checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)
+    layout = dev.layout
+    dev.close()
+    cfg = {
+        "workload": "DDP backward stream: %d fp32 elements as %d buckets (first %d B, then %d B) "
+                    "released from the end of the gradient to its start, K=%d contributions per "
+                    "bucket, one allreduce call per bucket, fused x1/%d (BASELINE configs[4])" % (
+                        numel, len(spans), MiB, args.slice_bytes, k, k),
+        "k": k, "numel": numel, "buckets": len(spans), "staging_total_bytes": args.total_memory,
+        "layout": layout, "reduce_streams": args.streams or "default",
+    }
+    return value, elapsed, cfg, roof, checked, None, "f32"
 
 
 def main():
@@ -122,6 +368,7 @@ def main():
     import torch
 
     import fairring_amd as fa
+    import oracle
     from fairring_amd import _capi
 
     if not torch.cuda.is_available():
@@ -130,73 +377,31 @@ def main():
     if args.blocks_per_cu or args.xcd_remap:
         _capi.lib().frg_set_tuning(args.blocks_per_cu, args.xcd_remap)
 
-    k, numel = args.k, args.numel
-    slice_elems = args.slice_bytes // 4
-    n_slices = (numel + slice_elems - 1) // slice_elems
-    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
-                            slice_size_in_bytes=args.slice_bytes,
-                            num_reduce_streams=args.streams)
+    if args.workload in ("c2", "copy"):
+        value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,
+                                                                       oracle, "f32")
+    elif args.workload == "c4":
+        value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,
+                                                                       oracle, "bf16")
+    elif args.workload == "c3":
+        value, elapsed, cfg, roof, checked, base, dtype = run_c3(args, np, torch, fa, oracle)
+    else:
+        value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle)
 
-    g = torch.Generator(device="cuda:0")
-    xs = []
-    for r in range(k):
-        g.manual_seed(20240 + r)
-        xs.append(torch.empty(numel, dtype=torch.float32, device="cuda:0")
-                  .normal_(0.0, 0.01, generator=g))
-    out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
-    torch.cuda.synchronize()
-
-    def step():
-        return dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
-
-    for _ in range(args.warmup):
-        step().wait()
-    dev.synchronize()
-    torch.cuda.synchronize()
-
-    t0 = time.perf_counter()
-    w = None
-    for _ in range(args.steps):
-        w = step()
-    w.wait()
-    dev.synchronize()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-
-    step_bytes = (k + 1) * numel * 4
-    value = step_bytes * args.steps / elapsed / 1e9
-
-    # Roofline of the dominant kernel: the same steps again on ONE reduce stream
-    # (launches back to back, never overlapping, so a launch's duration is its
-    # own), each launch bracketed by HIP events that take the dispatch's begin
-    # and end timestamps on that stream.
-    dev1 = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
-                             slice_size_in_bytes=args.slice_bytes, num_reduce_streams=1)
-    dev1.set_profiling(True)
-    prof_steps = max(1, min(args.steps, 5))
-    for _ in range(prof_steps):
-        dev1.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
-    times_ms = dev1.kernel_times_ms()
-    dev1.set_profiling(False)
-    dev1.close()
-    assert len(times_ms) == prof_steps * n_slices, (len(times_ms), n_slices)
-    # full 25 MiB slices only: the ragged last launch of each step is left out
-    full = [t for i, t in enumerate(times_ms) if (i % n_slices) != n_slices - 1 or
-            numel % slice_elems == 0]
-    avg_ms = sum(full) / len(full)
-    launch_bytes = (k + 1) * slice_elems * 4
-    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
-
-    checked = check_parity(fa, __import__("oracle"), np, torch, xs, out, numel, slice_elems, k)
-
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_traffic.json")
-    if os.path.exists(tpath) and k == 8 and args.slice_bytes == 25 * MiB:
+    tpath = os.path.join(ROOT, "profiles", "ksum_traffic.json")
+    if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+            roof["traffic"] = json.load(f).get(args.workload, {}).get("hbm_bytes_per_launch")
 
+    metric = {
+        "c2": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",
+        "c4": "reduce GB/s (bytes read+written), 8-way bf16, 25 MiB slices",
+        "c3": "reduce GB/s (bytes read+written at HBM level), 64-way fp32 host-staged, one slice",
+        "c5": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream",
+        "copy": "copy GB/s (bytes read+written), 25 MiB slices",
+    }[args.workload]
     result = {
-        "metric": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",
+        "metric": metric,
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -206,31 +411,16 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic: N(0, sigma=0.01) per contribution from fixed seeds, resident in HBM",
-        "config": {
-            "workload": "K=%d contributions x %d fp32 elements, %d slices of %d B, fused x1/%d, "
-                        "one output buffer (BASELINE configs[1])" % (k, numel, n_slices,
-                                                                      args.slice_bytes, k),
-            "k": k, "numel": numel, "slice_bytes": args.slice_bytes,
-            "staging_total_bytes": args.total_memory, "layout": dev.layout,
-            "reduce_streams": args.streams or "default",
-        },
+        "dtype": dtype,
+        "data": "synthetic: N(0, sigma=0.01) per contribution from fixed seeds, resident before "
+                "the timed region",
+        "config": cfg,
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "parity": "bit-exact vs CPU oracle on slices %s" % checked,
-        "roofline": {
-            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-            "kernel": "ksumKernel<F32Vec, SUM, K=8>", "launch_bytes": launch_bytes,
-            "avg_launch_us": round(avg_ms * 1e3, 3), "launches_timed": len(full),
-            "how": "HIP events on the launch's own stream, one reduce stream (no overlap)",
-        },
+        "roofline": roof,
     }
-    if not args.no_cpu_baseline:
-        import oracle
-        result["cpu_baseline"] = cpu_baseline(oracle, np, torch, xs, slice_elems, k,
-                                              min(args.cpu_slices, max(1, n_slices - 1)))
-    dev.close()
+    if base is not None:
+        result["cpu_baseline"] = base
     print(json.dumps(result))
 
 
