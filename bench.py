@@ -388,10 +388,16 @@ def main():
     else:
         value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle)
 
-    tpath = os.path.join(ROOT, "profiles", "ksum_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            roof["traffic"] = json.load(f).get(args.workload, {}).get("hbm_bytes_per_launch")
+    # HBM bytes per launch as measured with rocprofv3 --pmc (two counter runs,
+    # scaled by a copy of known size); the summary that holds the figure names
+    # the commands that produced it.
+    if args.workload == "c2" and args.slice_bytes == 25 * MiB and not args.k:
+        tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_25MiB_hbm_traffic.md")
+        if os.path.exists(tpath):
+            import re
+            m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", open(tpath).read())
+            if m:
+                roof["traffic"] = int(m.group(1).replace(",", ""))
 
     metric = {
         "c2": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",
