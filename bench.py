@@ -48,8 +48,9 @@ def parse_args():
     ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
     ap.add_argument("--total-memory", type=int, default=50 * MiB)
     ap.add_argument("--streams", type=int, default=0, help="reduce streams (0 = library default)")
+    ap.add_argument("--launch-bytes", type=int, default=0,
+                    help="bytes of one contribution per launch (0 = library default, -1 = slice)")
     ap.add_argument("--blocks-per-cu", type=int, default=0)
-    ap.add_argument("--xcd-remap", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-slices", type=int, default=8)
     return ap.parse_args()
@@ -158,46 +159,109 @@ def synth(torch, numel, k, dtype, seed0):
     return xs
 
 
-def kernel_roofline(fa, args, run_steps, n_launch_per_step, launch_bytes, keep):
-    """Average duration of the reduction launches on ONE reduce stream (launches
-    back to back, never overlapping, so a launch's duration is its own), each
-    bracketed by HIP events that take the dispatch's begin and end timestamps on
-    that stream. `keep(i)` selects the full-size launches of a step."""
-    dev1 = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
-                             slice_size_in_bytes=args.slice_bytes, num_reduce_streams=1)
-    dev1.set_profiling(True)
-    prof_steps = max(1, min(args.steps, 5))
-    for _ in range(prof_steps):
-        run_steps(dev1)
-    times_ms = dev1.kernel_times_ms()
-    dev1.set_profiling(False)
-    dev1.close()
-    assert len(times_ms) == prof_steps * n_launch_per_step, (len(times_ms), n_launch_per_step)
-    full = [t for i, t in enumerate(times_ms) if keep(i % n_launch_per_step)]
-    avg_ms = sum(full) / len(full)
-    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+def union_length(intervals):
+    """Total length of the union of (begin, end) intervals."""
+    total, cur_b, cur_e = 0.0, None, None
+    for b, e in sorted(intervals):
+        if cur_e is None or b > cur_e:
+            if cur_e is not None:
+                total += cur_e - cur_b
+            cur_b, cur_e = b, e
+        else:
+            cur_e = max(cur_e, e)
+    if cur_e is not None:
+        total += cur_e - cur_b
+    return total
+
+
+DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch size per contribution
+
+
+def launch_elems(args, slice_elems, elsize):
+    """Elements of one full-size launch: a slice is cut into equal parts no larger
+    than the launch size (what the pipeline does)."""
+    lb = args.launch_bytes or DEFAULT_LAUNCH_BYTES
+    if lb < 0:
+        return slice_elems
+    max_elems = (lb - lb % 16) // elsize
+    parts = -(-slice_elems // max_elems)
+    lanes = 16 // elsize
+    per = -(-slice_elems // parts)
+    return -(-per // lanes) * lanes
+
+
+def roofline_from_records(recs, bytes_per_elem, full_launch_elems, how):
+    """Roofline of the reduction kernel from HIP-event records on its streams.
+    Launches on the two reduce streams overlap on purpose, so a launch's
+    duration alone understates the kernel: while two launches run, each sees
+    half the bandwidth. The kernel's achieved rate is the algorithmic bytes of
+    the recorded launches divided by the time during which at least one of them
+    was running (the union of the recorded intervals); avg_launch_us and
+    concurrency (sum of durations / union) are reported beside it, so that
+    achieved = launch_bytes * concurrency / avg_launch (up to the ragged last
+    launch of a step)."""
+    durs = [r[1] - r[0] for r in recs]
+    launches = sum(r[5] for r in recs)
+    elems = sum(r[2] for r in recs)
+    busy_ms = union_length([(r[0], r[1]) for r in recs])
+    achieved = elems * bytes_per_elem / (busy_ms * 1e-3) / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-        "launch_bytes": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 3),
-        "launches_timed": len(full),
-        "how": "HIP events on the launch's own stream, one reduce stream (no overlap)",
+        "launch_bytes": full_launch_elems * bytes_per_elem, "launch_elems": full_launch_elems,
+        "avg_launch_us": round(sum(durs) / launches * 1e3, 3), "launches_timed": launches,
+        "concurrency": round(sum(durs) / busy_ms, 3),
+        "streams_used": len({r[4] for r in recs}),
+        "how": how,
     }
 
 
-def timed(torch, dev, steps, warmup, step):
+SPAN_HOW = ("HIP events on each reduce stream over the timed region: one before its first launch "
+            "of the region, one after its last (launches on a stream run back to back); achieved "
+            "= algorithmic bytes of those launches / union of the two spans")
+LAUNCH_HOW = ("HIP events taking begin/end of every dispatch on its own stream, in a separate "
+              "pass after the timed region; achieved = algorithmic bytes / union of the intervals")
+
+
+def timed(torch, dev, steps, warmup, step, spans=True):
+    """W untimed steps, then exactly `steps` timed ones between synchronisations.
+    With spans, one HIP event per reduce stream is recorded at the start of the
+    timed region and one at its end, on the streams the kernel runs on."""
     for _ in range(warmup):
         step(dev).wait()
     dev.synchronize()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    if spans:
+        dev.profile_mark()
     w = None
     for _ in range(steps):
         w = step(dev)
+    if spans:
+        dev.profile_mark()
     w.wait()
     dev.synchronize()
     torch.cuda.synchronize()
-    return time.perf_counter() - t0
+    elapsed = time.perf_counter() - t0
+    recs = dev.launch_records() if spans else None
+    return elapsed, recs
+
+
+def per_launch_pass(fa, args, run_steps):
+    """A separate pass with every launch timed by its own dispatch timestamps."""
+    dev1 = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                             slice_size_in_bytes=args.slice_bytes,
+                             num_reduce_streams=args.streams,
+                             max_launch_bytes=args.launch_bytes)
+    run_steps(dev1).wait()
+    dev1.synchronize()
+    dev1.set_profiling(True)
+    for _ in range(max(1, min(args.steps, 5))):
+        run_steps(dev1)
+    recs = dev1.launch_records()
+    dev1.set_profiling(False)
+    dev1.close()
+    return recs
 
 
 def run_resident(args, np, torch, fa, oracle, dtype):
@@ -213,7 +277,8 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     n_slices = (numel + slice_elems - 1) // slice_elems
     dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                             slice_size_in_bytes=args.slice_bytes,
-                            num_reduce_streams=args.streams)
+                            num_reduce_streams=args.streams,
+                            max_launch_bytes=args.launch_bytes)
     xs = synth(torch, numel, k, dtype, 20240)
     out = torch.empty(numel, dtype=xs[0].dtype, device="cuda:0")
     torch.cuda.synchronize()
@@ -222,12 +287,11 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     def step(d):
         return d.allreduce(out, xs, scale_mode=mode, scale=1.0 / k)
 
-    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     step_bytes = (k + 1) * numel * elsize
     value = step_bytes * args.steps / elapsed / 1e9
-    ragged = numel % slice_elems != 0
-    roof = kernel_roofline(fa, args, step, n_slices, (k + 1) * slice_elems * elsize,
-                           lambda i: not (ragged and i == n_slices - 1))
+    roof = roofline_from_records(recs, (k + 1) * elsize, launch_elems(args, slice_elems, elsize),
+                                 SPAN_HOW)
     roof["kernel"] = "ksumKernel<%s, SUM, K=%d>" % ("F32Vec" if dtype == "f32" else "Bf16Vec", k)
     step(dev).wait()
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale)
@@ -242,6 +306,7 @@ def run_resident(args, np, torch, fa, oracle, dtype):
         "k": k, "numel": numel, "slice_bytes": args.slice_bytes,
         "staging_total_bytes": args.total_memory, "layout": layout,
         "reduce_streams": args.streams or "default",
+        "launch_bytes_per_contribution": args.launch_bytes or "default",
     }
     base = None
     if not args.no_cpu_baseline and args.workload != "copy":
@@ -263,21 +328,22 @@ def run_c3(args, np, torch, fa, oracle):
     out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
     dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                             slice_size_in_bytes=args.slice_bytes,
-                            num_reduce_streams=args.streams)
+                            num_reduce_streams=args.streams,
+                            max_launch_bytes=args.launch_bytes)
 
     def step(d):
         return d.allreduce_host(out, hs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
 
-    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    elapsed, _ = timed(torch, dev, args.steps, args.warmup, step, spans=False)
     step_bytes = (k + 1) * numel * 4
     value = step_bytes * args.steps / elapsed / 1e9
     link = k * numel * 4 * args.steps / elapsed / 1e9
     slots = dev.layout["staging_slots"]
     batch = max(1, slots // 2)
-    n_launch = -(-(k - 1) // batch)
     # the accumulate kernel of a batch reads `batch` staged slots and `out`, writes `out`
-    roof = kernel_roofline(fa, args, step, n_launch, (batch + 2) * numel * 4,
-                           lambda i: (i + 1) * batch <= k - 1)
+    recs = per_launch_pass(fa, args, step)
+    recs = [r for r in recs if r[3] == batch]
+    roof = roofline_from_records(recs, (batch + 2) * 4, numel, LAUNCH_HOW)
     roof["kernel"] = "ksumKernel<F32Vec, SUM, carry, K=%d>" % batch
     step(dev).wait()
     want = oracle.sum_f32([h.numpy() for h in hs], oracle.SCALE_MUL, 1.0 / k,
@@ -317,11 +383,13 @@ def run_c5(args, np, torch, fa, oracle):
     spans = ddp_buckets(numel, slice_elems, MiB // 4)
     dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                             slice_size_in_bytes=args.slice_bytes,
-                            num_reduce_streams=args.streams)
+                            num_reduce_streams=args.streams,
+                            max_launch_bytes=args.launch_bytes)
     xs = synth(torch, numel, k, "f32", 20240)
     out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
     views = [(out[lo:hi], [x[lo:hi] for x in xs]) for lo, hi in spans]
     torch.cuda.synchronize()
+    prepared = {}
 
     class Last:
         def __init__(self, works):
@@ -332,15 +400,16 @@ def run_c5(args, np, torch, fa, oracle):
                 w.wait()
 
     def step(d):
-        return Last([d.allreduce(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
-                     for o, cs in views])
+        # one allreduce call per bucket, in release order; the calls are marshalled once
+        if id(d) not in prepared:
+            prepared[id(d)] = [d.prepare(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+                               for o, cs in views]
+        return Last([submit() for submit in prepared[id(d)]])
 
-    elapsed = timed(torch, dev, args.steps, args.warmup, step)
+    elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     step_bytes = (k + 1) * numel * 4
     value = step_bytes * args.steps / elapsed / 1e9
-    full = [i for i, (lo, hi) in enumerate(spans) if hi - lo == slice_elems]
-    roof = kernel_roofline(fa, args, step, len(spans), (k + 1) * slice_elems * 4,
-                           lambda i: i in set(full))
+    roof = roofline_from_records(recs, (k + 1) * 4, launch_elems(args, slice_elems, 4), SPAN_HOW)
     roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
     step(dev).wait()
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)
@@ -374,8 +443,8 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
     _capi.lib()  # fail now if the HIP library is missing
-    if args.blocks_per_cu or args.xcd_remap:
-        _capi.lib().frg_set_tuning(args.blocks_per_cu, args.xcd_remap)
+    if args.blocks_per_cu:
+        _capi.lib().frg_set_tuning(args.blocks_per_cu)
 
     if args.workload in ("c2", "copy"):
         value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,

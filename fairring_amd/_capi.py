@@ -19,7 +19,8 @@ EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_reduce_slice",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
-    "frg_synchronize", "frg_set_profiling", "frg_kernel_times", "frg_set_tuning",
+    "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
+    "frg_set_tuning",
     "frg_last_error", "frg_version",
 )
 
@@ -44,6 +45,14 @@ class Options(ctypes.Structure):
                 ("slice_size_in_bytes", ctypes.c_int64),
                 ("num_machines", ctypes.c_int64),
                 ("num_reduce_streams", ctypes.c_int32),
+                ("reserved", ctypes.c_int32),
+                ("max_launch_bytes", ctypes.c_int64)]
+
+
+class LaunchRecord(ctypes.Structure):
+    _fields_ = [("begin_ms", ctypes.c_float), ("end_ms", ctypes.c_float),
+                ("numel", ctypes.c_int64), ("num_contributions", ctypes.c_int32),
+                ("stream_index", ctypes.c_int32), ("launches", ctypes.c_int32),
                 ("reserved", ctypes.c_int32)]
 
 
@@ -80,12 +89,14 @@ def lib():
     L.frg_allreduce.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
     L.frg_allreduce_host.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp,
                                      DONE_FN, vp, pvp]
-    for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize):
+    for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize,
+               L.frg_profile_mark):
         fn.argtypes = [vp]
     L.frg_work_block_stream.argtypes = [vp, vp]
     L.frg_set_profiling.argtypes = [vp, i32]
     L.frg_kernel_times.argtypes = [vp, ctypes.POINTER(ctypes.c_float), i32, ctypes.POINTER(i32)]
-    L.frg_set_tuning.argtypes = [i32, i32]
+    L.frg_launch_records.argtypes = [vp, ctypes.POINTER(LaunchRecord), i32, ctypes.POINTER(i32)]
+    L.frg_set_tuning.argtypes = [i32]
     L.frg_last_error.restype = ctypes.c_char_p
     L.frg_version.restype = ctypes.c_char_p
     _lib = L

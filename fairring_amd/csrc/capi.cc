@@ -204,9 +204,17 @@ int frg_synchronize(frg_ctx* ctx) {
   return FRG_OK;
 }
 
-int frg_set_profiling(frg_ctx* ctx, int on) {
+int frg_profile_mark(frg_ctx* ctx) {
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  asCtx(ctx)->setProfiling(on != 0);
+  std::string err;
+  const int rc = asCtx(ctx)->profileMark(&err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_set_profiling(frg_ctx* ctx, int per_launch) {
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  asCtx(ctx)->setProfiling(per_launch != 0);
   return FRG_OK;
 }
 
@@ -218,8 +226,16 @@ int frg_kernel_times(frg_ctx* ctx, float* ms, int capacity, int* count) {
   return FRG_OK;
 }
 
-int frg_set_tuning(int blocks_per_cu, int xcd_remap) {
-  frg::setTuning(blocks_per_cu, xcd_remap);
+int frg_launch_records(frg_ctx* ctx, frg_launch_record* records, int capacity, int* count) {
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  std::string err;
+  const int rc = asCtx(ctx)->launchRecords(records, capacity, count, &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
+int frg_set_tuning(int blocks_per_cu) {
+  frg::setTuning(blocks_per_cu);
   return FRG_OK;
 }
 

@@ -32,6 +32,6 @@ struct ReduceArgs {
 int launchReduce(const ReduceArgs& args, hipStream_t stream, std::string* err);
 
 // Launch-shape knobs (process-wide); 0 keeps the default.
-void setTuning(int blocksPerCu, int xcdRemap);
+void setTuning(int blocksPerCu);
 
 }  // namespace frg

@@ -47,6 +47,11 @@
 // Loads in flight per CU that the grid is sized for: blocks per CU =
 // FRG_LOADS_PER_CU / (loads per lane), so that fewer contributions per launch
 // are made up for by more resident waves.
+// Vectors per lane in a piece of the remainder round (1 = pieces of kBlock
+// vectors, spread over the most blocks; FRG_UNROLL = whole tiles).
+#ifndef FRG_REMAINDER_PIECE_UNROLL
+#define FRG_REMAINDER_PIECE_UNROLL 1
+#endif
 #ifndef FRG_LOADS_PER_CU
 #define FRG_LOADS_PER_CU 32
 #endif
@@ -251,36 +256,42 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
 }
 
 // Body kernel. The slice is [head scalars][nvec vectors][tail scalars], where
-// `head` brings every pointer to a 16-byte boundary. Tiles of kBlock*kUnroll
-// vectors are dealt to the blocks round-robin; with xcdRemap each of the 8 XCDs
-// (hardware deals consecutive blocks to consecutive XCDs) walks its own
-// contiguous eighth of the slice.
+// `head` brings every pointer to a 16-byte boundary. Full tiles of
+// kBlock*kUnroll vectors are dealt to the blocks round-robin for as many whole
+// rounds as there are. What is left (fewer tiles than blocks) is dealt in
+// pieces of kBlock vectors, again from block 0 upwards: the hardware places
+// blocks on CUs round-robin, so spreading the remainder over twice as many
+// blocks in half-size pieces evens out the work per CU, and the launch does not
+// end on a few CUs finishing a whole extra tile.
 template <typename TRV, typename TRS, int OP, int KT>
 __global__ void __launch_bounds__(kBlock)
     ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K, int carry,
                int scaleMode, float scale, int64_t head, int64_t nvec,
-               int64_t tail, int xcdRemap) {
+               int64_t tail) {
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
-  const int64_t ntiles = (nvec + kTile - 1) / kTile;
-  const int64_t perXcd = ntiles >> 3;
-  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const int64_t tile = xcdRemap ? ((t & 7) * perXcd + (t >> 3)) : t;
-    const int64_t v0 = tile * kTile;
-    const int64_t elemBase = head + v0 * TRV::kLanes;
-    if (v0 + kTile <= nvec) {
+  const int64_t grid = gridDim.x;
+  const int64_t roundTiles = (nvec / kTile / grid) * grid;  // tiles in whole rounds
+  for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
+    const int64_t elemBase = head + t * kTile * TRV::kLanes;
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale, elemBase,
-                               threadIdx.x + u * kBlock);
-      }
-    } else {
+    for (int u = 0; u < kUnroll; ++u) {
+      reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale, elemBase,
+                             threadIdx.x + u * kBlock);
+    }
+  }
+  // remainder: pieces of kBlock vectors, the last one possibly partial
+  const int64_t restBase = roundTiles * kTile;
+  constexpr int kPiece = FRG_REMAINDER_PIECE_UNROLL;  // vectors per lane in a remainder piece
+  const int64_t pieceVecs = static_cast<int64_t>(kBlock) * kPiece;
+  const int64_t pieces = (nvec - restBase + pieceVecs - 1) / pieceVecs;
+  for (int64_t p = blockIdx.x; p < pieces; p += grid) {
+    const int64_t v0 = restBase + p * pieceVecs;
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const unsigned int lane = threadIdx.x + u * kBlock;
-        if (v0 + lane < nvec) {
-          reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale,
-                                 elemBase, lane);
-        }
+    for (int u = 0; u < kPiece; ++u) {
+      const unsigned int lane = threadIdx.x + u * kBlock;
+      if (v0 + lane < nvec) {
+        reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale,
+                               head + v0 * TRV::kLanes, lane);
       }
     }
   }
@@ -316,7 +327,6 @@ DeviceInfo& deviceInfo(int device) {
 }
 
 int gBlocksPerCu = 0;  // 0 = derive from the number of loads per lane
-int gXcdRemap = 0;
 
 template <typename TRV, typename TRS, int OP, int KT>
 hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
@@ -334,27 +344,24 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
     blocksPerCu = FRG_LOADS_PER_CU / perLane;
     if (blocksPerCu < 1) blocksPerCu = 1;
   }
-  // Persistent grid of at most `cap` blocks, shrunk so that every block walks
-  // the same number of tiles (within one): no half-empty last round.
+  // Persistent grid: a whole number of blocks per CU. The hardware deals blocks
+  // to CUs round-robin, every block gets the same share of tiles, and a CU that
+  // hosts one block more than its neighbours becomes the straggler the whole
+  // launch waits for; measured on MI355X, 520 blocks are 15 % slower than 512.
   const int64_t cap = static_cast<int64_t>(numCus) * blocksPerCu;
-  int64_t grid = 1;
-  if (ntiles > 0) {
-    const int64_t rounds = (ntiles + cap - 1) / cap;
-    grid = (ntiles + rounds - 1) / rounds;
-  }
-  int remap = 0;
-  if (gXcdRemap && (ntiles % 8 == 0) && (grid % 8 == 0)) remap = 1;
+  int64_t grid = ntiles < cap ? ntiles : cap;
+  if (grid < 1) grid = 1;
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
     // Timed launch: the events take the dispatch's own begin/end timestamps.
     hipExtLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT>), dim3(static_cast<unsigned>(grid)),
                           dim3(kBlock), 0, stream, a.startEvent, a.stopEvent, 0,
                           static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                          a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, remap);
+                          a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail);
   } else {
     hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT>), dim3(static_cast<unsigned>(grid)),
                        dim3(kBlock), 0, stream,
                        static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                       a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, remap);
+                       a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail);
   }
   return hipGetLastError();
 }
@@ -379,10 +386,7 @@ hipError_t dispatchK(const ReduceArgs& a, int64_t head, int64_t nvec,
 
 }  // namespace
 
-void setTuning(int blocksPerCu, int xcdRemap) {
-  gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0;
-  gXcdRemap = xcdRemap > 0 ? 1 : 0;
-}
+void setTuning(int blocksPerCu) { gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0; }
 
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   auto fail = [&](int code, const std::string& msg) {

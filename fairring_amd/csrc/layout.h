@@ -17,6 +17,7 @@ constexpr int64_t kAlignment = 8;
 constexpr int64_t kDefaultTotalMemory = 50ll * 1024 * 1024;   // fairring/__init__.py:26
 constexpr int64_t kDefaultPaddingMemory = 1024ll * 1024;      // fairring/__init__.py:30
 constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init__.py:34
+constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;  // per contribution and launch
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {
   return num == 0 ? 0 : (num - 1) / den + 1;

@@ -112,12 +112,17 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->layout_ = layout;
   c->numSlots_ = layout.numStagingSlots;
   c->slotBytes_ = layout.slotSizeInBytes;
+  // Measured on MI355X (K = 8 fp32): launches of 12.5 MiB per contribution,
+  // alternating over two streams, sustain 6.45 TB/s where one 25 MiB launch per
+  // slice sustains 6.25: short launches keep the blocks of a grid in step, and
+  // the second stream fills the ramp and drain of the first.
+  c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
+                                               : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
+  c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
   try {
     DeviceGuard g(device);
-    int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams
-                                            : static_cast<int>(c->numSlots_ < 2 ? c->numSlots_ : 2);
-    if (nStreams > c->numSlots_) nStreams = static_cast<int>(c->numSlots_);
-    if (nStreams < 1) nStreams = 1;
+    int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams : 2;
+    if (nStreams > 8) nStreams = 8;
     // Default priority on purpose: all streams of the pipeline share one level.
     for (int i = 0; i < nStreams; ++i) {
       hipStream_t s;
@@ -135,6 +140,8 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
       c->slotFilledEvents_.push_back(b);
     }
     c->slotUsed_.assign(static_cast<size_t>(c->numSlots_), 0);
+    c->streamLaunches_.assign(c->reduceStreams_.size(), 0);
+    c->streamElems_.assign(c->reduceStreams_.size(), 0);
   } catch (const std::exception& e) {
     *err = e.what();
     // partially built: release what exists, without a command thread to join
@@ -171,8 +178,11 @@ Context::~Context() {
   for (hipEvent_t e : slotFilledEvents_) (void)hipEventDestroy(e);
   for (hipEvent_t e : freeEvents_) (void)hipEventDestroy(e);
   for (auto& p : profEvents_) {
-    (void)hipEventDestroy(p.first);
-    (void)hipEventDestroy(p.second);
+    (void)hipEventDestroy(p.begin);
+    (void)hipEventDestroy(p.end);
+  }
+  for (auto& m : marks_) {
+    for (hipEvent_t e : m.events) (void)hipEventDestroy(e);
   }
   // The streams are not destroyed: a consumer may still hold an event that
   // orders its own stream after one of them (fairring/machine.cc:162-175).
@@ -200,7 +210,7 @@ void Context::giveEvent(hipEvent_t e) {
 
 void Context::releaseWork(Work* w) {
   if (w->refs.fetch_sub(1) == 1) {
-    if (w->doneEvent) (void)hipEventDestroy(w->doneEvent);
+
     delete w;
   }
 }
@@ -221,7 +231,7 @@ int Context::waitWork(Work* w, std::string* err) {
   }
   try {
     DeviceGuard g(w->device);
-    FRG_HIP_CHECK(hipEventSynchronize(w->doneEvent));
+    for (hipStream_t s : w->doneStreams) FRG_HIP_CHECK(hipStreamSynchronize(s));
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;
@@ -240,7 +250,15 @@ int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
   }
   try {
     DeviceGuard g(w->device);
-    FRG_HIP_CHECK(hipStreamWaitEvent(stream, w->doneEvent, 0));
+    for (hipStream_t s : w->doneStreams) {
+      if (s == stream) continue;
+      hipEvent_t e;
+      FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      hipError_t r = hipEventRecord(e, s);
+      if (r == hipSuccess) r = hipStreamWaitEvent(stream, e, 0);
+      (void)hipEventDestroy(e);  // released once the recorded work has passed
+      FRG_HIP_CHECK(r);
+    }
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;
@@ -296,7 +314,6 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   hipEvent_t initial = nullptr;
   try {
     DeviceGuard g(device_);
-    FRG_HIP_CHECK(hipEventCreateWithFlags(&work->doneEvent, hipEventDisableTiming));
     // Orders the pipeline after whatever produced the inputs
     // (fairring/device.cc:294-295).
     initial = takeEvent();
@@ -324,10 +341,19 @@ void Context::launch(const ReduceArgs& args, hipStream_t stream) {
   }
   std::string err;
   const int rc = launchReduce(a, stream, &err);
+  if (rc == FRG_OK && args.n > 0) {
+    for (size_t i = 0; i < reduceStreams_.size(); ++i) {
+      if (reduceStreams_[i] == stream) {
+        streamLaunches_[i] += 1;
+        streamElems_[i] += args.n;
+      }
+    }
+    lastContribs_ = args.K;
+  }
   if (prof) {
     if (rc == FRG_OK) {
       std::lock_guard<std::mutex> g(profMu_);
-      profEvents_.emplace_back(a.startEvent, a.stopEvent);
+      profEvents_.push_back(ProfRecord{a.startEvent, a.stopEvent, a.n, a.K, stream, 1});
     } else {
       (void)hipEventDestroy(a.startEvent);
       (void)hipEventDestroy(a.stopEvent);
@@ -337,71 +363,94 @@ void Context::launch(const ReduceArgs& args, hipStream_t stream) {
   if (rc != FRG_OK) throw ContractFailure(rc, err);
 }
 
-// Device-resident contributions: one reduction launch per slice, slices
-// rotating over the reduce streams so that the tail of one launch overlaps
-// the head of the next (the slicing of fairring/device.cc:315-326).
-void Context::runResident(const Request& req, hipEvent_t initialEvent, hipStream_t* last) {
+// Device-resident contributions: every slice (the slicing of
+// fairring/device.cc:315-326) is reduced by one launch, or by several when it
+// is larger than the launch size; launches are dealt round-robin to the reduce
+// streams so that neighbouring launches overlap.
+void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired) {
+  // Once the producer's event has fired no stream needs to wait for it: a
+  // wait that is already satisfied still costs a barrier packet on the queue.
+  if (!*fired) {
+    if (hipEventQuery(initialEvent) == hipSuccess) {
+      *fired = true;
+    } else {
+      (void)hipGetLastError();  // "not ready" is an answer, not a failure to keep
+    }
+  }
+  if (!*fired) FRG_HIP_CHECK(hipStreamWaitEvent(stream, initialEvent, 0));
+}
+
+std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   const int64_t nSlices = numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
   const size_t nStreams = reduceStreams_.size();
+  const int64_t maxLaunchElems = maxLaunchBytes_ > 0 ? maxLaunchBytes_ / elsize : 0;
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
-  size_t lastIdx = 0;
+  const int total = static_cast<int>(ptrs.size());
+  size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
+  bool initialFired = false;
+
   for (int64_t i = 0; i < nSlices; ++i) {
-    int64_t off, len;
-    sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &off, &len);
-    const int64_t slot = (nextStagingSlot_++) % numSlots_;
-    const size_t si = static_cast<size_t>(slot) % nStreams;
-    hipStream_t s = reduceStreams_[si];
-    if (!waited[si]) {
-      // Only the first slice on a stream needs the producer's event; later
-      // ones follow it in stream order (fairring/device.cc:334-336,507-509).
-      FRG_HIP_CHECK(hipStreamWaitEvent(s, initialEvent, 0));
-      waited[si] = 1;
-    }
-    for (size_t k = 0; k < ptrs.size(); ++k) {
-      ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * elsize;
-    }
-    // More contributions than one launch takes: chain launches, carrying the
-    // partial result in `out`; the post-scale goes on the last one only.
-    const int total = static_cast<int>(ptrs.size());
-    if (total == 1 && ptrs[0] == static_cast<char*>(req.out) + off * elsize &&
-        req.scaleMode == FRG_SCALE_NONE) {
+    int64_t sliceOff, sliceLen;
+    sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &sliceOff, &sliceLen);
+    nextStagingSlot_++;  // a slice still takes its turn in the slot rotation (device.cc:482)
+    if (total == 1 && req.contribs[0] == req.out && req.scaleMode == FRG_SCALE_NONE) {
       // A lone contribution reduced in place is the identity (what the
       // reference does for one machine and one device: device.cc:523,569).
-      lastIdx = si;
       continue;
     }
-    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
-      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
-      const bool lastLaunch = k0 + kn == total;
-      ReduceArgs a;
-      a.out = static_cast<char*>(req.out) + off * elsize;
-      a.contribs = ptrs.data() + k0;
-      a.K = kn;
-      a.n = len;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = lastLaunch ? req.scaleMode : FRG_SCALE_NONE;
-      a.scale = req.scale;
-      a.carry = k0 > 0;
-      launch(a, s);
+    // Equal parts no larger than the launch size.
+    int64_t parts = 1;
+    if (maxLaunchElems > 0 && sliceLen > maxLaunchElems) {
+      parts = ceilOfRatio(sliceLen, maxLaunchElems);
     }
-    lastIdx = si;
+    const int64_t lanes = 16 / elsize;
+    const int64_t partLen = roundUpToNearestMultiple(ceilOfRatio(sliceLen, parts), lanes);
+    for (int64_t off = sliceOff; off < sliceOff + sliceLen; off += partLen) {
+      const int64_t len = off + partLen <= sliceOff + sliceLen ? partLen : sliceOff + sliceLen - off;
+      const size_t si = static_cast<size_t>(nextLaunch_++) % nStreams;
+      hipStream_t s = reduceStreams_[si];
+      if (!waited[si]) {
+        // Only the first launch on a stream needs the producer's event; later
+        // ones follow it in stream order (fairring/device.cc:334-336,507-509).
+        waitInitial(s, initialEvent, &initialFired);
+        waited[si] = 1;
+      }
+      for (size_t k = 0; k < ptrs.size(); ++k) {
+        ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * elsize;
+      }
+      // More contributions than one launch takes: chain launches, carrying the
+      // partial result in `out`; the post-scale goes on the last one only.
+      for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
+        const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
+        const bool lastLaunch = k0 + kn == total;
+        ReduceArgs a;
+        a.out = static_cast<char*>(req.out) + off * elsize;
+        a.contribs = ptrs.data() + k0;
+        a.K = kn;
+        a.n = len;
+        a.dtype = req.dtype;
+        a.op = req.op;
+        a.scale_mode = lastLaunch ? req.scaleMode : FRG_SCALE_NONE;
+        a.scale = req.scale;
+        a.carry = k0 > 0;
+        launch(a, s);
+      }
+      lastIdx = si;
+    }
   }
-  // Join: the stream of the last slice waits for the others that took part.
-  hipStream_t ls = reduceStreams_[lastIdx];
-  if (nSlices == 0) {
-    FRG_HIP_CHECK(hipStreamWaitEvent(ls, initialEvent, 0));
+  // The streams that took part, the one of the last launch at the back.
+  if (!waited[lastIdx]) {
+    waitInitial(reduceStreams_[lastIdx], initialEvent, &initialFired);
+    waited[lastIdx] = 1;
   }
+  std::vector<hipStream_t> used;
   for (size_t si = 0; si < nStreams; ++si) {
-    if (si == lastIdx || !waited[si]) continue;
-    hipEvent_t j = takeEvent();
-    FRG_HIP_CHECK(hipEventRecord(j, reduceStreams_[si]));
-    FRG_HIP_CHECK(hipStreamWaitEvent(ls, j, 0));
-    giveEvent(j);
+    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
   }
-  *last = ls;
+  used.push_back(reduceStreams_[lastIdx]);
+  return used;
 }
 
 // Contributions in pinned host memory (server-side accumulation): contribution
@@ -411,7 +460,7 @@ void Context::runResident(const Request& req, hipEvent_t initialEvent, hipStream
 // (slot rule of fairring/device.cc:543-545,587-589; cursor of :482). With four
 // or more slots, half the pool is folded per launch so that copies into the
 // other half overlap it.
-void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStream_t* last) {
+std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   // A staged slice must fit a slot as well as the slice size.
   const int64_t sliceBytes =
@@ -419,8 +468,9 @@ void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStre
   const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
   const int K = static_cast<int>(req.contribs.size());
   hipStream_t s = reduceStreams_[0];
-  FRG_HIP_CHECK(hipStreamWaitEvent(s, initialEvent, 0));
-  FRG_HIP_CHECK(hipStreamWaitEvent(copyStream_, initialEvent, 0));
+  bool initialFired = false;
+  waitInitial(s, initialEvent, &initialFired);
+  waitInitial(copyStream_, initialEvent, &initialFired);
   int64_t batch = numSlots_ / 2;
   if (batch < 1) batch = 1;
   if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
@@ -498,7 +548,7 @@ void Context::runHostStaged(const Request& req, hipEvent_t initialEvent, hipStre
     // The next slice's first copy overwrites nothing this slice still reads
     // (it targets another range of `out`), so no extra wait is needed here.
   }
-  *last = s;
+  return {s};
 }
 
 void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
@@ -507,12 +557,23 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
   std::string error;
   hipStream_t lastStream = reduceStreams_[0];
   try {
-    if (req.fromHost) {
-      runHostStaged(req, initialEvent, &lastStream);
-    } else {
-      runResident(req, initialEvent, &lastStream);
+    std::vector<hipStream_t> used =
+        req.fromHost ? runHostStaged(req, initialEvent) : runResident(req, initialEvent);
+    lastStream = used.back();
+    if (req.done != nullptr && used.size() > 1) {
+      // The callback orders consumers after ONE stream (fairring/device.cc:337-340
+      // marks the future under a guard of the last stream): join the others into it.
+      for (size_t i = 0; i + 1 < used.size(); ++i) {
+        hipEvent_t j = takeEvent();
+        FRG_HIP_CHECK(hipEventRecord(j, used[i]));
+        FRG_HIP_CHECK(hipStreamWaitEvent(lastStream, j, 0));
+        giveEvent(j);
+      }
+      used.assign(1, lastStream);
     }
-    FRG_HIP_CHECK(hipEventRecord(work->doneEvent, lastStream));
+    // Without a callback nothing needs a single stream, and the streams keep
+    // running independently of each other.
+    work->doneStreams = used;
   } catch (const ContractFailure& e) {
     status = e.code;
     error = e.what();
@@ -563,32 +624,105 @@ int Context::synchronize(std::string* err) {
   return FRG_OK;
 }
 
-void Context::setProfiling(bool on) { profiling_.store(on); }
+void Context::setProfiling(bool perLaunch) { profiling_.store(perLaunch); }
 
-int Context::kernelTimes(float* ms, int capacity, int* count, std::string* err) {
+int Context::profileMark(std::string* err) {
+  std::mutex mu;
+  std::condition_variable cv;
+  bool reached = false;
+  int status = FRG_OK;
+  queue_.enqueue([&] {
+    Mark m;
+    try {
+      for (hipStream_t s : reduceStreams_) {
+        hipEvent_t e;
+        FRG_HIP_CHECK(hipEventCreate(&e));
+        m.events.push_back(e);
+        FRG_HIP_CHECK(hipEventRecord(e, s));
+      }
+      m.launches = streamLaunches_;
+      m.elems = streamElems_;
+      std::lock_guard<std::mutex> g(profMu_);
+      marks_.push_back(std::move(m));
+    } catch (const std::exception& e) {
+      for (hipEvent_t ev : m.events) (void)hipEventDestroy(ev);
+      status = FRG_ERR_HIP;
+      *err = e.what();
+    }
+    std::lock_guard<std::mutex> g(mu);
+    reached = true;
+    cv.notify_all();
+  });
+  std::unique_lock<std::mutex> lock(mu);
+  cv.wait(lock, [&] { return reached; });
+  return status;
+}
+
+int Context::launchRecords(frg_launch_record* recs, int capacity, int* count, std::string* err) {
   const int rc = synchronize(err);
   if (rc != FRG_OK) return rc;
-  std::vector<std::pair<hipEvent_t, hipEvent_t>> evs;
+  std::vector<ProfRecord> evs;
+  std::vector<Mark> marks;
   {
     std::lock_guard<std::mutex> g(profMu_);
     evs.swap(profEvents_);
+    marks.swap(marks_);
   }
   int n = 0;
   int status = FRG_OK;
-  for (auto& p : evs) {
+  auto elapsed = [&](hipEvent_t from, hipEvent_t to) {
     float t = 0.f;
-    const hipError_t e = hipEventElapsedTime(&t, p.first, p.second);
-    if (e != hipSuccess && status == FRG_OK) {
+    const hipError_t r = hipEventElapsedTime(&t, from, to);
+    if (r != hipSuccess && status == FRG_OK) {
       status = FRG_ERR_HIP;
-      *err = std::string("hipEventElapsedTime: ") + hipGetErrorString(e);
+      *err = std::string("hipEventElapsedTime: ") + hipGetErrorString(r);
     }
-    if (n < capacity && ms) ms[n] = t;
+    return t;
+  };
+  auto emit = [&](float b, float e, int64_t numel, int contribs, int si, int64_t launches) {
+    if (n < capacity && recs) {
+      recs[n] = frg_launch_record{b, e, numel, contribs, si, static_cast<int32_t>(launches), 0};
+    }
     ++n;
-    (void)hipEventDestroy(p.first);
-    (void)hipEventDestroy(p.second);
+  };
+  // regions between consecutive marks, one record per stream that ran anything
+  for (size_t m = 0; m + 1 < marks.size(); ++m) {
+    for (size_t si = 0; si < marks[m].events.size(); ++si) {
+      const int64_t launches = marks[m + 1].launches[si] - marks[m].launches[si];
+      if (launches <= 0) continue;
+      emit(elapsed(marks[0].events[0], marks[m].events[si]),
+           elapsed(marks[0].events[0], marks[m + 1].events[si]),
+           marks[m + 1].elems[si] - marks[m].elems[si], lastContribs_, static_cast<int>(si),
+           launches);
+    }
+  }
+  // per-launch records
+  for (auto& p : evs) {
+    int si = 0;
+    for (size_t i = 0; i < reduceStreams_.size(); ++i) {
+      if (reduceStreams_[i] == p.stream) si = static_cast<int>(i);
+    }
+    emit(elapsed(evs.front().begin, p.begin), elapsed(evs.front().begin, p.end), p.numel,
+         p.numContribs, si, 1);
+  }
+  for (auto& p : evs) {
+    (void)hipEventDestroy(p.begin);
+    (void)hipEventDestroy(p.end);
+  }
+  for (auto& m : marks) {
+    for (hipEvent_t e : m.events) (void)hipEventDestroy(e);
   }
   if (count) *count = n;
   return status;
+}
+
+int Context::kernelTimes(float* ms, int capacity, int* count, std::string* err) {
+  std::vector<frg_launch_record> recs(static_cast<size_t>(capacity > 0 ? capacity : 0));
+  int n = 0;
+  const int rc = launchRecords(recs.data(), capacity, &n, err);
+  for (int i = 0; i < n && i < capacity && ms; ++i) ms[i] = recs[i].end_ms - recs[i].begin_ms;
+  if (count) *count = n;
+  return rc;
 }
 
 }  // namespace frg

@@ -41,7 +41,12 @@ struct Work {
   bool enqueued = false;  // the command thread is done with it
   int status = FRG_OK;
   std::string error;
-  hipEvent_t doneEvent = nullptr;  // recorded on lastStream after the last slice
+  // The streams the operation's work ended on. No event is recorded per
+  // operation (an event record is a packet on the stream, between two launches
+  // that would otherwise run back to back): waiting is done against the
+  // streams themselves, which are in order, so it covers the operation and
+  // whatever was enqueued on them up to the moment of the wait.
+  std::vector<hipStream_t> doneStreams;
   hipStream_t lastStream = nullptr;
   int device = 0;
   std::atomic<int> refs{1};
@@ -80,8 +85,10 @@ class Context {
   int submit(Request req, Work** work, std::string* err);
 
   int synchronize(std::string* err);
-  void setProfiling(bool on);
+  void setProfiling(bool perLaunch);
+  int profileMark(std::string* err);
   int kernelTimes(float* ms, int capacity, int* count, std::string* err);
+  int launchRecords(frg_launch_record* recs, int capacity, int* count, std::string* err);
 
   static void releaseWork(Work* w);
   // Host blocks until the operation is enqueued and its GPU work is done.
@@ -94,8 +101,12 @@ class Context {
   Context() = default;
 
   void run(const Request& req, hipEvent_t initialEvent, Work* work);
-  void runResident(const Request& req, hipEvent_t initialEvent, hipStream_t* last);
-  void runHostStaged(const Request& req, hipEvent_t initialEvent, hipStream_t* last);
+  // Both return the streams the operation's work ended on, the last one used
+  // at the back.
+  std::vector<hipStream_t> runResident(const Request& req, hipEvent_t initialEvent);
+  std::vector<hipStream_t> runHostStaged(const Request& req, hipEvent_t initialEvent);
+  // Makes `stream` wait for `initialEvent` unless that event has already fired.
+  void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
   void launch(const struct ReduceArgs& args, hipStream_t stream);
   hipEvent_t takeEvent();
   void giveEvent(hipEvent_t e);
@@ -104,6 +115,8 @@ class Context {
   Layout layout_;
   int64_t numSlots_ = 0;
   int64_t slotBytes_ = 0;
+  int64_t maxLaunchBytes_ = 0;   // per contribution and launch; 0 = whole slice
+  int64_t nextLaunch_ = 0;       // deals launches to the reduce streams
 
   std::vector<hipStream_t> reduceStreams_;
   hipStream_t copyStream_ = nullptr;
@@ -118,9 +131,27 @@ class Context {
   std::mutex eventMu_;
   std::vector<hipEvent_t> freeEvents_;
 
-  std::atomic<bool> profiling_{false};
+  std::atomic<bool> profiling_{false};  // per-launch dispatch timestamps
   std::mutex profMu_;
-  std::vector<std::pair<hipEvent_t, hipEvent_t>> profEvents_;
+  struct ProfRecord {
+    hipEvent_t begin;
+    hipEvent_t end;
+    int64_t numel;
+    int numContribs;
+    hipStream_t stream;
+    int launches;
+  };
+  std::vector<ProfRecord> profEvents_;
+  // marks: one timing event per reduce stream plus the running totals then
+  struct Mark {
+    std::vector<hipEvent_t> events;
+    std::vector<int64_t> launches;
+    std::vector<int64_t> elems;
+  };
+  std::vector<Mark> marks_;
+  std::vector<int64_t> streamLaunches_;  // running totals per reduce stream (command thread)
+  std::vector<int64_t> streamElems_;
+  int lastContribs_ = 0;
 
   CommandQueue queue_;
   std::thread thread_;

@@ -135,10 +135,11 @@ class Work:
 class DeviceFairring:
     def __init__(self, device=0, max_memory_allocated_in_bytes=50 * MiB,
                  max_padding_allocated_in_bytes=MiB, min_parallelism=16,
-                 slice_size_in_bytes=0, num_machines=1, num_reduce_streams=0):
+                 slice_size_in_bytes=0, num_machines=1, num_reduce_streams=0,
+                 max_launch_bytes=0):
         o = _capi.Options(max_memory_allocated_in_bytes, max_padding_allocated_in_bytes,
                           min_parallelism, slice_size_in_bytes, num_machines,
-                          num_reduce_streams, 0)
+                          num_reduce_streams, 0, max_launch_bytes)
         h = ctypes.c_void_p()
         self._h = None
         _capi.check(_capi.lib().frg_create(int(device), ctypes.byref(o), ctypes.byref(h)))
@@ -191,17 +192,60 @@ class DeviceFairring:
         return self._submit(out, host_contribs, op, scale_mode, scale, stream, host=True,
                             carry=carry)
 
+    def prepare(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+        """Validate and marshal an allreduce once; the returned callable submits
+        it with a single foreign call (for callers that repeat the same
+        operation, e.g. one per DDP bucket per step). The callable returns a
+        Work; the tensors stay referenced by it."""
+        import torch
+        _check_dense(out, "output")
+        for c in contribs:
+            _check_dense(c, "contribution")
+            if c.numel() != out.numel() or c.dtype != out.dtype:
+                raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+        stream = torch.cuda.current_stream(out.device) if stream is None else stream
+        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        L = _capi.lib()
+        fn = L.frg_allreduce
+        args = (self._h, ctypes.c_void_p(out.data_ptr()), tab, len(contribs),
+                ctypes.c_int64(out.numel()), _dtype_code(out), op, scale_mode,
+                ctypes.c_float(scale), ctypes.c_void_p(stream.cuda_stream), _capi.DONE_FN(), None)
+        keep = (out, list(contribs), tab)
+
+        def submit():
+            wh = ctypes.c_void_p()
+            rc = fn(*args, ctypes.byref(wh))
+            if rc != _capi.OK:
+                _capi.check(rc)
+            return Work(wh, keep)
+
+        return submit
+
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))
 
-    def set_profiling(self, on):
-        _capi.check(_capi.lib().frg_set_profiling(self._h, 1 if on else 0))
+    def set_profiling(self, per_launch):
+        """Per-launch dispatch timestamps on or off."""
+        _capi.check(_capi.lib().frg_set_profiling(self._h, 1 if per_launch else 0))
+
+    def profile_mark(self):
+        """One timing event on every reduce stream, in submission order; two
+        marks bracket a region that launch_records() reports per stream."""
+        _capi.check(_capi.lib().frg_profile_mark(self._h))
 
     def kernel_times_ms(self, capacity=1 << 16):
         buf = (ctypes.c_float * capacity)()
         n = ctypes.c_int()
         _capi.check(_capi.lib().frg_kernel_times(self._h, buf, capacity, ctypes.byref(n)))
         return list(buf[:min(n.value, capacity)])
+
+    def launch_records(self, capacity=1 << 16):
+        """(begin_ms, end_ms, numel, K, stream_index, launches) of every record."""
+        buf = (_capi.LaunchRecord * capacity)()
+        n = ctypes.c_int()
+        _capi.check(_capi.lib().frg_launch_records(self._h, buf, capacity, ctypes.byref(n)))
+        return [(r.begin_ms, r.end_ms, r.numel, r.num_contributions, r.stream_index, r.launches)
+                for r in buf[:min(n.value, capacity)]]
 
     def close(self):
         h, self._h = self._h, None

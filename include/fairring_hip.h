@@ -101,8 +101,13 @@ typedef struct frg_options {
   int64_t min_parallelism;                /* FAIRRING_PARALLELISM, default 16 (__init__.py:31-34) */
   int64_t slice_size_in_bytes;            /* FAIRRING_SLICE_SIZE; 0 = derive with computeLayout */
   int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
-  int32_t num_reduce_streams;             /* 0 = default (min(slots, 2)) */
+  int32_t num_reduce_streams;             /* 0 = default (2) */
   int32_t reserved;
+  int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
+                                             launch covers; a slice larger than this is reduced by
+                                             several launches dealt round-robin to the reduce
+                                             streams. 0 = default (12.5 MiB), < 0 = one launch per
+                                             slice */
 } frg_options;
 
 /* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,
@@ -180,14 +185,48 @@ FRG_API int frg_synchronize(frg_ctx* ctx);
 
 /* ---- measurement hooks -------------------------------------------------- */
 
-/* When on, every reduction launch is bracketed by timing events on its own
- * stream; frg_kernel_times() returns the durations (milliseconds) recorded
- * since the last call, after synchronising. */
-FRG_API int frg_set_profiling(frg_ctx* ctx, int on);
+/* Timing with HIP events on the streams the reduction kernel is launched on.
+ *
+ * frg_profile_mark: goes through the command queue like an operation and
+ * records one timing event on every reduce stream, at that point of the
+ * stream. Two consecutive marks bracket a region: for each reduce stream that
+ * launched anything in between, frg_launch_records yields one record spanning
+ * the two events, with the launches and elements that stream ran in the
+ * region. Launches on a stream run back to back, so span / launches is the
+ * average launch duration on that stream; the cost is one event record per
+ * stream and mark, nothing per launch.
+ *
+ * frg_set_profiling(ctx, 1): instead, every launch gets the begin and end
+ * timestamps of its own dispatch (one record per launch). Exact per launch,
+ * but the per-dispatch bookkeeping slows a two-stream pipeline by several
+ * percent. 0 switches it off. */
+FRG_API int frg_profile_mark(frg_ctx* ctx);
+FRG_API int frg_set_profiling(frg_ctx* ctx, int per_launch);
+
+/* Durations in milliseconds of the records collected since the last call
+ * (after synchronising); consumes them. */
 FRG_API int frg_kernel_times(frg_ctx* ctx, float* ms, int capacity, int* count);
 
-/* Launch-shape knobs of the reduction kernel (0 keeps the built-in default). */
-FRG_API int frg_set_tuning(int blocks_per_cu, int xcd_remap);
+/* The same records with their position in time: begin and end in milliseconds
+ * after the first record began, the elements and launches they cover, the
+ * number of contributions and the index of the reduce stream. Records on
+ * different streams overlap; the union of their intervals is the time during
+ * which the kernel was running at all. Consumes the records. */
+typedef struct frg_launch_record {
+  float begin_ms;
+  float end_ms;
+  int64_t numel;
+  int32_t num_contributions;
+  int32_t stream_index;
+  int32_t launches;
+  int32_t reserved;
+} frg_launch_record;
+FRG_API int frg_launch_records(frg_ctx* ctx, frg_launch_record* records, int capacity,
+                               int* count);
+
+/* Launch-shape knob of the reduction kernel: blocks of the persistent grid per
+ * CU (0 keeps the built-in default, which depends on the loads per lane). */
+FRG_API int frg_set_tuning(int blocks_per_cu);
 
 /* Message of the last failure on the calling thread (or of the failed work). */
 FRG_API const char* frg_last_error(void);
