@@ -460,8 +460,9 @@ def main():
     # HBM bytes per launch as measured with rocprofv3 --pmc (two counter runs,
     # scaled by a copy of known size); the summary that holds the figure names
     # the commands that produced it.
-    if args.workload == "c2" and args.slice_bytes == 25 * MiB and not args.k:
-        tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_25MiB_hbm_traffic.md")
+    if (args.workload == "c2" and args.slice_bytes == 25 * MiB and not args.k
+            and not args.launch_bytes):
+        tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_c2_hbm_traffic.md")
         if os.path.exists(tpath):
             import re
             m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", open(tpath).read())
