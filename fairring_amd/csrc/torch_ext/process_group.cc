@@ -41,8 +41,8 @@ int dtypeCode(const at::Tensor& t) {
 // What travels through the C ABI's completion callback.
 struct Pending {
   c10::intrusive_ptr<c10::ivalue::Future> future;
-  at::Tensor tensor;               // the caller's tensor: result and keep-alive
-  std::vector<at::Tensor> peers;   // keep-alive
+  at::Tensor tensor;               // the result tensor (the caller's, reduced in place)
+  std::vector<at::Tensor> inputs;  // keep-alive: own input, peers' contributions
   c10::DeviceIndex device;
 };
 
@@ -187,22 +187,81 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduce(
   FRG_CHECK(t.is_cuda());
   FRG_CHECK(t.is_non_overlapping_and_dense());
   t = viewAsFlat(t);
+  return reduceCommon(c10d::OpType::ALLREDUCE, opts.reduceOp, t, t, /*chunkOffset=*/0,
+                      /*peerNumel=*/t.numel(), {});
+}
 
+// fairring/process_group.cc:330-364: input holds `size` chunks, chunk r goes to
+// rank r; this rank's output is the reduction of everyone's chunk `rank`.
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::_reduce_scatter_base(
+    at::Tensor& outputBuffer, at::Tensor& inputBuffer, const c10d::ReduceScatterOptions& opts) {
+  FRG_CHECK(inputBuffer.layout() == at::kStrided);
+  FRG_CHECK(inputBuffer.is_cuda());
+  FRG_CHECK(inputBuffer.is_non_overlapping_and_dense());
+  FRG_CHECK(outputBuffer.layout() == at::kStrided);
+  FRG_CHECK(outputBuffer.is_cuda());
+  FRG_CHECK(outputBuffer.is_non_overlapping_and_dense());
+  FRG_CHECK(inputBuffer.device() == outputBuffer.device());
+  FRG_CHECK(inputBuffer.scalar_type() == outputBuffer.scalar_type());
+  FRG_CHECK(inputBuffer.numel() == outputBuffer.numel() * getSize());
+  at::Tensor in = viewAsFlat(inputBuffer);
+  at::Tensor out = viewAsFlat(outputBuffer);
+  return reduceCommon(c10d::OpType::_REDUCE_SCATTER_BASE, opts.reduceOp, in, out,
+                      /*chunkOffset=*/out.numel() * getRank(), /*peerNumel=*/in.numel(), {});
+}
+
+// fairring/process_group.cc:283-328: the list form; inputTensors[0][r] is the
+// chunk this rank contributes to rank r.
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduce_scatter(
+    std::vector<at::Tensor>& outputTensors, std::vector<std::vector<at::Tensor>>& inputTensors,
+    const c10d::ReduceScatterOptions& opts) {
+  FRG_CHECK(inputTensors.size() == outputTensors.size());
+  FRG_CHECK(outputTensors.size() == 1);  // one device per process here
+  FRG_CHECK(static_cast<int64_t>(inputTensors[0].size()) == getSize());
+  at::Tensor& o = outputTensors[0];
+  FRG_CHECK(o.layout() == at::kStrided);
+  FRG_CHECK(o.is_cuda());
+  FRG_CHECK(o.is_non_overlapping_and_dense());
+  std::vector<at::Tensor> keep;
+  for (const at::Tensor& t : inputTensors[0]) {
+    FRG_CHECK(t.layout() == at::kStrided);
+    FRG_CHECK(t.is_cuda());
+    FRG_CHECK(t.is_non_overlapping_and_dense());
+    FRG_CHECK(t.device() == o.device());
+    FRG_CHECK(t.scalar_type() == o.scalar_type());
+    FRG_CHECK(t.numel() == o.numel());
+    keep.push_back(t);
+  }
+  at::Tensor own = viewAsFlat(inputTensors[0][getRank()]);
+  at::Tensor out = viewAsFlat(o);
+  return reduceCommon(c10d::OpType::REDUCE_SCATTER, opts.reduceOp, own, out, /*chunkOffset=*/0,
+                      /*peerNumel=*/out.numel() * getSize(), std::move(keep));
+}
+
+// The shared body: `out` (n elements) = reduction in rank order of this rank's
+// own n elements (own[ownOffset ...]) and, from every simulated peer, the n
+// elements at offset rank*n of its flat input when the peer hands in a whole
+// input (peerNumel == size*n), or its n elements when it hands in just that.
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
+    c10d::OpType opType, const c10d::ReduceOp& reduceOp, at::Tensor own, at::Tensor out,
+    int64_t chunkOffset, int64_t peerNumel, std::vector<at::Tensor> keepAlive) {
   // fairring/machine.cc:181: SUM and MAX only
-  const c10d::ReduceOp::RedOpType op = opts.reduceOp.op_;
+  const c10d::ReduceOp::RedOpType op = reduceOp.op_;
   FRG_CHECK(op == c10d::ReduceOp::SUM || op == c10d::ReduceOp::MAX);
   // fairring/device.cc:316
-  FRG_CHECK(8 % t.element_size() == 0);
-  const int dtype = dtypeCode(t);
-  TORCH_CHECK(dtype >= 0, "fairring: unsupported dtype ", t.scalar_type(),
-              " (float32 and bfloat16 are implemented)");
+  FRG_CHECK(8 % out.element_size() == 0);
+  const int dtype = dtypeCode(out);
+  TORCH_CHECK(dtype >= 0, "fairring: unsupported dtype ", out.scalar_type());
 
   std::lock_guard<std::mutex> g(mutex_);
-  const c10::DeviceIndex device = t.device().index();
+  const c10::DeviceIndex device = out.device().index();
   frg_ctx* ctx = contextFor(device);
 
   const int size = getSize();
   const int rank = getRank();
+  const int64_t n = out.numel();
+  const int64_t elsize = out.element_size();
+  std::vector<int64_t> peerOffsets;
   std::vector<at::Tensor> peers = peers_;
   TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
               "fairring: this build runs on one GPU without a transport; a group of size ",
@@ -212,23 +271,31 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduce(
     at::Tensor& p = peers[i];
     TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense(),
                 "fairring: peer contribution must be dense");
-    TORCH_CHECK(p.scalar_type() == t.scalar_type() && p.numel() == t.numel(),
-                "fairring: peer contribution must match the tensor's dtype and size");
+    TORCH_CHECK(p.scalar_type() == out.scalar_type() &&
+                    (p.numel() == n || p.numel() == peerNumel),
+                "fairring: peer contribution must match the operation's dtype and hold ", n,
+                " or ", peerNumel, " elements, got ", p.numel());
+    // a whole flat input: the chunk meant for this rank; otherwise just that chunk
+    peerOffsets.push_back(p.numel() == n ? 0 : n * rank);
     p = viewAsFlat(p);
     if (i == 0) fromHost = !p.is_cuda();
     TORCH_CHECK(fromHost == !p.is_cuda(), "fairring: peers must be all on the GPU or all pinned");
     if (fromHost) {
       TORCH_CHECK(p.is_pinned(), "fairring: host-side peer contributions must be pinned");
     } else {
-      TORCH_CHECK(p.device() == t.device(), "fairring: peer contribution on another device");
+      TORCH_CHECK(p.device() == out.device(), "fairring: peer contribution on another device");
     }
   }
 
-  // Contribution table in rank order, this rank's own tensor at its index.
+  // Contribution table in rank order, this rank's own chunk at its index.
+  const char* ownPtr = static_cast<const char*>(own.data_ptr()) + chunkOffset * elsize;
   std::vector<const void*> table;
   table.reserve(size);
   for (int r = 0, pi = 0; r < size; ++r) {
-    table.push_back(r == rank ? t.data_ptr() : peers[pi++].data_ptr());
+    table.push_back(r == rank ? static_cast<const void*>(ownPtr)
+                              : static_cast<const char*>(peers[pi].data_ptr()) +
+                                    peerOffsets[pi] * elsize);
+    if (r != rank) ++pi;
   }
 
   // Tell the caching allocator which streams will touch these buffers
@@ -239,46 +306,51 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduce(
   for (int i = 0; i < nStreams && i < 16; ++i) {
     c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
         static_cast<hipStream_t>(streams[i]), device);
-    t.record_stream(s);
+    out.record_stream(s);
+    own.record_stream(s);
     if (!fromHost) {
       for (at::Tensor& p : peers) p.record_stream(s);
     }
   }
 
   auto future = c10::make_intrusive<c10::ivalue::Future>(
-      c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
+      c10::ListType::ofTensors(), std::vector<c10::Device>{out.device()});
 
   const bool divide = fusedDivide_ && op == c10d::ReduceOp::SUM && size > 1;
   const bool pow2 = (size & (size - 1)) == 0;
   const int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
   const float scale = !divide ? 1.0f : (pow2 ? 1.0f / static_cast<float>(size)
                                               : static_cast<float>(size));
+  const int frgOp = op == c10d::ReduceOp::SUM ? FRG_SUM : FRG_MAX;
+
+  if (fromHost) {
+    // Server-side accumulation: this rank's own shard sits in `out`, the
+    // peers' are staged from pinned memory and folded into it in rank order.
+    // The fixed order needs the resident contribution to be first.
+    TORCH_CHECK(rank == 0, "fairring: pinned peer contributions are folded after the resident "
+                           "tensor, which must therefore be rank 0 (got rank ", rank, ")");
+    if (out.data_ptr() != static_cast<const void*>(ownPtr)) {
+      out.copy_(own.narrow(0, chunkOffset, n), /*non_blocking=*/true);  // on the current stream
+    }
+  }
 
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
-  auto* pending = new Pending{future, t, std::move(peers), device};
+  keepAlive.push_back(own);
+  for (at::Tensor& p : peers) keepAlive.push_back(p);
+  auto* pending = new Pending{future, out, std::move(keepAlive), device};
   int rc;
-  const int frgOp = op == c10d::ReduceOp::SUM ? FRG_SUM : FRG_MAX;
   if (fromHost) {
-    // Server-side accumulation: this rank's own shard is already in the
-    // tensor, the peers' are staged from pinned memory and folded into it in
-    // rank order. The fixed order needs the resident contribution to be first.
-    if (rank != 0) {
-      delete pending;
-      TORCH_CHECK(false, "fairring: pinned peer contributions are folded after the resident "
-                         "tensor, which must therefore be rank 0 (got rank ", rank, ")");
-    }
-    rc = frg_allreduce_host(ctx, t.data_ptr(), table.data() + 1, size - 1, t.numel(), dtype,
-                            frgOp, scaleMode, scale, /*carry=*/1, current, &onDone, pending,
-                            nullptr);
+    rc = frg_allreduce_host(ctx, out.data_ptr(), table.data() + 1, size - 1, n, dtype, frgOp,
+                            scaleMode, scale, /*carry=*/1, current, &onDone, pending, nullptr);
   } else {
-    rc = frg_allreduce(ctx, t.data_ptr(), table.data(), size, t.numel(), dtype, frgOp,
-                       scaleMode, scale, current, &onDone, pending, nullptr);
+    rc = frg_allreduce(ctx, out.data_ptr(), table.data(), size, n, dtype, frgOp, scaleMode,
+                       scale, current, &onDone, pending, nullptr);
   }
   if (rc != FRG_OK) {
     delete pending;
     TORCH_CHECK(false, "fairring: ", frg_last_error());
   }
-  return c10::make_intrusive<WorkFairring>(c10d::OpType::ALLREDUCE, std::move(future));
+  return c10::make_intrusive<WorkFairring>(opType, std::move(future));
 }
 
 }  // namespace fairring

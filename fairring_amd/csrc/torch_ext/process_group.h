@@ -79,10 +79,24 @@ class ProcessGroupFairring : public c10d::Backend {
       std::vector<at::Tensor>& data,
       const c10d::AllreduceOptions& opts = c10d::AllreduceOptions()) override;
 
+  // fairring/process_group.cc:283-364: the server-side sum with a separate
+  // output. One GPU: only this rank's output chunk is produced.
+  c10::intrusive_ptr<c10d::Work> reduce_scatter(
+      std::vector<at::Tensor>& outputTensors,
+      std::vector<std::vector<at::Tensor>>& inputTensors,
+      const c10d::ReduceScatterOptions& opts = c10d::ReduceScatterOptions()) override;
+
+  c10::intrusive_ptr<c10d::Work> _reduce_scatter_base(
+      at::Tensor& outputBuffer, at::Tensor& inputBuffer,
+      const c10d::ReduceScatterOptions& opts = c10d::ReduceScatterOptions()) override;
+
   // Not in the reference. The contributions of the other size-1 ranks, in rank
   // order with this rank left out; GPU tensors on the caller's device or
-  // pinned CPU tensors (then they are staged through the pool). Used by every
-  // allreduce until replaced; an empty list clears them.
+  // pinned CPU tensors (then they are staged through the pool). For allreduce
+  // each has the tensor's size; for the reduce-scatter forms each is either a
+  // peer's whole flat input (size * n elements, its chunk for this rank is
+  // taken) or just the n elements it would send here. Used by every operation
+  // until replaced; an empty list clears them.
   void setSimulatedPeerContributions(std::vector<at::Tensor> peers);
 
   // Not in the reference. When on, SUM results are divided by the group size
@@ -94,6 +108,11 @@ class ProcessGroupFairring : public c10d::Backend {
 
  private:
   frg_ctx* contextFor(c10::DeviceIndex device);
+  c10::intrusive_ptr<c10d::Work> reduceCommon(c10d::OpType opType,
+                                              const c10d::ReduceOp& reduceOp, at::Tensor own,
+                                              at::Tensor out, int64_t chunkOffset,
+                                              int64_t peerNumel,
+                                              std::vector<at::Tensor> keepAlive);
 
   c10::intrusive_ptr<c10d::Store> store_;
   c10::intrusive_ptr<OptionsFairring> options_;

@@ -182,3 +182,53 @@ pg.allreduce([torch.zeros(8, device="cuda:0")[::2]])
 print("survived")
 """], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode != 0 and "is_non_overlapping_and_dense" in r.stderr
+
+
+@pytest.mark.parametrize("rank,size", [(0, 2), (3, 8), (6, 7)])
+def test_reduce_scatter_base_and_list_form(rank, size):
+    # server-side sum with a separate output (fairring/process_group.cc:283-364)
+    print("[case] pg reduce_scatter", rank, size, flush=True)
+    n = 70_003
+    rng = np.random.default_rng(rank * 10 + size)
+    x = (rng.standard_normal((size, size * n)) * 0.01).astype(np.float32)   # x[r] = rank r's input
+    want = oracle.sum_f32([x[r][rank * n:(rank + 1) * n] for r in range(size)])
+    pg = make_pg(rank, size)
+    full_in = torch.from_numpy(x[rank].copy()).to(DEV)
+    out = torch.empty(n, device=DEV)
+    # peers hand in their whole flat inputs
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(x[r].copy()).to(DEV) for r in range(size) if r != rank])
+    w = pg._reduce_scatter_base(out, full_in)
+    assert w.wait() is True
+    torch.cuda.synchronize()
+    assert_bits_equal(out.cpu().numpy(), want)
+    assert_bits_equal(full_in.cpu().numpy(), x[rank])          # the input is left alone
+    # list form, peers hand in just the chunk meant for this rank
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(x[r][rank * n:(rank + 1) * n].copy()).to(DEV)
+         for r in range(size) if r != rank])
+    out2 = torch.empty(n, device=DEV)
+    chunks = list(full_in.view(size, n).unbind(0))
+    pg.reduce_scatter([out2], [chunks]).wait()
+    torch.cuda.synchronize()
+    assert_bits_equal(out2.cpu().numpy(), want)
+
+
+def test_reduce_scatter_tensor_through_torch_distributed_world_one():
+    print("[case] reduce_scatter_tensor world 1", flush=True)
+    code = """
+import torch, torch.distributed as dist
+import fairring
+dist.init_process_group("fairring", store=dist.HashStore(), rank=0, world_size=1)
+x = torch.arange(1000, dtype=torch.float32, device="cuda:0")
+out = torch.empty(1000, device="cuda:0")
+dist.reduce_scatter_tensor(out, x)
+torch.cuda.synchronize()
+assert bool((out == x).all())
+print("copy ok")
+dist.destroy_process_group()
+"""
+    r = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, PYTHONPATH=ROOT),
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "copy ok" in r.stdout
