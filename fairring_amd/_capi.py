@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libfairring_hip.so")
 
 OK, ERR_INVALID, ERR_HIP, ERR_LAYOUT, ERR_UNSUPPORTED, ERR_NOT_READY = range(6)
-F32, BF16 = 0, 1
+F32, BF16, F16, F64, I32, I64, U8, I8 = range(8)
 SUM, MAX = 0, 1
 SCALE_NONE, SCALE_MUL, SCALE_DIV = 0, 1, 2
 

@@ -10,12 +10,16 @@ namespace frg {
 
 constexpr int kMaxContribsPerLaunch = 64;
 
+// Bytes per element of an FRG_* dtype code, 0 for an unknown code.
+int64_t elementSize(int dtype);
+bool isFloating(int dtype);
+
 struct ReduceArgs {
   void* out = nullptr;
   const void* const* contribs = nullptr;  // host array of K device pointers
   int K = 0;
   int64_t n = 0;  // elements
-  int dtype = 0;  // FRG_F32 / FRG_BF16
+  int dtype = 0;  // an FRG_* dtype code
   int op = 0;     // FRG_SUM / FRG_MAX
   int scale_mode = 0;
   float scale = 1.0f;

@@ -96,15 +96,22 @@ __device__ __forceinline__ unsigned int f32ToBf16Rne(float f) {
 }
 
 // ---- storage traits: how a "vector" of elements is loaded and unpacked ------
+//
+// elem_t: storage element; vec_t: what one lane loads (16 bytes in the vector
+// variants, one element in the scalar ones); acc_t: the type the fold runs in
+// (fp32 for fp32/bf16/fp16 as ATen accumulates them, fp64 for fp64, the
+// element's own width with wrap-around for integers).
 
 struct F32Vec {
   using elem_t = float;
   using vec_t = f32x4;
+  using acc_t = float;
   static constexpr int kLanes = 4;
-  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+  static constexpr bool kFloating = true;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) {
     f[0] = v[0]; f[1] = v[1]; f[2] = v[2]; f[3] = v[3];
   }
-  __device__ static vec_t pack(const float (&f)[kLanes]) {
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) {
     vec_t v;
     v[0] = f[0]; v[1] = f[1]; v[2] = f[2]; v[3] = f[3];
     return v;
@@ -114,23 +121,27 @@ struct F32Vec {
 struct F32Scalar {
   using elem_t = float;
   using vec_t = float;
+  using acc_t = float;
   static constexpr int kLanes = 1;
-  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) { f[0] = v; }
-  __device__ static vec_t pack(const float (&f)[kLanes]) { return f[0]; }
+  static constexpr bool kFloating = true;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) { f[0] = v; }
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) { return f[0]; }
 };
 
 struct Bf16Vec {  // 8 bf16 in 16 bytes
   using elem_t = unsigned short;
   using vec_t = u32x4;
+  using acc_t = float;
   static constexpr int kLanes = 8;
-  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+  static constexpr bool kFloating = true;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       f[2 * j] = bitsToFloat(v[j] << 16);
       f[2 * j + 1] = bitsToFloat(v[j] & 0xFFFF0000u);
     }
   }
-  __device__ static vec_t pack(const float (&f)[kLanes]) {
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) {
     vec_t v;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -143,21 +154,82 @@ struct Bf16Vec {  // 8 bf16 in 16 bytes
 struct Bf16Scalar {
   using elem_t = unsigned short;
   using vec_t = unsigned short;
+  using acc_t = float;
   static constexpr int kLanes = 1;
-  __device__ static void unpack(const vec_t& v, float (&f)[kLanes]) {
+  static constexpr bool kFloating = true;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) {
     f[0] = bitsToFloat(static_cast<unsigned int>(v) << 16);
   }
-  __device__ static vec_t pack(const float (&f)[kLanes]) {
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) {
     return static_cast<unsigned short>(f32ToBf16Rne(f[0]));
   }
 };
 
-template <int OP>
-__device__ __forceinline__ float combine(float a, float b) {
+// Element-wise traits for types whose vector is an ext_vector of the element:
+// convert up on unpack, down (round to nearest even for fp16, wrap-around for
+// integers) on pack.
+template <typename E, typename A, int LANES, bool FLOATING>
+struct PlainVec {
+  using elem_t = E;
+  typedef E vec_t __attribute__((ext_vector_type(LANES)));
+  using acc_t = A;
+  static constexpr int kLanes = LANES;
+  static constexpr bool kFloating = FLOATING;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) {
+#pragma unroll
+    for (int j = 0; j < LANES; ++j) f[j] = static_cast<A>(v[j]);
+  }
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) {
+    vec_t v;
+#pragma unroll
+    for (int j = 0; j < LANES; ++j) v[j] = static_cast<E>(f[j]);
+    return v;
+  }
+};
+
+template <typename E, typename A, bool FLOATING>
+struct PlainScalar {
+  using elem_t = E;
+  using vec_t = E;
+  using acc_t = A;
+  static constexpr int kLanes = 1;
+  static constexpr bool kFloating = FLOATING;
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) { f[0] = static_cast<A>(v); }
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) { return static_cast<E>(f[0]); }
+};
+
+using F16Vec = PlainVec<_Float16, float, 8, true>;
+using F16Scalar = PlainScalar<_Float16, float, true>;
+using F64Vec = PlainVec<double, double, 2, true>;
+using F64Scalar = PlainScalar<double, double, true>;
+// Integers fold in an unsigned type of the element's width or wider (sums wrap
+// like two's complement); the maximum compares in the element's own signedness.
+using I32Vec = PlainVec<int, int, 4, false>;
+using I32Scalar = PlainScalar<int, int, false>;
+using I64Vec = PlainVec<long long, long long, 2, false>;
+using I64Scalar = PlainScalar<long long, long long, false>;
+using U8Vec = PlainVec<unsigned char, unsigned int, 16, false>;
+using U8Scalar = PlainScalar<unsigned char, unsigned int, false>;
+using I8Vec = PlainVec<signed char, int, 16, false>;
+using I8Scalar = PlainScalar<signed char, int, false>;
+
+__device__ __forceinline__ int addWrap(int a, int b) {
+  return static_cast<int>(static_cast<unsigned int>(a) + static_cast<unsigned int>(b));
+}
+__device__ __forceinline__ long long addWrap(long long a, long long b) {
+  return static_cast<long long>(static_cast<unsigned long long>(a) +
+                                static_cast<unsigned long long>(b));
+}
+__device__ __forceinline__ unsigned int addWrap(unsigned int a, unsigned int b) { return a + b; }
+__device__ __forceinline__ float addWrap(float a, float b) { return a + b; }
+__device__ __forceinline__ double addWrap(double a, double b) { return a + b; }
+
+template <int OP, typename A>
+__device__ __forceinline__ A combine(A a, A b) {
   if (OP == FRG_SUM) {
-    return a + b;
+    return addWrap(a, b);
   } else {
-    // maximum with NaN propagation, as at::amax
+    // maximum with NaN propagation, as at::amax (the NaN tests fold away for integers)
     return (a != a) ? a : ((b != b) ? b : (a > b ? a : b));
   }
 }
@@ -172,7 +244,7 @@ struct Ptrs {
 // Loads N contributions [k0, k0+N) at (base + lane), then folds them into acc
 // in index order. `first` makes contribution k0 initialise acc instead.
 template <typename TR, int OP, int N, typename PT>
-__device__ __forceinline__ void foldChunk(float (&acc)[TR::kLanes], const PT& in,
+__device__ __forceinline__ void foldChunk(typename TR::acc_t (&acc)[TR::kLanes], const PT& in,
                                           int k0, int64_t elemBase,
                                           unsigned int laneBytes, bool first) {
   using vec_t = typename TR::vec_t;
@@ -187,7 +259,7 @@ __device__ __forceinline__ void foldChunk(float (&acc)[TR::kLanes], const PT& in
   }
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    float f[TR::kLanes];
+    typename TR::acc_t f[TR::kLanes];
     TR::unpack(v[k], f);
     if (k == 0 && first) {
 #pragma unroll
@@ -208,7 +280,7 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
   using vec_t = typename TR::vec_t;
   const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
   vec_t* o = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(out + elemBase) + laneBytes);
-  float acc[TR::kLanes];
+  typename TR::acc_t acc[TR::kLanes];
   bool first = true;
   vec_t c;
   if (carry) c = *o;  // issued before the contribution loads, consumed first
@@ -243,13 +315,17 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
       foldChunk<TR, OP, 1>(acc, in, k, elemBase, laneBytes, first);
     }
   }
-  if (OP == FRG_SUM) {
-    if (scaleMode == FRG_SCALE_MUL) {
+  if constexpr (TR::kFloating) {
+    if (OP == FRG_SUM) {
+      // in the accumulator's precision: fp32, or fp64 for fp64 data
+      const typename TR::acc_t sc = static_cast<typename TR::acc_t>(scale);
+      if (scaleMode == FRG_SCALE_MUL) {
 #pragma unroll
-      for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] * scale;
-    } else if (scaleMode == FRG_SCALE_DIV) {
+        for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] * sc;
+      } else if (scaleMode == FRG_SCALE_DIV) {
 #pragma unroll
-      for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] / scale;
+        for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] / sc;
+      }
     }
   }
   stStream(TR::pack(acc), o);
@@ -366,25 +442,62 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   return hipGetLastError();
 }
 
-template <typename TRV, typename TRS>
+// FAST: also instantiate the compile-time-K variants (the gradient types);
+// the other types run the runtime-K variant for every K.
+template <typename TRV, typename TRS, bool FAST>
 hipError_t dispatchK(const ReduceArgs& a, int64_t head, int64_t nvec,
                      int64_t tail, int numCus, hipStream_t stream) {
   if (a.op == FRG_MAX) {
     return launchVariant<TRV, TRS, FRG_MAX, 0>(a, head, nvec, tail, numCus, stream);
   }
-  switch (a.K) {
-    case 2:
-      return launchVariant<TRV, TRS, FRG_SUM, 2>(a, head, nvec, tail, numCus, stream);
-    case 4:
-      return launchVariant<TRV, TRS, FRG_SUM, 4>(a, head, nvec, tail, numCus, stream);
-    case 8:
-      return launchVariant<TRV, TRS, FRG_SUM, 8>(a, head, nvec, tail, numCus, stream);
-    default:
-      return launchVariant<TRV, TRS, FRG_SUM, 0>(a, head, nvec, tail, numCus, stream);
+  if constexpr (FAST) {
+    switch (a.K) {
+      case 2:
+        return launchVariant<TRV, TRS, FRG_SUM, 2>(a, head, nvec, tail, numCus, stream);
+      case 4:
+        return launchVariant<TRV, TRS, FRG_SUM, 4>(a, head, nvec, tail, numCus, stream);
+      case 8:
+        return launchVariant<TRV, TRS, FRG_SUM, 8>(a, head, nvec, tail, numCus, stream);
+      default:
+        break;
+    }
   }
+  return launchVariant<TRV, TRS, FRG_SUM, 0>(a, head, nvec, tail, numCus, stream);
+}
+
+// Vector variant when the pointers allow it (nvec > 0), else the element-wise
+// one: pointers that disagree modulo 16, or a slice shorter than a vector.
+template <typename TRV, typename TRS, bool FAST>
+hipError_t dispatchType(const ReduceArgs& a, int64_t head, int64_t nvec, int64_t tail,
+                        int numCus, hipStream_t stream) {
+  if (nvec > 0) return dispatchK<TRV, TRS, FAST>(a, head, nvec, tail, numCus, stream);
+  return dispatchK<TRS, TRS, false>(a, 0, a.n, 0, numCus, stream);
 }
 
 }  // namespace
+
+int64_t elementSize(int dtype) {
+  switch (dtype) {
+    case FRG_F32:
+    case FRG_I32:
+      return 4;
+    case FRG_BF16:
+    case FRG_F16:
+      return 2;
+    case FRG_F64:
+    case FRG_I64:
+      return 8;
+    case FRG_U8:
+    case FRG_I8:
+      return 1;
+    default:
+      return 0;
+  }
+}
+
+bool isFloating(int dtype) {
+  return dtype == FRG_F32 || dtype == FRG_BF16 || dtype == FRG_F16 || dtype == FRG_F64;
+}
 
 void setTuning(int blocksPerCu) { gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0; }
 
@@ -393,7 +506,8 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
     if (err) *err = msg;
     return code;
   };
-  if (a.dtype != FRG_F32 && a.dtype != FRG_BF16) {
+  const int64_t elsize = elementSize(a.dtype);
+  if (elsize == 0) {
     return fail(FRG_ERR_UNSUPPORTED, "unsupported dtype " + std::to_string(a.dtype));
   }
   if (a.op != FRG_SUM && a.op != FRG_MAX) {
@@ -410,11 +524,13 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   if (a.op == FRG_MAX && a.scale_mode != FRG_SCALE_NONE) {
     return fail(FRG_ERR_INVALID, "MAX takes no post-scale");
   }
+  if (a.scale_mode != FRG_SCALE_NONE && !isFloating(a.dtype)) {
+    return fail(FRG_ERR_INVALID, "integer types take no post-scale");
+  }
   if (a.contribs == nullptr) return fail(FRG_ERR_INVALID, "null contribution table");
   if (a.n == 0) return FRG_OK;  // device.cc:120-122
   if (a.out == nullptr) return fail(FRG_ERR_INVALID, "null output");
 
-  const int64_t elsize = a.dtype == FRG_F32 ? 4 : 2;
   const int lanes = static_cast<int>(16 / elsize);
   const uintptr_t o = reinterpret_cast<uintptr_t>(a.out);
   const uintptr_t bytes = static_cast<uintptr_t>(a.n) * elsize;
@@ -446,24 +562,34 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
     nvec = (a.n - head) / lanes;
     tail = a.n - head - nvec * lanes;
   }
-  hipError_t e;
-  if (nvec > 0) {
-    e = a.dtype == FRG_F32
-            ? dispatchK<F32Vec, F32Scalar>(a, head, nvec, tail, numCus, stream)
-            : dispatchK<Bf16Vec, Bf16Scalar>(a, head, nvec, tail, numCus, stream);
-  } else {
-    // Pointers disagree modulo 16 (or the slice is shorter than a vector):
-    // element-wise variant, still coalesced, one element per lane.
-    ReduceArgs s = a;
-    if (a.dtype == FRG_F32) {
-      e = a.op == FRG_MAX
-              ? launchVariant<F32Scalar, F32Scalar, FRG_MAX, 0>(s, 0, a.n, 0, numCus, stream)
-              : launchVariant<F32Scalar, F32Scalar, FRG_SUM, 0>(s, 0, a.n, 0, numCus, stream);
-    } else {
-      e = a.op == FRG_MAX
-              ? launchVariant<Bf16Scalar, Bf16Scalar, FRG_MAX, 0>(s, 0, a.n, 0, numCus, stream)
-              : launchVariant<Bf16Scalar, Bf16Scalar, FRG_SUM, 0>(s, 0, a.n, 0, numCus, stream);
-    }
+  hipError_t e = hipErrorInvalidValue;
+  switch (a.dtype) {
+    case FRG_F32:
+      e = dispatchType<F32Vec, F32Scalar, true>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_BF16:
+      e = dispatchType<Bf16Vec, Bf16Scalar, true>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_F16:
+      e = dispatchType<F16Vec, F16Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_F64:
+      e = dispatchType<F64Vec, F64Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_I32:
+      e = dispatchType<I32Vec, I32Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_I64:
+      e = dispatchType<I64Vec, I64Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_U8:
+      e = dispatchType<U8Vec, U8Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    case FRG_I8:
+      e = dispatchType<I8Vec, I8Scalar, false>(a, head, nvec, tail, numCus, stream);
+      break;
+    default:
+      break;
   }
   if (e != hipSuccess) {
     return fail(FRG_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString(e));

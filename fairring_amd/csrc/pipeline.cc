@@ -49,8 +49,6 @@ class DeviceGuard {
   bool changed_ = false;
 };
 
-int64_t elementSize(int dtype) { return dtype == FRG_F32 ? 4 : 2; }
-
 }  // namespace
 
 void setLastError(const std::string& msg) { tlsError = msg; }
@@ -268,7 +266,7 @@ int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
 
 int Context::submit(Request req, Work** workOut, std::string* err) {
   // Contract checks made on the caller's thread, before anything is queued.
-  if (req.dtype != FRG_F32 && req.dtype != FRG_BF16) {
+  if (elementSize(req.dtype) == 0) {
     *err = "unsupported dtype";
     return FRG_ERR_UNSUPPORTED;
   }
@@ -290,6 +288,10 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   }
   if (req.scaleMode < FRG_SCALE_NONE || req.scaleMode > FRG_SCALE_DIV) {
     *err = "bad scale mode";
+    return FRG_ERR_INVALID;
+  }
+  if (req.scaleMode != FRG_SCALE_NONE && !isFloating(req.dtype)) {
+    *err = "integer types take no post-scale";
     return FRG_ERR_INVALID;
   }
   if (kAlignment % elementSize(req.dtype) != 0) {  // fairring/device.cc:316

@@ -33,6 +33,18 @@ int dtypeCode(const at::Tensor& t) {
       return FRG_F32;
     case at::kBFloat16:
       return FRG_BF16;
+    case at::kHalf:
+      return FRG_F16;
+    case at::kDouble:
+      return FRG_F64;
+    case at::kInt:
+      return FRG_I32;
+    case at::kLong:
+      return FRG_I64;
+    case at::kByte:
+      return FRG_U8;
+    case at::kChar:
+      return FRG_I8;
     default:
       return -1;
   }

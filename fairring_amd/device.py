@@ -10,8 +10,8 @@ import os
 import sys
 
 from . import _capi
-from ._capi import (BF16, F32, MAX, SCALE_DIV, SCALE_MUL, SCALE_NONE, SUM,
-                    FairringError)
+from ._capi import (BF16, F16, F32, F64, I8, I32, I64, MAX, SCALE_DIV, SCALE_MUL,
+                    SCALE_NONE, SUM, U8, FairringError)
 
 MiB = 1024 * 1024
 
@@ -54,11 +54,12 @@ def compute_layout(max_memory, max_padding, min_parallelism, num_machines, devic
 
 def _dtype_code(t):
     import torch
-    if t.dtype == torch.float32:
-        return F32
-    if t.dtype == torch.bfloat16:
-        return BF16
-    raise FairringError(_capi.ERR_UNSUPPORTED, "unsupported dtype %s" % t.dtype)
+    codes = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16, torch.float64: F64,
+             torch.int32: I32, torch.int64: I64, torch.uint8: U8, torch.int8: I8}
+    try:
+        return codes[t.dtype]
+    except KeyError:
+        raise FairringError(_capi.ERR_UNSUPPORTED, "unsupported dtype %s" % t.dtype)
 
 
 def is_non_overlapping_and_dense(t):

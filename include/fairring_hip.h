@@ -32,14 +32,27 @@ enum {
   FRG_ERR_NOT_READY = 5    /* non-blocking query: work not finished yet */
 };
 
-/* element types of a slice (storage type; accumulation is fp32 for both) */
-enum { FRG_F32 = 0, FRG_BF16 = 1 };
+/* Element types of a slice: the types the reference maps to NCCL types
+ * (fairring/utils.h:221-245). Storage type; the fold runs in fp32 for fp32,
+ * bf16 and fp16 (one rounding on the store), in fp64 for fp64, and with
+ * two's-complement wrap-around in the element's own width for integers. */
+enum {
+  FRG_F32 = 0,
+  FRG_BF16 = 1,
+  FRG_F16 = 2,
+  FRG_F64 = 3,
+  FRG_I32 = 4,
+  FRG_I64 = 5,
+  FRG_U8 = 6,
+  FRG_I8 = 7
+};
 
 /* reduction ops accepted by MachineFairring::allReduce (machine.cc:181) */
 enum { FRG_SUM = 0, FRG_MAX = 1 };
 
 /* fused post-scale applied once to the accumulated value before the store */
 enum {
+  /* floating-point types only */
   FRG_SCALE_NONE = 0, /* out = acc                                     */
   FRG_SCALE_MUL = 1,  /* out = acc * scale  (scale = 1/K; exact for K = 2^p) */
   FRG_SCALE_DIV = 2   /* out = acc / scale  (scale = K; IEEE division, at::div) */

@@ -40,7 +40,12 @@ def lib():
         for name in ("orc_sum_f32", "orc_sum_f32_chain", "orc_sum_bf16"):
             getattr(L, name).argtypes = [vp, vp, i32, i64, i32, f32]
             getattr(L, name).restype = None
-        for name in ("orc_max_f32", "orc_max_bf16"):
+        for name in ("orc_sum_f16", "orc_sum_f64"):
+            getattr(L, name).argtypes = [vp, vp, i32, i64, i32, f32]
+            getattr(L, name).restype = None
+        for name in ("orc_max_f32", "orc_max_bf16", "orc_max_f16", "orc_max_f64",
+                     "orc_sum_i32", "orc_max_i32", "orc_sum_i64", "orc_max_i64",
+                     "orc_sum_u8", "orc_max_u8", "orc_sum_i8", "orc_max_i8"):
             getattr(L, name).argtypes = [vp, vp, i32, i64]
             getattr(L, name).restype = None
         L.orc_ceil_of_ratio.argtypes = [i64, i64]
@@ -107,6 +112,29 @@ def max_bf16(contribs):
     arrs, n = _prep(contribs, np.uint16)
     out = np.empty(n, np.uint16)
     lib().orc_max_bf16(out.ctypes.data, _ptr_table(arrs), len(arrs), n)
+    return out
+
+
+# name -> (numpy storage dtype, takes a post-scale)
+TYPES = {"f32": (np.float32, True), "bf16": (np.uint16, True), "f16": (np.uint16, True),
+         "f64": (np.float64, True), "i32": (np.int32, False), "i64": (np.int64, False),
+         "u8": (np.uint8, False), "i8": (np.int8, False)}
+
+
+def reduce(kind, contribs, op="sum", scale_mode=SCALE_NONE, scale=1.0):
+    """Any element type by name ("f32", "bf16", "f16", "f64", "i32", "i64", "u8",
+    "i8"); bf16 and f16 are passed as uint16 bit patterns."""
+    npdt, scalable = TYPES[kind]
+    arrs, n = _prep(contribs, npdt)
+    out = np.empty(n, npdt)
+    L = lib()
+    L.orc_set_threads(1)
+    fn = getattr(L, "orc_%s_%s" % (op, kind))
+    if op == "sum" and scalable:
+        fn(out.ctypes.data, _ptr_table(arrs), len(arrs), n, scale_mode, scale)
+    else:
+        assert scale_mode == SCALE_NONE
+        fn(out.ctypes.data, _ptr_table(arrs), len(arrs), n)
     return out
 
 

@@ -193,3 +193,123 @@ int orc_max_threads(void) { return omp_get_max_threads(); }
 void orc_set_threads(int n) { (void)n; }
 int orc_max_threads(void) { return 1; }
 #endif
+
+/* ---- the other element types the reference maps to NCCL types ------------
+ * (fairring/utils.h:221-245): fp16 folds in fp32 with one rounding on the
+ * store (ATen's accumulate type for Half), fp64 in fp64, integers with
+ * two's-complement wrap-around in their own width. Same left fold. */
+
+/* IEEE binary16 <-> binary32 without relying on compiler half support. */
+static inline float f16_to_f32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1Fu;
+  uint32_t man = h & 0x3FFu;
+  uint32_t u;
+  if (exp == 0) {
+    if (man == 0) {
+      u = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do {
+        man <<= 1;
+        ++e;
+      } while ((man & 0x400u) == 0);
+      u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+    }
+  } else if (exp == 31) {
+    u = sign | 0x7F800000u | (man << 13);
+  } else {
+    u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+static inline uint16_t f32_to_f16_rne(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  uint32_t sign = (u >> 16) & 0x8000u;
+  uint32_t a = u & 0x7FFFFFFFu;
+  if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu)); /* NaN */
+  if (a >= 0x47800000u) return (uint16_t)(sign | 0x7C00u); /* >= 65536 (incl. inf) -> inf */
+  if (a >= 0x38800000u) { /* normal half range */
+    uint32_t m = a - 0x38000000u; /* rebias exponent by 112 */
+    uint32_t r = m >> 13;
+    uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) ++r; /* may carry into inf: correct */
+    return (uint16_t)(sign | r);
+  }
+  if (a < 0x33000000u) return (uint16_t)sign; /* < 2^-25: rounds to zero */
+  /* subnormal half: value = mant * 2^(e-150), target unit 2^-24 */
+  uint32_t e = a >> 23;
+  uint32_t mant = (a & 0x7FFFFFu) | 0x800000u;
+  uint32_t shift = 126 - e; /* e in [102, 112] -> shift in [14, 24] */
+  uint32_t r = mant >> shift;
+  uint32_t rem = mant & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (r & 1u))) ++r;
+  return (uint16_t)(sign | r);
+}
+
+void orc_sum_f16(uint16_t* out, const uint16_t* const* in, int K, int64_t n, int scale_mode,
+                 float scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = f16_to_f32(in[0][i]);
+    for (int k = 1; k < K; ++k) acc = acc + f16_to_f32(in[k][i]);
+    out[i] = f32_to_f16_rne(apply_scale(acc, scale_mode, scale));
+  }
+}
+
+void orc_max_f16(uint16_t* out, const uint16_t* const* in, int K, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = f16_to_f32(in[0][i]);
+    for (int k = 1; k < K; ++k) acc = max_nan(acc, f16_to_f32(in[k][i]));
+    out[i] = f32_to_f16_rne(acc);
+  }
+}
+
+void orc_sum_f64(double* out, const double* const* in, int K, int64_t n, int scale_mode,
+                 float scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    double acc = in[0][i];
+    for (int k = 1; k < K; ++k) acc = acc + in[k][i];
+    if (scale_mode == ORC_SCALE_MUL) acc = acc * (double)scale;
+    if (scale_mode == ORC_SCALE_DIV) acc = acc / (double)scale;
+    out[i] = acc;
+  }
+}
+
+void orc_max_f64(double* out, const double* const* in, int K, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    double acc = in[0][i];
+    for (int k = 1; k < K; ++k) {
+      double b = in[k][i];
+      acc = (acc != acc) ? acc : ((b != b) ? b : (acc > b ? acc : b));
+    }
+    out[i] = acc;
+  }
+}
+
+#define ORC_INT_REDUCE(NAME, T, UT)                                               \
+  void orc_sum_##NAME(T* out, const T* const* in, int K, int64_t n) {              \
+    for (int64_t i = 0; i < n; ++i) {                                              \
+      UT acc = (UT)in[0][i];                                                       \
+      for (int k = 1; k < K; ++k) acc = (UT)(acc + (UT)in[k][i]);                  \
+      out[i] = (T)acc;                                                             \
+    }                                                                              \
+  }                                                                                \
+  void orc_max_##NAME(T* out, const T* const* in, int K, int64_t n) {              \
+    for (int64_t i = 0; i < n; ++i) {                                              \
+      T acc = in[0][i];                                                            \
+      for (int k = 1; k < K; ++k) acc = in[k][i] > acc ? in[k][i] : acc;           \
+      out[i] = acc;                                                                \
+    }                                                                              \
+  }
+
+ORC_INT_REDUCE(i32, int32_t, uint32_t)
+ORC_INT_REDUCE(i64, int64_t, uint64_t)
+ORC_INT_REDUCE(u8, uint8_t, uint8_t)
+ORC_INT_REDUCE(i8, int8_t, uint8_t)

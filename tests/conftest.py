@@ -24,17 +24,23 @@ def bits32(a):
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
 
-def assert_bits_equal(a, b, what=""):
-    """Bit-exact comparison; any NaN payload counts as equal to any NaN."""
+def assert_bits_equal(a, b, what="", half=False):
+    """Bit-exact comparison; any NaN payload counts as equal to any NaN. uint16
+    arrays hold bf16 bit patterns, or fp16 ones with half=True."""
     a = np.ascontiguousarray(a)
     b = np.ascontiguousarray(b)
     assert a.shape == b.shape, (what, a.shape, b.shape)
+    assert a.dtype == b.dtype, (what, a.dtype, b.dtype)
     if a.dtype == np.float32:
         ua, ub = a.view(np.uint32), b.view(np.uint32)
         both_nan = np.isnan(a) & np.isnan(b)
-    elif a.dtype == np.uint16:  # bf16 bit patterns
+    elif a.dtype == np.float64:
+        ua, ub = a.view(np.uint64), b.view(np.uint64)
+        both_nan = np.isnan(a) & np.isnan(b)
+    elif a.dtype == np.uint16:
         ua, ub = a, b
-        both_nan = ((a & 0x7FFF) > 0x7F80) & ((b & 0x7FFF) > 0x7F80)
+        top = 0x7C00 if half else 0x7F80
+        both_nan = ((a & 0x7FFF) > top) & ((b & 0x7FFF) > top)
     else:
         ua, ub = a, b
         both_nan = np.zeros(a.shape, bool)

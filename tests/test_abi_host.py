@@ -91,7 +91,8 @@ def test_reduce_slice_rejects_bad_arguments_before_touching_the_gpu():
     L = _capi.lib()
     tab = _capi.ptr_table([16, 32])
     assert L.frg_reduce_slice(64, tab, 0, 4, 0, 0, 0, 1.0, 0, None) == _capi.ERR_INVALID
-    assert L.frg_reduce_slice(64, tab, 2, 4, 7, 0, 0, 1.0, 0, None) == _capi.ERR_UNSUPPORTED
+    assert L.frg_reduce_slice(64, tab, 2, 4, 8, 0, 0, 1.0, 0, None) == _capi.ERR_UNSUPPORTED  # dtype code
+    assert L.frg_reduce_slice(64, tab, 2, 4, 4, 0, 1, 0.5, 0, None) == _capi.ERR_INVALID  # int32 with a scale
     assert L.frg_reduce_slice(64, tab, 2, 4, 0, 3, 0, 1.0, 0, None) == _capi.ERR_UNSUPPORTED
     assert L.frg_reduce_slice(64, tab, 2, -1, 0, 0, 0, 1.0, 0, None) == _capi.ERR_INVALID
     assert L.frg_reduce_slice(64, tab, 2, 4, 0, 1, 1, 0.5, 0, None) == _capi.ERR_INVALID

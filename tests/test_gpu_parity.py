@@ -197,7 +197,7 @@ def test_error_paths():
     with pytest.raises(fa.FairringError):  # partial overlap of output and input
         fa.reduce_slice(a[0:600], [a[100:700], a[0:600]])
     with pytest.raises(fa.FairringError):  # unsupported dtype
-        fa.reduce_slice(a.double(), [a.double()])
+        fa.reduce_slice(a.to(torch.int16), [a.to(torch.int16)])
     with pytest.raises(fa.FairringError):  # K beyond one launch
         fa.reduce_slice(a, [a] * 65)
     with pytest.raises(fa.FairringError):  # MAX with a scale
@@ -344,3 +344,83 @@ def test_full_slice_parity_k8_25mib():
     torch.cuda.synchronize()
     host = [t.cpu().numpy() for t in xs]
     assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(host, oracle.SCALE_MUL, 0.125, threads=8))
+
+
+# ---- the other element types (fairring/utils.h:221-245) ---------------------------
+
+def _np_to_gpu(a, tdt):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if tdt in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).to(DEV).view(tdt)
+    return t.to(DEV)
+
+
+def _gpu_to_np(t):
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.cpu().numpy()
+
+
+OTHER_TYPES = [("f16", torch.float16), ("f64", torch.float64), ("i32", torch.int32),
+               ("i64", torch.int64), ("u8", torch.uint8), ("i8", torch.int8)]
+
+
+def _random_of(kind, rng, k, n):
+    if kind == "f16":
+        x = (rng.standard_normal((k, n)) * np.exp(rng.uniform(-8, 6, (k, n)))).astype(np.float32)
+        x[:, 0] = np.inf
+        x[k - 1, 0] = -np.inf
+        x[:, 1] = 60000.0          # overflows fp16 only after the fp32 sum is rounded
+        x[0, 2] = np.nan
+        return x.astype(np.float16).view(np.uint16)
+    if kind == "f64":
+        x = rng.standard_normal((k, n)) * np.exp(rng.uniform(-40, 40, (k, n)))
+        x[0, 0] = np.nan
+        return x
+    info = np.iinfo(oracle.TYPES[kind][0])
+    return rng.integers(info.min, int(info.max) + 1, (k, n), dtype=oracle.TYPES[kind][0])
+
+
+@pytest.mark.parametrize("kind,tdt", OTHER_TYPES)
+@pytest.mark.parametrize("k,n", [(1, 5), (2, 1000), (8, 70001), (13, 4099), (64, 2050)])
+def test_kernel_other_types_vs_oracle(kind, tdt, k, n):
+    _print_case("type", kind, k, n)
+    rng = np.random.default_rng(hash((kind, k, n)) % 2**32)
+    x = _random_of(kind, rng, k, n)
+    xs = [_np_to_gpu(r, tdt) for r in x]
+    out = torch.empty_like(xs[0])
+    half = kind == "f16"
+    fa.reduce_slice(out, xs)
+    torch.cuda.synchronize()
+    assert_bits_equal(_gpu_to_np(out), oracle.reduce(kind, list(x)), kind + " sum", half=half)
+    fa.reduce_slice(out, xs, op=fa.MAX)
+    torch.cuda.synchronize()
+    got, want = _gpu_to_np(out), oracle.reduce(kind, list(x), "max")
+    if kind in ("f16", "f64"):   # the sign of a zero maximum is not specified
+        z = (want == 0) if kind == "f64" else ((want & 0x7FFF) == 0)
+        got, want = got[~z], want[~z]
+    assert_bits_equal(got, want, kind + " max", half=half)
+    if oracle.TYPES[kind][1]:
+        fa.reduce_slice(out, xs, scale_mode=fa.SCALE_DIV, scale=float(k))
+        torch.cuda.synchronize()
+        assert_bits_equal(_gpu_to_np(out), oracle.reduce(kind, list(x), "sum", oracle.SCALE_DIV, float(k)),
+                          kind + " div", half=half)
+    else:
+        with pytest.raises(fa.FairringError):
+            fa.reduce_slice(out, xs, scale_mode=fa.SCALE_MUL, scale=0.5)
+
+
+@pytest.mark.parametrize("kind,tdt", OTHER_TYPES)
+def test_pipeline_other_types_unaligned(kind, tdt):
+    _print_case("type pipeline", kind)
+    k, n, shift = 5, 300_011, 3
+    rng = np.random.default_rng(99)
+    x = _random_of(kind, rng, k, n + shift)
+    big = [_np_to_gpu(r, tdt) for r in x]
+    out = torch.zeros(n + shift, dtype=tdt, device=DEV)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=256 * 1024, max_memory_allocated_in_bytes=MiB)
+    dev.allreduce(out[shift:], [b[shift:] for b in big]).wait()
+    assert_bits_equal(_gpu_to_np(out[shift:]), oracle.reduce(kind, list(x[:, shift:])), kind,
+                      half=kind == "f16")
+    assert int(torch.count_nonzero(out[:shift].view(torch.uint8) if tdt != torch.uint8 else out[:shift])) == 0
+    dev.close()

@@ -194,6 +194,59 @@ def test_max_semantics():
     assert got[4] == 0.0
 
 
+# ---- the other element types ----------------------------------------------------------
+
+def test_f16_conversions_exhaustive_and_sum_vs_aten():
+    bits = np.arange(65536, dtype=np.uint16)
+    vals = bits.view(np.float16).astype(np.float32)
+    back = oracle.reduce("f16", [bits])          # K = 1: f16 -> f32 -> f16 must be the identity
+    assert_bits_equal(back, bits, "f16 round trip", half=True)
+    # every binary32 midpoint between neighbouring halves rounds to even, checked with numpy
+    rng = np.random.default_rng(17)
+    x = (rng.standard_normal((8, 50000)) * np.exp(rng.uniform(-14, 12, (8, 50000)))).astype(np.float32)
+    h = x.astype(np.float16)
+    got = oracle.reduce("f16", list(h.view(np.uint16)))
+    want = torch.sum(torch.from_numpy(h), dim=0).numpy().view(np.uint16)   # fp32 accumulate, one RNE
+    assert_bits_equal(got, want, "f16 sum", half=True)
+    got = oracle.reduce("f16", list(h.view(np.uint16)), "sum", oracle.SCALE_MUL, 0.125)
+    acc = h[0].astype(np.float32)
+    for k in range(1, 8):
+        acc = acc + h[k].astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = (acc * np.float32(0.125)).astype(np.float16).view(np.uint16)
+    assert_bits_equal(got, want, "f16 mul", half=True)
+    assert vals[0x3C00] == 1.0
+
+
+def test_f64_and_integer_types_vs_numpy_and_aten():
+    rng = np.random.default_rng(18)
+    d = rng.standard_normal((9, 20000)) * np.exp(rng.uniform(-40, 40, (9, 20000)))
+    acc = d[0].copy()
+    for k in range(1, 9):
+        acc = acc + d[k]
+    assert_bits_equal(oracle.reduce("f64", list(d)), acc, "f64 chain")
+    assert_bits_equal(oracle.reduce("f64", list(d), "sum", oracle.SCALE_DIV, 9.0), acc / 9.0, "f64 div")
+    t = torch.from_numpy(d)
+    chain = t[0].clone()
+    for k in range(1, 9):
+        chain = torch.add(chain, t[k])
+    assert_bits_equal(oracle.reduce("f64", list(d)), chain.numpy(), "f64 vs at::add")
+    for kind, npdt, lo, hi in (("i32", np.int32, -2**31, 2**31), ("i64", np.int64, -2**63, 2**63),
+                               ("u8", np.uint8, 0, 256), ("i8", np.int8, -128, 128)):
+        x = rng.integers(lo, hi, (7, 5000), dtype=npdt)       # full range: sums wrap around
+        with np.errstate(over="ignore"):
+            want = x[0].copy()
+            for k in range(1, 7):
+                want = (want + x[k]).astype(npdt)
+        assert (oracle.reduce(kind, list(x)) == want).all(), kind
+        # ATen sums integers in int64 and casts to the output type: the same wrap-around
+        tw = torch.sum(torch.from_numpy(x), dim=0).to(torch.from_numpy(x).dtype).numpy()
+        assert (oracle.reduce(kind, list(x)) == tw).all(), kind + " vs aten"
+        assert (oracle.reduce(kind, list(x), "max") == x.max(axis=0)).all(), kind + " max"
+    m = oracle.reduce("f64", list(d), "max")
+    assert (m == d.max(axis=0)).all()
+
+
 # ---- layout and slicing ---------------------------------------------------------------
 
 MiB = 1024 * 1024
