@@ -1,0 +1,77 @@
+// A CPU stand-in for the few HIP runtime calls the slice pipeline makes, so
+// that its host logic (slicing, stream/event choreography, slot reuse, error
+// paths) can run on a machine without a GPU and under ThreadSanitizer.
+// Test infrastructure only: the shipped library is never built against it.
+//
+// Semantics kept: a stream is an in-order queue drained by its own thread; an
+// event record is a point in its stream; a stream wait snapshots the event's
+// record at the time of the call; "device memory" is host memory.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+typedef int hipError_t;
+enum {
+  hipSuccess = 0,
+  hipErrorInvalidValue = 1,
+  hipErrorOutOfMemory = 2,
+  hipErrorInvalidDevice = 101,
+  hipErrorNotReady = 600,
+  hipErrorUnknown = 999
+};
+
+struct FakeStream;
+struct FakeEvent;
+typedef FakeStream* hipStream_t;
+typedef FakeEvent* hipEvent_t;
+
+enum hipMemcpyKind {
+  hipMemcpyHostToHost = 0,
+  hipMemcpyHostToDevice = 1,
+  hipMemcpyDeviceToHost = 2,
+  hipMemcpyDeviceToDevice = 3
+};
+
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 0 };
+
+#define hipStreamNonBlocking 0x01
+#define hipEventDisableTiming 0x02
+
+extern "C" {
+hipError_t hipGetDeviceCount(int* count);
+hipError_t hipGetDevice(int* device);
+hipError_t hipSetDevice(int device);
+hipError_t hipDeviceGetAttribute(int* value, hipDeviceAttribute_t attr, int device);
+hipError_t hipGetLastError(void);
+const char* hipGetErrorString(hipError_t e);
+
+hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags);
+hipError_t hipStreamSynchronize(hipStream_t stream);
+hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int flags);
+
+hipError_t hipEventCreate(hipEvent_t* event);
+hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned int flags);
+hipError_t hipEventDestroy(hipEvent_t event);
+hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream);
+hipError_t hipEventQuery(hipEvent_t event);
+hipError_t hipEventSynchronize(hipEvent_t event);
+hipError_t hipEventElapsedTime(float* ms, hipEvent_t start, hipEvent_t stop);
+
+hipError_t hipMalloc(void** ptr, size_t size);
+hipError_t hipFree(void* ptr);
+hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind kind,
+                          hipStream_t stream);
+
+// ---- hooks for tests ------------------------------------------------------
+// Occupies `stream` (nullptr = the default stream) for `ms` milliseconds.
+void fake_hip_occupy(hipStream_t stream, int ms);
+// Makes the `nth` next call (1 = the very next) of the named API fail once.
+void fake_hip_fail_call(const char* api, int nth);
+// Calls made so far to the named API.
+long fake_hip_calls(const char* api);
+}
+
+// C++ only: run `fn(arg)` as one unit of work on a stream (how the test build's
+// stand-in for the reduction kernel gets onto the fake streams).
+void fake_hip_enqueue(hipStream_t stream, void (*fn)(void*), void* arg);

@@ -1,0 +1,366 @@
+// Host-logic tests of the slice pipeline (fairring_amd/csrc/pipeline.cc behind
+// the C ABI) on the fake HIP runtime: no GPU, meant to run under
+// ThreadSanitizer and AddressSanitizer. Each scenario prints its name and
+// aborts on the first failed check.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/fairring_hip.h"
+
+#define CHECK(cond)                                                                  \
+  do {                                                                               \
+    if (!(cond)) {                                                                   \
+      std::fprintf(stderr, "CHECK failed: %s (%s:%d) last error: %s\n", #cond, __FILE__, \
+                   __LINE__, frg_last_error());                                      \
+      std::abort();                                                                  \
+    }                                                                                \
+  } while (0)
+
+namespace {
+
+using Vec = std::vector<float>;
+
+std::vector<Vec> randomContribs(int k, int64_t n, unsigned seed) {
+  std::mt19937 rng(seed);
+  std::normal_distribution<float> d(0.f, 0.01f);
+  std::vector<Vec> v(k, Vec(static_cast<size_t>(n)));
+  for (auto& c : v) {
+    for (auto& x : c) x = d(rng);
+  }
+  return v;
+}
+
+Vec fold(const std::vector<Vec>& c, int scaleMode, float scale, const Vec* carry = nullptr) {
+  Vec out(c[0].size());
+  for (size_t i = 0; i < out.size(); ++i) {
+    size_t k = 0;
+    float acc = carry ? (*carry)[i] : c[k++][i];
+    for (; k < c.size(); ++k) acc = acc + c[k][i];
+    if (scaleMode == FRG_SCALE_MUL) acc = acc * scale;
+    if (scaleMode == FRG_SCALE_DIV) acc = acc / scale;
+    out[i] = acc;
+  }
+  return out;
+}
+
+bool same(const Vec& a, const Vec& b) {
+  return a.size() == b.size() && std::memcmp(a.data(), b.data(), a.size() * 4) == 0;
+}
+
+std::vector<const void*> table(const std::vector<Vec>& c) {
+  std::vector<const void*> t;
+  for (auto& v : c) t.push_back(v.data());
+  return t;
+}
+
+frg_ctx* makeCtx(int64_t total, int64_t slice, int streams, int64_t launchBytes) {
+  frg_options o = {};
+  o.max_memory_allocated_in_bytes = total;
+  o.slice_size_in_bytes = slice;
+  o.num_reduce_streams = streams;
+  o.max_launch_bytes = launchBytes;
+  frg_ctx* ctx = nullptr;
+  CHECK(frg_create(0, &o, &ctx) == FRG_OK);
+  return ctx;
+}
+
+void scenarioResident() {
+  std::puts("resident: slicing, launch splitting, stream rotation");
+  for (int streams : {1, 2, 3}) {
+    for (int64_t launch : {int64_t(-1), int64_t(1024), int64_t(4096)}) {
+      frg_ctx* ctx = makeCtx(16384, 4096, streams, launch);
+      auto c = randomContribs(8, 10007, 1);
+      Vec out(10007);
+      frg_work* w = nullptr;
+      auto t = table(c);
+      CHECK(frg_allreduce(ctx, out.data(), t.data(), 8, 10007, FRG_F32, FRG_SUM, FRG_SCALE_MUL,
+                          0.125f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(frg_work_is_completed(w) == FRG_OK);
+      CHECK(same(out, fold(c, FRG_SCALE_MUL, 0.125f)));
+      frg_work_release(w);
+      // more contributions than one launch takes: chained with carry
+      auto big = randomContribs(150, 3001, 2);
+      Vec out2(3001);
+      auto t2 = table(big);
+      CHECK(frg_allreduce(ctx, out2.data(), t2.data(), 150, 3001, FRG_F32, FRG_SUM, FRG_SCALE_DIV,
+                          150.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(out2, fold(big, FRG_SCALE_DIV, 150.f)));
+      frg_work_release(w);
+      CHECK(frg_destroy(ctx) == FRG_OK);
+    }
+  }
+}
+
+void scenarioBusyProducer() {
+  std::puts("many operations submitted while the producer stream is busy");
+  frg_ctx* ctx = makeCtx(2 * 65536, 65536, 2, 32768);
+  const int ops = 211;
+  std::vector<std::vector<Vec>> inputs;
+  std::vector<Vec> outs(ops);
+  std::vector<frg_work*> works(ops);
+  fake_hip_occupy(nullptr, 100);  // the default stream is busy for a while
+  for (int i = 0; i < ops; ++i) {
+    const int64_t n = 1000 + 37 * i;
+    inputs.push_back(randomContribs(8, n, 100 + i));
+    outs[i].assign(static_cast<size_t>(n), -1.f);
+    auto t = table(inputs.back());
+    CHECK(frg_allreduce(ctx, outs[i].data(), t.data(), 8, n, FRG_F32, FRG_SUM, FRG_SCALE_MUL,
+                        0.125f, /*producer=*/nullptr, nullptr, nullptr, &works[i]) == FRG_OK);
+  }
+  for (int i = 0; i < ops; ++i) {
+    CHECK(frg_work_wait(works[i]) == FRG_OK);
+    CHECK(same(outs[i], fold(inputs[i], FRG_SCALE_MUL, 0.125f)));
+    frg_work_release(works[i]);
+  }
+  CHECK(frg_synchronize(ctx) == FRG_OK);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+void scenarioProducerOrdering() {
+  std::puts("the pipeline waits for the producer stream");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  hipStream_t producer;
+  CHECK(hipStreamCreateWithFlags(&producer, hipStreamNonBlocking) == hipSuccess);
+  const int64_t n = 5000;
+  Vec a(n, 0.f), b(n, 0.f), out(n, -1.f);
+  // the producer fills a and b late, on its own stream
+  fake_hip_occupy(producer, 50);
+  Vec srcA(n, 1.5f), srcB(n, 2.5f);
+  CHECK(hipMemcpyAsync(a.data(), srcA.data(), n * 4, hipMemcpyHostToDevice, producer) == hipSuccess);
+  CHECK(hipMemcpyAsync(b.data(), srcB.data(), n * 4, hipMemcpyHostToDevice, producer) == hipSuccess);
+  const void* t[2] = {a.data(), b.data()};
+  frg_work* w = nullptr;
+  CHECK(frg_allreduce(ctx, out.data(), t, 2, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f, producer,
+                      nullptr, nullptr, &w) == FRG_OK);
+  // a consumer stream ordered after the work without a host wait
+  hipStream_t consumer;
+  CHECK(hipStreamCreateWithFlags(&consumer, hipStreamNonBlocking) == hipSuccess);
+  Vec copy(n, 0.f);
+  CHECK(frg_work_block_stream(w, consumer) == FRG_OK);
+  CHECK(hipMemcpyAsync(copy.data(), out.data(), n * 4, hipMemcpyDeviceToHost, consumer) == hipSuccess);
+  CHECK(hipStreamSynchronize(consumer) == hipSuccess);
+  for (float x : copy) CHECK(x == 4.0f);
+  frg_work_release(w);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+void scenarioHostStaged() {
+  std::puts("host-staged accumulation: slot rotation and reuse");
+  for (int slots : {1, 2, 3, 5, 8}) {
+    frg_ctx* ctx = makeCtx(4096 * slots, 4096, 0, 0);
+    frg_layout l;
+    CHECK(frg_get_layout(ctx, &l) == FRG_OK && l.num_staging_slots == slots);
+    for (int k : {1, 2, 7, 20}) {
+      auto c = randomContribs(k, 2500, 7 * k + slots);  // 3 staged slices of <= 1024 elements
+      Vec out(2500, -1.f);
+      auto t = table(c);
+      frg_work* w = nullptr;
+      CHECK(frg_allreduce_host(ctx, out.data(), t.data(), k, 2500, FRG_F32, FRG_SUM,
+                               FRG_SCALE_DIV, static_cast<float>(k), /*carry=*/0, nullptr, nullptr,
+                               nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(out, fold(c, FRG_SCALE_DIV, static_cast<float>(k))));
+      frg_work_release(w);
+      // carry: the output already holds the first term
+      Vec own = c[0];
+      std::vector<Vec> rest(c.begin() + 1, c.end());
+      auto tr = table(rest);
+      CHECK(frg_allreduce_host(ctx, own.data(), tr.data(), k - 1, 2500, FRG_F32, FRG_SUM,
+                               FRG_SCALE_DIV, static_cast<float>(k), /*carry=*/1, nullptr, nullptr,
+                               nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(own, fold(c, FRG_SCALE_DIV, static_cast<float>(k))));
+      frg_work_release(w);
+    }
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
+struct CallbackState {
+  std::atomic<int> calls{0};
+  std::atomic<int> status{-1};
+  std::atomic<void*> stream{nullptr};
+};
+
+void onDone(void* user, int status, void* lastStream) {
+  auto* s = static_cast<CallbackState*>(user);
+  s->status = status;
+  s->stream = lastStream;
+  s->calls++;
+}
+
+void scenarioCallback() {
+  std::puts("completion callback: once per operation, ordered on the last stream");
+  frg_ctx* ctx = makeCtx(8192, 4096, 3, 512);
+  auto c = randomContribs(4, 9001, 5);
+  Vec out(9001, -1.f);
+  auto t = table(c);
+  CallbackState st;
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 4, 9001, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, &onDone, &st, nullptr) == FRG_OK);
+  while (st.calls.load() == 0) std::this_thread::yield();
+  CHECK(st.status.load() == FRG_OK && st.stream.load() != nullptr);
+  // everything the operation launched is ordered before the end of that one stream
+  CHECK(hipStreamSynchronize(static_cast<hipStream_t>(st.stream.load())) == hipSuccess);
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  CHECK(frg_synchronize(ctx) == FRG_OK);
+  CHECK(st.calls.load() == 1);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+void scenarioErrors() {
+  std::puts("error paths: injected HIP failures, contract violations");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+  auto c = randomContribs(3, 3000, 9);
+  Vec out(3000);
+  auto t = table(c);
+  frg_work* w = nullptr;
+  // a copy fails while the command thread enqueues: the work reports it, the context lives on
+  fake_hip_fail_call("hipMemcpyAsync", 2);
+  CallbackState st;
+  CHECK(frg_allreduce_host(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                           1.f, 0, nullptr, &onDone, &st, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_ERR_HIP);
+  CHECK(std::strstr(frg_last_error(), "HIP error") != nullptr);
+  while (st.calls.load() == 0) std::this_thread::yield();
+  CHECK(st.status.load() == FRG_ERR_HIP);
+  frg_work_release(w);
+  CHECK(frg_allreduce_host(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                           1.f, 0, nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  frg_work_release(w);
+  // recording the initial event fails on the caller's thread: the call itself reports it
+  fake_hip_fail_call("hipEventRecord", 1);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, nullptr, nullptr, &w) == FRG_ERR_HIP);
+  CHECK(w == nullptr);
+  // contract violations
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 0, 3000, FRG_F32, FRG_SUM, 0, 1.f, nullptr,
+                      nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, 42, FRG_SUM, 0, 1.f, nullptr, nullptr,
+                      nullptr, nullptr) == FRG_ERR_UNSUPPORTED);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, 5, 0, 1.f, nullptr, nullptr,
+                      nullptr, nullptr) == FRG_ERR_UNSUPPORTED);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_MAX, FRG_SCALE_MUL, .5f,
+                      nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+  CHECK(frg_allreduce(ctx, nullptr, t.data(), 3, 3000, FRG_F32, FRG_SUM, 0, 1.f, nullptr,
+                      nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 0, FRG_F32, FRG_SUM, 0, 1.f, nullptr, nullptr,
+                      nullptr, &w) == FRG_OK);  // empty: completes, nothing launched
+  CHECK(frg_work_wait(w) == FRG_OK);
+  frg_work_release(w);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+  // creation failures
+  frg_options o = {};
+  o.max_memory_allocated_in_bytes = 1000;
+  o.slice_size_in_bytes = 4096;
+  frg_ctx* bad = nullptr;
+  CHECK(frg_create(0, &o, &bad) == FRG_ERR_LAYOUT && bad == nullptr);
+  o.max_memory_allocated_in_bytes = 8192;
+  fake_hip_fail_call("hipMalloc", 1);
+  CHECK(frg_create(0, &o, &bad) == FRG_ERR_HIP && bad == nullptr);
+  CHECK(frg_create(7, &o, &bad) == FRG_ERR_INVALID);
+}
+
+void scenarioProfiling() {
+  std::puts("profile marks and per-launch records");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  auto c = randomContribs(8, 4096, 3);
+  Vec out(4096);
+  auto t = table(c);
+  CHECK(frg_profile_mark(ctx) == FRG_OK);
+  for (int i = 0; i < 3; ++i) {
+    CHECK(frg_allreduce(ctx, out.data(), t.data(), 8, 4096, FRG_F32, FRG_SUM, 0, 1.f, nullptr,
+                        nullptr, nullptr, nullptr) == FRG_OK);
+  }
+  CHECK(frg_profile_mark(ctx) == FRG_OK);
+  frg_launch_record recs[64];
+  int n = 0;
+  CHECK(frg_launch_records(ctx, recs, 64, &n) == FRG_OK);
+  CHECK(n == 2);  // one region, two reduce streams
+  int64_t launches = 0, elems = 0;
+  for (int i = 0; i < n; ++i) {
+    CHECK(recs[i].end_ms >= recs[i].begin_ms && recs[i].num_contributions == 8);
+    launches += recs[i].launches;
+    elems += recs[i].numel;
+  }
+  CHECK(launches == 3 * 16 && elems == 3 * 4096);  // 4 slices x 4 launches of 256 elements
+  CHECK(frg_set_profiling(ctx, 1) == FRG_OK);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 8, 4096, FRG_F32, FRG_SUM, 0, 1.f, nullptr,
+                      nullptr, nullptr, nullptr) == FRG_OK);
+  float ms[64];
+  CHECK(frg_kernel_times(ctx, ms, 64, &n) == FRG_OK && n == 16);
+  for (int i = 0; i < n; ++i) CHECK(ms[i] >= 0.f);
+  CHECK(frg_set_profiling(ctx, 0) == FRG_OK);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+void scenarioDestroyWithPendingWork() {
+  std::puts("destroy drains what was submitted");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  auto c = randomContribs(8, 50000, 11);
+  Vec out(50000, -1.f);
+  auto t = table(c);
+  fake_hip_occupy(nullptr, 30);
+  frg_work* w = nullptr;
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 8, 50000, FRG_F32, FRG_SUM, 0, 1.f, nullptr,
+                      nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_destroy(ctx) == FRG_OK);  // no wait before it
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  CHECK(frg_work_wait(w) == FRG_OK);  // the handle outlives the context
+  frg_work_release(w);
+}
+
+void scenarioConcurrentSubmitters() {
+  std::puts("several threads submit to one context");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  std::vector<std::thread> threads;
+  std::atomic<int> ok{0};
+  for (int tix = 0; tix < 4; ++tix) {
+    threads.emplace_back([ctx, tix, &ok] {
+      for (int i = 0; i < 25; ++i) {
+        auto c = randomContribs(3, 2000 + i, 1000 * tix + i);
+        Vec out(c[0].size());
+        auto t = table(c);
+        frg_work* w = nullptr;
+        CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, static_cast<int64_t>(out.size()),
+                            FRG_F32, FRG_SUM, 0, 1.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+        CHECK(frg_work_wait(w) == FRG_OK);
+        CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+        frg_work_release(w);
+        ok++;
+      }
+    });
+  }
+  for (auto& th : threads) th.join();
+  CHECK(ok.load() == 100);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+}  // namespace
+
+int main() {
+  scenarioResident();
+  scenarioBusyProducer();
+  scenarioProducerOrdering();
+  scenarioHostStaged();
+  scenarioCallback();
+  scenarioErrors();
+  scenarioProfiling();
+  scenarioDestroyWithPendingWork();
+  scenarioConcurrentSubmitters();
+  std::puts("ALL HOST SCENARIOS PASSED");
+  return 0;
+}
