@@ -50,6 +50,7 @@ def parse_args():
     ap.add_argument("--streams", type=int, default=0, help="reduce streams (0 = library default)")
     ap.add_argument("--launch-bytes", type=int, default=0,
                     help="bytes of one contribution per launch (0 = library default, -1 = slice)")
+    ap.add_argument("--copy-streams", type=int, default=0, help="host-staged path (0 = default)")
     ap.add_argument("--blocks-per-cu", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-slices", type=int, default=8)
@@ -252,7 +253,8 @@ def per_launch_pass(fa, args, run_steps):
     dev1 = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                              slice_size_in_bytes=args.slice_bytes,
                              num_reduce_streams=args.streams,
-                             max_launch_bytes=args.launch_bytes)
+                             max_launch_bytes=args.launch_bytes,
+                             num_copy_streams=args.copy_streams)
     run_steps(dev1).wait()
     dev1.synchronize()
     dev1.set_profiling(True)
@@ -329,7 +331,8 @@ def run_c3(args, np, torch, fa, oracle):
     dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                             slice_size_in_bytes=args.slice_bytes,
                             num_reduce_streams=args.streams,
-                            max_launch_bytes=args.launch_bytes)
+                            max_launch_bytes=args.launch_bytes,
+                            num_copy_streams=args.copy_streams)
 
     def step(d):
         return d.allreduce_host(out, hs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)

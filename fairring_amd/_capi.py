@@ -45,7 +45,7 @@ class Options(ctypes.Structure):
                 ("slice_size_in_bytes", ctypes.c_int64),
                 ("num_machines", ctypes.c_int64),
                 ("num_reduce_streams", ctypes.c_int32),
-                ("reserved", ctypes.c_int32),
+                ("num_copy_streams", ctypes.c_int32),
                 ("max_launch_bytes", ctypes.c_int64)]
 
 

@@ -127,7 +127,12 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
       FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
       c->reduceStreams_.push_back(s);
     }
-    FRG_HIP_CHECK(hipStreamCreateWithFlags(&c->copyStream_, hipStreamNonBlocking));
+    const int nCopy = o.num_copy_streams > 0 ? o.num_copy_streams : 2;
+    for (int i = 0; i < nCopy && i < 4; ++i) {
+      hipStream_t s;
+      FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+      c->copyStreams_.push_back(s);
+    }
     FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->stagingPool_),
                             static_cast<size_t>(c->numSlots_ * c->slotBytes_)));
     for (int64_t i = 0; i < c->numSlots_; ++i) {
@@ -170,7 +175,7 @@ Context::~Context() {
   (void)hipGetDevice(&prev);
   (void)hipSetDevice(device_);
   for (hipStream_t s : reduceStreams_) (void)hipStreamSynchronize(s);
-  if (copyStream_) (void)hipStreamSynchronize(copyStream_);
+  for (hipStream_t s : copyStreams_) (void)hipStreamSynchronize(s);
   if (stagingPool_) (void)hipFree(stagingPool_);
   for (hipEvent_t e : slotFreeEvents_) (void)hipEventDestroy(e);
   for (hipEvent_t e : slotFilledEvents_) (void)hipEventDestroy(e);
@@ -472,7 +477,8 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
   hipStream_t s = reduceStreams_[0];
   bool initialFired = false;
   waitInitial(s, initialEvent, &initialFired);
-  waitInitial(copyStream_, initialEvent, &initialFired);
+  for (hipStream_t cs : copyStreams_) waitInitial(cs, initialEvent, &initialFired);
+  const size_t nCopy = copyStreams_.size();
   int64_t batch = numSlots_ / 2;
   if (batch < 1) batch = 1;
   if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
@@ -488,9 +494,9 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       // contribution 0 needs no staging: it lands in `out` directly
       FRG_HIP_CHECK(hipMemcpyAsync(outp,
                                    static_cast<const char*>(req.contribs[0]) + off * elsize,
-                                   bytes, hipMemcpyHostToDevice, copyStream_));
+                                   bytes, hipMemcpyHostToDevice, copyStreams_[0]));
       hipEvent_t first = takeEvent();
-      FRG_HIP_CHECK(hipEventRecord(first, copyStream_));
+      FRG_HIP_CHECK(hipEventRecord(first, copyStreams_[0]));
       FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
       giveEvent(first);
       firstStaged = 1;
@@ -518,19 +524,23 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       slots.clear();
       for (; k < K && static_cast<int64_t>(staged.size()) < batch; ++k) {
         const int64_t slot = (nextStagingSlot_++) % numSlots_;
+        hipStream_t cs = copyStreams_[static_cast<size_t>(slot) % nCopy];
         if (slotUsed_[slot]) {
-          FRG_HIP_CHECK(hipStreamWaitEvent(copyStream_, slotFreeEvents_[slot], 0));
+          FRG_HIP_CHECK(hipStreamWaitEvent(cs, slotFreeEvents_[slot], 0));
         }
         char* dst = stagingPool_ + slot * slotBytes_;
         FRG_HIP_CHECK(hipMemcpyAsync(dst,
                                      static_cast<const char*>(req.contribs[k]) + off * elsize,
-                                     bytes, hipMemcpyHostToDevice, copyStream_));
-        FRG_HIP_CHECK(hipEventRecord(slotFilledEvents_[slot], copyStream_));
+                                     bytes, hipMemcpyHostToDevice, cs));
+        FRG_HIP_CHECK(hipEventRecord(slotFilledEvents_[slot], cs));
         staged.push_back(dst);
         slots.push_back(slot);
       }
-      // The copy stream is in order: the last slot's event covers the batch.
-      FRG_HIP_CHECK(hipStreamWaitEvent(s, slotFilledEvents_[slots.back()], 0));
+      // A copy stream is in order, so per copy stream the last slot's event
+      // covers the earlier ones of the batch.
+      for (size_t b = slots.size() > nCopy ? slots.size() - nCopy : 0; b < slots.size(); ++b) {
+        FRG_HIP_CHECK(hipStreamWaitEvent(s, slotFilledEvents_[slots[b]], 0));
+      }
       ReduceArgs a;
       a.out = outp;
       a.contribs = staged.data();
@@ -618,7 +628,7 @@ int Context::synchronize(std::string* err) {
   try {
     DeviceGuard g(device_);
     for (hipStream_t s : reduceStreams_) FRG_HIP_CHECK(hipStreamSynchronize(s));
-    FRG_HIP_CHECK(hipStreamSynchronize(copyStream_));
+    for (hipStream_t s : copyStreams_) FRG_HIP_CHECK(hipStreamSynchronize(s));
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;

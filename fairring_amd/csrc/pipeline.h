@@ -61,7 +61,7 @@ class Context {
   int device() const { return device_; }
   std::vector<hipStream_t> streams() const {
     std::vector<hipStream_t> v = reduceStreams_;
-    v.push_back(copyStream_);
+    v.insert(v.end(), copyStreams_.begin(), copyStreams_.end());
     return v;
   }
 
@@ -119,7 +119,9 @@ class Context {
   int64_t nextLaunch_ = 0;       // deals launches to the reduce streams
 
   std::vector<hipStream_t> reduceStreams_;
-  hipStream_t copyStream_ = nullptr;
+  // Slot s is filled on copy stream s % copyStreams_.size(): while one stream works through the
+  // event packets around its copy, the other's copy keeps the host link busy.
+  std::vector<hipStream_t> copyStreams_;
 
   char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
   std::vector<hipEvent_t> slotFreeEvents_;    // recorded after a slot's last consumer

@@ -137,10 +137,10 @@ class DeviceFairring:
     def __init__(self, device=0, max_memory_allocated_in_bytes=50 * MiB,
                  max_padding_allocated_in_bytes=MiB, min_parallelism=16,
                  slice_size_in_bytes=0, num_machines=1, num_reduce_streams=0,
-                 max_launch_bytes=0):
+                 max_launch_bytes=0, num_copy_streams=0):
         o = _capi.Options(max_memory_allocated_in_bytes, max_padding_allocated_in_bytes,
                           min_parallelism, slice_size_in_bytes, num_machines,
-                          num_reduce_streams, 0, max_launch_bytes)
+                          num_reduce_streams, num_copy_streams, max_launch_bytes)
         h = ctypes.c_void_p()
         self._h = None
         _capi.check(_capi.lib().frg_create(int(device), ctypes.byref(o), ctypes.byref(h)))

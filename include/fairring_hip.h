@@ -115,7 +115,7 @@ typedef struct frg_options {
   int64_t slice_size_in_bytes;            /* FAIRRING_SLICE_SIZE; 0 = derive with computeLayout */
   int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
   int32_t num_reduce_streams;             /* 0 = default (2) */
-  int32_t reserved;
+  int32_t num_copy_streams;               /* host-staged path; 0 = default (2), at most 4 */
   int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
                                              launch covers; a slice larger than this is reduced by
                                              several launches dealt round-robin to the reduce
@@ -136,8 +136,8 @@ FRG_API int frg_destroy(frg_ctx* ctx);
 /* The layout in force (slice size, number of staging slots). */
 FRG_API int frg_get_layout(frg_ctx* ctx, frg_layout* out);
 
-/* The streams the pipeline launches on (reduce streams first, the copy stream
- * last), for callers that must tell an allocator which streams touch a buffer
+/* The streams the pipeline launches on (reduce streams first, then the copy
+ * streams), for callers that must tell an allocator which streams touch a buffer
  * (the reference calls record_stream on its five streams, device.cc:297-301). */
 FRG_API int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count);
 
