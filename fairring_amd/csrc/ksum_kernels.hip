@@ -300,19 +300,16 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
       foldChunk<TR, OP, kChunk>(acc, in, k, elemBase, laneBytes, first);
       first = false;
     }
-    const int rem = K - k;
-    if (rem & 4) {
-      foldChunk<TR, OP, 4>(acc, in, k, elemBase, laneBytes, first);
-      first = false;
-      k += 4;
-    }
-    if (rem & 2) {
-      foldChunk<TR, OP, 2>(acc, in, k, elemBase, laneBytes, first);
-      first = false;
-      k += 2;
-    }
-    if (rem & 1) {
-      foldChunk<TR, OP, 1>(acc, in, k, elemBase, laneBytes, first);
+    // what is left (1..7 contributions) is loaded in one go as well
+    switch (K - k) {
+      case 7: foldChunk<TR, OP, 7>(acc, in, k, elemBase, laneBytes, first); break;
+      case 6: foldChunk<TR, OP, 6>(acc, in, k, elemBase, laneBytes, first); break;
+      case 5: foldChunk<TR, OP, 5>(acc, in, k, elemBase, laneBytes, first); break;
+      case 4: foldChunk<TR, OP, 4>(acc, in, k, elemBase, laneBytes, first); break;
+      case 3: foldChunk<TR, OP, 3>(acc, in, k, elemBase, laneBytes, first); break;
+      case 2: foldChunk<TR, OP, 2>(acc, in, k, elemBase, laneBytes, first); break;
+      case 1: foldChunk<TR, OP, 1>(acc, in, k, elemBase, laneBytes, first); break;
+      default: break;
     }
   }
   if constexpr (TR::kFloating) {
@@ -419,6 +416,7 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
     int perLane = (a.K < kChunk ? a.K : kChunk) * kUnroll;
     blocksPerCu = FRG_LOADS_PER_CU / perLane;
     if (blocksPerCu < 1) blocksPerCu = 1;
+    if (blocksPerCu > 8) blocksPerCu = 8;  // a plain copy (K = 1) peaks at 8, not 16
   }
   // Persistent grid: a whole number of blocks per CU. The hardware deals blocks
   // to CUs round-robin, every block gets the same share of tiles, and a CU that
