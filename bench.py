@@ -11,7 +11,7 @@ fused into the store, processed as 25 MiB slices (210 of them, the last
 gradient; inputs are resident in HBM before the timed region starts. Bytes
 counted are the algorithmic ones: (K + 1) * numel * elsize per step.
 
-Other workloads (the remaining BASELINE configurations, for the record):
+Other workloads (the remaining configurations of the benchmark definition, for the record):
   c4    bf16, K = 8 x 1.3 G elements, fp32 accumulate, RNE store, fused /8
   c3    K = 64 contributions of one 25 MiB fp32 slice staged from pinned host
         memory with hipMemcpyAsync, overlapped with the accumulate kernel
@@ -299,7 +299,7 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale)
     layout = dev.layout
     dev.close()
-    name = {"c2": "BASELINE configs[1]", "c4": "BASELINE configs[3]",
+    name = {"c2": "configs[1]", "c4": "configs[3]",
             "copy": "calibration copy"}[args.workload]
     cfg = {
         "workload": "K=%d contributions x %d %s elements, %d slices of %d B, %s, one output "
@@ -358,7 +358,7 @@ def run_c3(args, np, torch, fa, oracle):
     dev.close()
     cfg = {
         "workload": "K=%d pinned-host contributions of one %d-element fp32 slice, staged with "
-                    "hipMemcpyAsync through %d slots, fused x1/%d (BASELINE configs[2])" % (
+                    "hipMemcpyAsync through %d slots, fused x1/%d (configs[2])" % (
                         k, numel, slots, k),
         "k": k, "numel": numel, "layout": layout, "host_link_GBps": round(link, 2),
         "bound": "host link (PCIe): every contribution crosses it once",
@@ -421,7 +421,7 @@ def run_c5(args, np, torch, fa, oracle):
     cfg = {
         "workload": "DDP backward stream: %d fp32 elements as %d buckets (first %d B, then %d B) "
                     "released from the end of the gradient to its start, K=%d contributions per "
-                    "bucket, one allreduce call per bucket, fused x1/%d (BASELINE configs[4])" % (
+                    "bucket, one allreduce call per bucket, fused x1/%d (configs[4])" % (
                         numel, len(spans), MiB, args.slice_bytes, k, k),
         "k": k, "numel": numel, "buckets": len(spans), "staging_total_bytes": args.total_memory,
         "layout": layout, "reduce_streams": args.streams or "default",

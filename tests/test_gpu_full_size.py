@@ -1,4 +1,4 @@
-"""The BASELINE configurations at their full sizes, through the C ABI.
+"""The benchmark configurations at their full sizes, through the C ABI.
 
 At these sizes the oracle cannot re-reduce everything in seconds, so each case
 combines (a) properties whose answer is known in closed form for every element
