@@ -1,39 +1,55 @@
-// Python module _fairring: ProcessGroup and ProcessGroup.Options, as the
-// reference binds them (fairring/bindings.cc:20-47), on the c10d::Backend base
-// that current PyTorch exposes as torch._C._distributed_c10d.Backend.
+// Python module _fairring. It exposes the same two names the reference's
+// module does (fairring/bindings.cc:20-47): ProcessGroup, constructed from
+// (store, rank, size, options) with the GIL released, and the nested
+// ProcessGroup.Options with keyword-capable staging parameters. The base class
+// is c10d::Backend, which current PyTorch shows to Python as
+// torch._C._distributed_c10d.Backend.
 #include <pybind11/chrono.h>
 #include <pybind11/pybind11.h>
 #include <torch/csrc/utils/pybind.h>
 
 #include "process_group.h"
 
+namespace {
+
 namespace py = pybind11;
+using PG = fairring::ProcessGroupFairring;
+using Opts = PG::OptionsFairring;
+using Millis = std::chrono::milliseconds;
 
-using fairring::ProcessGroupFairring;
+c10::intrusive_ptr<Opts> makeOptions(int64_t totalBytes, int64_t paddingBytes, int64_t parallelism,
+                                     bool highPriority, Millis timeout, int64_t sliceBytes) {
+  return Opts::create(totalBytes, paddingBytes, parallelism, highPriority, timeout, sliceBytes);
+}
 
-PYBIND11_MODULE(_fairring, module) {
+c10::intrusive_ptr<PG> makeGroup(const c10::intrusive_ptr<c10d::Store>& store, int rank, int size,
+                                 c10::intrusive_ptr<Opts> options) {
+  return c10::make_intrusive<PG>(store, rank, size, std::move(options));
+}
+
+void bind(py::module& m) {
+  // torch.distributed must be loaded first: it registers the Backend base type
   py::module::import("torch.distributed");
 
-  py::class_<ProcessGroupFairring, c10::intrusive_ptr<ProcessGroupFairring>, c10d::Backend>
-      processGroupFairring(module, "ProcessGroup");
+  py::class_<PG, c10::intrusive_ptr<PG>, c10d::Backend> group(m, "ProcessGroup");
+  py::class_<Opts, c10::intrusive_ptr<Opts>, c10d::Backend::Options> options(group, "Options");
 
-  py::class_<ProcessGroupFairring::OptionsFairring,
-             c10::intrusive_ptr<ProcessGroupFairring::OptionsFairring>, c10d::Backend::Options>(
-      processGroupFairring, "Options")
-      .def(py::init<int64_t, int64_t, int64_t, bool, std::chrono::milliseconds, int64_t>(),
-           py::arg("max_memory_allocated_in_bytes"),
-           py::arg("max_padding_allocated_in_bytes"), py::arg("min_parallelism"),
-           py::arg("is_high_priority_stream") = false,
-           py::arg("timeout") = kBackendDefaultTimeout,
-           py::arg("slice_size_in_bytes") = static_cast<int64_t>(0));
+  options.def(py::init(&makeOptions), py::arg("max_memory_allocated_in_bytes"),
+              py::arg("max_padding_allocated_in_bytes"), py::arg("min_parallelism"),
+              py::arg("is_high_priority_stream") = false,
+              py::arg("timeout") = Millis(kBackendDefaultTimeout),
+              py::arg("slice_size_in_bytes") = int64_t{0});
 
-  processGroupFairring
-      .def(py::init<const c10::intrusive_ptr<c10d::Store>&, int, int,
-                    c10::intrusive_ptr<ProcessGroupFairring::OptionsFairring>>(),
-           py::call_guard<py::gil_scoped_release>())
-      .def("_set_simulated_peer_contributions",
-           &ProcessGroupFairring::setSimulatedPeerContributions, py::arg("peers"),
-           py::call_guard<py::gil_scoped_release>())
-      .def("_set_fused_divide", &ProcessGroupFairring::setFusedDivide, py::arg("on"))
-      .def("_layout", &ProcessGroupFairring::layout);
+  group.def(py::init(&makeGroup), py::arg("store"), py::arg("rank"), py::arg("size"),
+            py::arg("options"), py::call_guard<py::gil_scoped_release>());
+
+  // one-GPU additions, not in the reference
+  group.def("_set_simulated_peer_contributions", &PG::setSimulatedPeerContributions,
+            py::arg("peers"), py::call_guard<py::gil_scoped_release>());
+  group.def("_set_fused_divide", &PG::setFusedDivide, py::arg("on"));
+  group.def("_layout", &PG::layout);
 }
+
+}  // namespace
+
+PYBIND11_MODULE(_fairring, m) { bind(m); }
