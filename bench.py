@@ -175,20 +175,27 @@ def union_length(intervals):
     return total
 
 
-DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch size per contribution
+DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch target per contribution
+LAUNCH_QUANTUM_BYTES = 4096
 
 
 def launch_elems(args, slice_elems, elsize):
-    """Elements of one full-size launch: a slice is cut into equal parts no larger
-    than the launch size (what the pipeline does)."""
+    """Elements of the commonest launch: a slice much larger than the launch
+    target is cut on 4 KiB boundaries into parts of about that size (what the
+    pipeline does); the last part of a slice takes the rest."""
     lb = args.launch_bytes or DEFAULT_LAUNCH_BYTES
     if lb < 0:
         return slice_elems
     max_elems = (lb - lb % 16) // elsize
-    parts = -(-slice_elems // max_elems)
-    lanes = 16 // elsize
-    per = -(-slice_elems // parts)
-    return -(-per // lanes) * lanes
+    if 2 * slice_elems <= 3 * max_elems:
+        return slice_elems
+    parts = (slice_elems + max_elems // 2) // max_elems
+    quantum = LAUNCH_QUANTUM_BYTES // elsize
+    per = (slice_elems // parts) // quantum * quantum
+    if per < quantum:
+        lanes = 16 // elsize
+        per = -(-(-(-slice_elems // parts)) // lanes) * lanes
+    return per
 
 
 def roofline_from_records(recs, bytes_per_elem, full_launch_elems, how):

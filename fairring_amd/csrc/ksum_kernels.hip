@@ -272,11 +272,19 @@ __device__ __forceinline__ void foldChunk(typename TR::acc_t (&acc)[TR::kLanes],
 }
 
 // One vector of the output: out = scale(carry? (+) in[0] (+) ... (+) in[K-1]).
-template <typename TR, int OP, int KT>
+// SC >= 0 fixes the scale mode at compile time and rules out a carry: the hot
+// variants then hold nothing but loads, adds, one multiply and the store (a
+// third of the code, which matters when a launch lasts 10 us and every CU
+// starts it with a cold instruction cache).
+template <typename TR, int OP, int KT, int SC>
 __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
                                           const Ptrs<KT>& in, int K, bool carry,
                                           int scaleMode, float scale,
                                           int64_t elemBase, unsigned int lane) {
+  if (SC >= 0) {
+    carry = false;
+    scaleMode = SC;
+  }
   using vec_t = typename TR::vec_t;
   const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
   vec_t* o = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(out + elemBase) + laneBytes);
@@ -336,34 +344,36 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
 // blocks on CUs round-robin, so spreading the remainder over twice as many
 // blocks in half-size pieces evens out the work per CU, and the launch does not
 // end on a few CUs finishing a whole extra tile.
-template <typename TRV, typename TRS, int OP, int KT>
+template <typename TRV, typename TRS, int OP, int KT, int SC>
 __global__ void __launch_bounds__(kBlock)
     ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K, int carry,
                int scaleMode, float scale, int64_t head, int64_t nvec,
-               int64_t tail) {
+               int64_t tail, int64_t roundTiles, int64_t pieces) {
+  // roundTiles (tiles in whole rounds of the grid) and pieces (remainder pieces
+  // of kBlock * FRG_REMAINDER_PIECE_UNROLL vectors) come from the host: a
+  // 64-bit division by the grid size at the top of every wave is a third of a
+  // microsecond that a 10 us launch does not have.
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
   const int64_t grid = gridDim.x;
-  const int64_t roundTiles = (nvec / kTile / grid) * grid;  // tiles in whole rounds
   for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
     const int64_t elemBase = head + t * kTile * TRV::kLanes;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale, elemBase,
+      reduceOne<TRV, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale, elemBase,
                              threadIdx.x + u * kBlock);
     }
   }
-  // remainder: pieces of kBlock vectors, the last one possibly partial
+  // remainder: pieces of kBlock * kPiece vectors, the last one possibly partial
   const int64_t restBase = roundTiles * kTile;
   constexpr int kPiece = FRG_REMAINDER_PIECE_UNROLL;  // vectors per lane in a remainder piece
-  const int64_t pieceVecs = static_cast<int64_t>(kBlock) * kPiece;
-  const int64_t pieces = (nvec - restBase + pieceVecs - 1) / pieceVecs;
+  constexpr int64_t pieceVecs = static_cast<int64_t>(kBlock) * kPiece;
   for (int64_t p = blockIdx.x; p < pieces; p += grid) {
     const int64_t v0 = restBase + p * pieceVecs;
 #pragma unroll
     for (int u = 0; u < kPiece; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
       if (v0 + lane < nvec) {
-        reduceOne<TRV, OP, KT>(out, in, K, carry != 0, scaleMode, scale,
+        reduceOne<TRV, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale,
                                head + v0 * TRV::kLanes, lane);
       }
     }
@@ -373,7 +383,7 @@ __global__ void __launch_bounds__(kBlock)
     const int64_t e = threadIdx.x < head
                           ? static_cast<int64_t>(threadIdx.x)
                           : head + nvec * TRV::kLanes + (threadIdx.x - head);
-    reduceOne<TRS, OP, KT>(out, in, K, carry != 0, scaleMode, scale, e, 0u);
+    reduceOne<TRS, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale, e, 0u);
   }
 }
 
@@ -401,7 +411,7 @@ DeviceInfo& deviceInfo(int device) {
 
 int gBlocksPerCu = 0;  // 0 = derive from the number of loads per lane
 
-template <typename TRV, typename TRS, int OP, int KT>
+template <typename TRV, typename TRS, int OP, int KT, int SC = -1>
 hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
                          int64_t tail, int numCus, hipStream_t stream) {
   Ptrs<KT> tab;
@@ -425,17 +435,20 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   const int64_t cap = static_cast<int64_t>(numCus) * blocksPerCu;
   int64_t grid = ntiles < cap ? ntiles : cap;
   if (grid < 1) grid = 1;
+  const int64_t roundTiles = (nvec / kTile / grid) * grid;
+  constexpr int64_t kPieceVecs = static_cast<int64_t>(kBlock) * FRG_REMAINDER_PIECE_UNROLL;
+  const int64_t pieces = (nvec - roundTiles * kTile + kPieceVecs - 1) / kPieceVecs;
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
     // Timed launch: the events take the dispatch's own begin/end timestamps.
-    hipExtLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT>), dim3(static_cast<unsigned>(grid)),
+    hipExtLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
                           dim3(kBlock), 0, stream, a.startEvent, a.stopEvent, 0,
                           static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                          a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail);
+                          a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, roundTiles, pieces);
   } else {
-    hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT>), dim3(static_cast<unsigned>(grid)),
+    hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
                        dim3(kBlock), 0, stream,
                        static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                       a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail);
+                       a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, roundTiles, pieces);
   }
   return hipGetLastError();
 }
@@ -449,15 +462,24 @@ hipError_t dispatchK(const ReduceArgs& a, int64_t head, int64_t nvec,
     return launchVariant<TRV, TRS, FRG_MAX, 0>(a, head, nvec, tail, numCus, stream);
   }
   if constexpr (FAST) {
-    switch (a.K) {
-      case 2:
-        return launchVariant<TRV, TRS, FRG_SUM, 2>(a, head, nvec, tail, numCus, stream);
-      case 4:
-        return launchVariant<TRV, TRS, FRG_SUM, 4>(a, head, nvec, tail, numCus, stream);
-      case 8:
-        return launchVariant<TRV, TRS, FRG_SUM, 8>(a, head, nvec, tail, numCus, stream);
-      default:
-        break;
+    // the gradient shapes: 2, 4 or 8 contributions, nothing carried in, no
+    // scale or the multiply by 1/K
+    if (!a.carry && a.scale_mode != FRG_SCALE_DIV) {
+      const bool mul = a.scale_mode == FRG_SCALE_MUL;
+#define FRG_FAST_CASE(KK)                                                                       \
+  case KK:                                                                                       \
+    return mul ? launchVariant<TRV, TRS, FRG_SUM, KK, FRG_SCALE_MUL>(a, head, nvec, tail, numCus, \
+                                                                     stream)                      \
+               : launchVariant<TRV, TRS, FRG_SUM, KK, FRG_SCALE_NONE>(a, head, nvec, tail,       \
+                                                                      numCus, stream);
+      switch (a.K) {
+        FRG_FAST_CASE(2)
+        FRG_FAST_CASE(4)
+        FRG_FAST_CASE(8)
+        default:
+          break;
+      }
+#undef FRG_FAST_CASE
     }
   }
   return launchVariant<TRV, TRS, FRG_SUM, 0>(a, head, nvec, tail, numCus, stream);

@@ -17,7 +17,8 @@ constexpr int64_t kAlignment = 8;
 constexpr int64_t kDefaultTotalMemory = 50ll * 1024 * 1024;   // fairring/__init__.py:26
 constexpr int64_t kDefaultPaddingMemory = 1024ll * 1024;      // fairring/__init__.py:30
 constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init__.py:34
-constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;  // per contribution and launch
+constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;  // per contribution and launch (target)
+constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {
   return num == 0 ? 0 : (num - 1) / den + 1;

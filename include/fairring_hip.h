@@ -116,11 +116,12 @@ typedef struct frg_options {
   int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
   int32_t num_reduce_streams;             /* 0 = default (2) */
   int32_t num_copy_streams;               /* host-staged path; 0 = default (2), at most 4 */
-  int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
-                                             launch covers; a slice larger than this is reduced by
-                                             several launches dealt round-robin to the reduce
-                                             streams. 0 = default (12.5 MiB), < 0 = one launch per
-                                             slice */
+  int64_t max_launch_bytes;               /* target bytes of one contribution that a single
+                                             reduction launch covers; a slice much larger than
+                                             this is reduced by several launches (cut on 4 KiB
+                                             boundaries from the slice start) dealt round-robin
+                                             to the reduce streams. 0 = default (12.5 MiB), < 0
+                                             = one launch per slice */
 } frg_options;
 
 /* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,
