@@ -13,10 +13,12 @@ OK, ERR_INVALID, ERR_HIP, ERR_LAYOUT, ERR_UNSUPPORTED, ERR_NOT_READY = range(6)
 F32, BF16, F16, F64, I32, I64, U8, I8 = range(8)
 SUM, MAX = 0, 1
 SCALE_NONE, SCALE_MUL, SCALE_DIV = 0, 1, 2
+SCALE_PRE_MUL, SCALE_PRE_DIV = 3, 4
 
 # every symbol include/fairring_hip.h declares
 EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_reduce_slice",
+    "frg_reduce_slice_compressed", "frg_allreduce_compressed",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
@@ -87,6 +89,9 @@ def lib():
     L.frg_get_layout.argtypes = [vp, ctypes.POINTER(Layout)]
     L.frg_get_streams.argtypes = [vp, pvp, i32, ctypes.POINTER(i32)]
     L.frg_allreduce.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    L.frg_reduce_slice_compressed.argtypes = [vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp]
+    L.frg_allreduce_compressed.argtypes = [vp, vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp,
+                                           DONE_FN, vp, pvp]
     L.frg_allreduce_host.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp,
                                      DONE_FN, vp, pvp]
     for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize,

@@ -112,6 +112,25 @@ int frg_reduce_slice(void* out, const void* const* contribs, int K, int64_t n, i
   return FRG_OK;
 }
 
+int frg_reduce_slice_compressed(void* out, int out_dtype, const void* const* contribs, int K,
+                                int raw_index, int64_t n, int wire_dtype, int scale_mode,
+                                float scale, void* stream) {
+  frg::CompressedArgs a;
+  a.out = out;
+  a.out_dtype = out_dtype;
+  a.contribs = contribs;
+  a.K = K;
+  a.raw_index = raw_index;
+  a.n = n;
+  a.wire_dtype = wire_dtype;
+  a.scale_mode = scale_mode;
+  a.scale = scale;
+  std::string err;
+  const int rc = frg::launchCompressedReduce(a, static_cast<hipStream_t>(stream), &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  return FRG_OK;
+}
+
 int frg_create(int device, const frg_options* opts, frg_ctx** out) {
   if (out == nullptr) return fail(FRG_ERR_INVALID, "null context output");
   *out = nullptr;
@@ -160,6 +179,37 @@ int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, i
                   frg_done_fn done, void* user, frg_work** work) {
   return submitCommon(ctx, out, contribs, K, numel, dtype, op, scale_mode, scale,
                       producer_stream, done, user, work, /*fromHost=*/false, /*carry=*/false);
+}
+
+int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype, const void* const* contribs,
+                             int K, int raw_index, int64_t numel, int wire_dtype, int scale_mode,
+                             float scale, void* producer_stream, frg_done_fn done, void* user,
+                             frg_work** work) {
+  if (work) *work = nullptr;
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  if (K < 1 || contribs == nullptr) {
+    return fail(FRG_ERR_INVALID, "at least one contribution is required");
+  }
+  Context::Request r;
+  r.out = out;
+  r.contribs.assign(contribs, contribs + K);
+  r.numel = numel;
+  r.dtype = wire_dtype;
+  r.op = FRG_SUM;
+  r.scaleMode = scale_mode;
+  r.scale = scale;
+  r.compressed = true;
+  r.outDtype = out_dtype;
+  r.rawIndex = raw_index;
+  r.producerStream = static_cast<hipStream_t>(producer_stream);
+  r.done = done;
+  r.user = user;
+  std::string err;
+  Work* w = nullptr;
+  const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+  if (rc != FRG_OK) return fail(rc, err);
+  if (work) *work = reinterpret_cast<frg_work*>(w);
+  return FRG_OK;
 }
 
 int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs, int K,

@@ -1,0 +1,362 @@
+// The reduction with torch's gradient-compression hooks folded in (gfx950).
+//
+// With a bf16 or fp16 compression hook registered, every rank of a DDP job
+// does, per bucket
+// (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:57-93):
+//     compressed = buffer.to(wire).div_(world)   two passes over the bucket
+//     allreduce(compressed)                      fairring/process_group.cc:131-155
+//     buffer.copy_(result)                       one more pass
+// Here the three are one pass: the rank's own fp32 bucket is cast, divided and
+// rounded in registers, the peers' contributions are read in the wire type, the
+// fold runs in fp32 in contribution order with one rounding to the wire type
+// (as the plain bf16 / fp16 reduction does), and the result is stored widened
+// into the fp32 bucket, which may be the very buffer the raw term was read
+// from. Per element that is 4 + 2 (K - 1) + 4 bytes of HBM traffic instead of
+// (4 + 2) + (2 K + 2) + (2 + 4).
+//
+// One lane owns 8 consecutive elements: one 16-byte vector of every wire
+// contribution, two of the fp32 buffer on either side.
+
+#include <hip/hip_ext.h>
+#include <hip/hip_runtime.h>
+
+#include "../../include/fairring_hip.h"
+#include "device_traits.h"
+#include "ksum_kernels.h"
+
+namespace frg {
+namespace {
+
+// The fp32 side of a lane's elements: 8 floats as two vectors, or one float in
+// the element-wise variant.
+template <int LANES>
+struct Fp32Side;
+
+template <>
+struct Fp32Side<8> {
+  struct regs_t {
+    f32x4 a, b;
+  };
+  __device__ static regs_t load(const float* base, unsigned int lane) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(base) + lane * 32u);
+    regs_t r;
+    r.a = ldStream(p);
+    r.b = ldStream(p + 1);
+    return r;
+  }
+  __device__ static void unpack(const regs_t& r, float (&f)[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[j] = r.a[j];
+      f[4 + j] = r.b[j];
+    }
+  }
+  __device__ static void store(float* base, unsigned int lane, const float (&f)[8]) {
+    f32x4* p = reinterpret_cast<f32x4*>(reinterpret_cast<char*>(base) + lane * 32u);
+    f32x4 a, b;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      a[j] = f[j];
+      b[j] = f[4 + j];
+    }
+    stStream(a, p);
+    stStream(b, p + 1);
+  }
+};
+
+template <>
+struct Fp32Side<1> {
+  struct regs_t {
+    float a;
+  };
+  __device__ static regs_t load(const float* base, unsigned int lane) {
+    regs_t r;
+    r.a = ldStream(base + lane);
+    return r;
+  }
+  __device__ static void unpack(const regs_t& r, float (&f)[1]) { f[0] = r.a; }
+  __device__ static void store(float* base, unsigned int lane, const float (&f)[1]) {
+    stStream(f[0], base + lane);
+  }
+};
+
+// State of one lane's fold: the accumulator, whether it holds a term yet, and
+// this rank's own term (compressed once the loads that follow it are issued).
+template <typename W>
+struct Fold {
+  float acc[W::kLanes];
+  float own[W::kLanes];
+  bool first = true;
+  bool ownReady = false;
+
+  __device__ __forceinline__ void add(const float (&t)[W::kLanes]) {
+    if (first) {
+#pragma unroll
+      for (int j = 0; j < W::kLanes; ++j) acc[j] = t[j];
+      first = false;
+    } else {
+#pragma unroll
+      for (int j = 0; j < W::kLanes; ++j) acc[j] = acc[j] + t[j];
+    }
+  }
+
+  // buffer.to(wire) then div_(world) in the wire type: two roundings
+  __device__ __forceinline__ void compress(const typename Fp32Side<W::kLanes>::regs_t& raw,
+                                           int scaleMode, float scale) {
+    if (ownReady) return;
+    Fp32Side<W::kLanes>::unpack(raw, own);
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) {
+      float c = W::roundStorage(own[j]);
+      if (scaleMode == FRG_SCALE_MUL) {
+        c = W::roundStorage(c * scale);
+      } else if (scaleMode == FRG_SCALE_DIV) {
+        c = W::roundStorage(c / scale);
+      }
+      own[j] = c;
+    }
+    ownReady = true;
+  }
+};
+
+// Loads wire contributions [k0, k0+N), then folds them in order; the own term
+// goes in ahead of wire contribution `rawPos`.
+template <typename W, int N>
+__device__ __forceinline__ void foldWire(Fold<W>& st, const Ptrs<0>& in, int k0, int64_t elemBase,
+                                         unsigned int laneBytes, int rawPos,
+                                         const typename Fp32Side<W::kLanes>::regs_t& raw,
+                                         int scaleMode, float scale) {
+  using vec_t = typename W::vec_t;
+  using elem_t = typename W::elem_t;
+  vec_t v[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    const char* b = reinterpret_cast<const char*>(static_cast<const elem_t*>(in.p[k0 + k]) + elemBase);
+    v[k] = ldStream(reinterpret_cast<const vec_t*>(b + laneBytes));
+  }
+  if (rawPos >= 0) st.compress(raw, scaleMode, scale);
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    if (k0 + k == rawPos) st.add(st.own);
+    float f[W::kLanes];
+    W::unpack(v[k], f);
+    st.add(f);
+  }
+}
+
+// One lane's group of elements. `wire` holds the Kw peers' pointers in order,
+// `raw` this rank's fp32 buffer (rawPos = its place in the chain, -1: absent).
+template <typename W, bool OUT32>
+__device__ __forceinline__ void compressedOne(void* out, const float* raw, const Ptrs<0>& wire,
+                                              int Kw, int rawPos, int scaleMode, float scale,
+                                              int64_t elemBase, unsigned int lane) {
+  using vec_t = typename W::vec_t;
+  using Side = Fp32Side<W::kLanes>;
+  const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
+  typename Side::regs_t rawRegs = {};
+  if (rawPos >= 0) rawRegs = Side::load(raw + elemBase, lane);
+  Fold<W> st;
+  int k = 0;
+  for (; k + kChunk <= Kw; k += kChunk) {
+    foldWire<W, kChunk>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale);
+  }
+  switch (Kw - k) {
+    case 7: foldWire<W, 7>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 6: foldWire<W, 6>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 5: foldWire<W, 5>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 4: foldWire<W, 4>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 3: foldWire<W, 3>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 2: foldWire<W, 2>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    case 1: foldWire<W, 1>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale); break;
+    default: break;
+  }
+  if (rawPos == Kw) {  // own term last (or alone)
+    st.compress(rawRegs, scaleMode, scale);
+    st.add(st.own);
+  }
+  // one rounding to the wire type; the fp32 output holds that value widened
+  if (OUT32) {
+    float r[W::kLanes];
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) r[j] = W::roundStorage(st.acc[j]);
+    Side::store(static_cast<float*>(out) + elemBase, lane, r);
+  } else {
+    vec_t* o = reinterpret_cast<vec_t*>(
+        reinterpret_cast<char*>(static_cast<typename W::elem_t*>(out) + elemBase) + laneBytes);
+    stStream(W::pack(st.acc), o);
+  }
+}
+
+// Same dealing of tiles, remainder pieces and ragged edges as the plain
+// reduction kernel; a "vector" is a lane's group of 8 elements.
+template <typename WV, typename WS, bool OUT32>
+__global__ void __launch_bounds__(kBlock)
+    compressedKernel(void* out, const float* raw, Ptrs<0> wire, int Kw, int rawPos, int scaleMode,
+                     float scale, int64_t head, int64_t nvec, int64_t tail, int64_t roundTiles,
+                     int64_t pieces) {
+  constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
+  const int64_t grid = gridDim.x;
+  for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
+    const int64_t elemBase = head + t * kTile * WV::kLanes;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      compressedOne<WV, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
+                               threadIdx.x + u * kBlock);
+    }
+  }
+  const int64_t restBase = roundTiles * kTile;
+  constexpr int kPiece = FRG_REMAINDER_PIECE_UNROLL;
+  constexpr int64_t pieceVecs = static_cast<int64_t>(kBlock) * kPiece;
+  for (int64_t p = blockIdx.x; p < pieces; p += grid) {
+    const int64_t v0 = restBase + p * pieceVecs;
+#pragma unroll
+    for (int u = 0; u < kPiece; ++u) {
+      const unsigned int lane = threadIdx.x + u * kBlock;
+      if (v0 + lane < nvec) {
+        compressedOne<WV, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale,
+                                 head + v0 * WV::kLanes, lane);
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < head + tail) {
+    const int64_t e = threadIdx.x < head
+                          ? static_cast<int64_t>(threadIdx.x)
+                          : head + nvec * WV::kLanes + (threadIdx.x - head);
+    compressedOne<WS, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, e, 0u);
+  }
+}
+
+template <typename WV, typename WS, bool OUT32>
+hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptrs<0>& wire, int Kw,
+                            int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
+                            hipStream_t stream) {
+  const GridPlan plan = planGrid(nvec, a.K, numCus);
+  if (a.startEvent != nullptr || a.stopEvent != nullptr) {
+    hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32>),
+                          dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream,
+                          a.startEvent, a.stopEvent, 0, a.out, raw, wire, Kw, rawPos, a.scale_mode,
+                          a.scale, head, nvec, tail, plan.roundTiles, plan.pieces);
+  } else {
+    hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32>), dim3(static_cast<unsigned>(plan.grid)),
+                       dim3(kBlock), 0, stream, a.out, raw, wire, Kw, rawPos, a.scale_mode,
+                       a.scale, head, nvec, tail, plan.roundTiles, plan.pieces);
+  }
+  return hipGetLastError();
+}
+
+template <typename WV, typename WS>
+hipError_t dispatchOut(const CompressedArgs& a, const float* raw, const Ptrs<0>& wire, int Kw,
+                       int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
+                       hipStream_t stream) {
+  if (nvec > 0) {
+    return a.out_dtype == FRG_F32
+               ? launchCompressed<WV, WS, true>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus,
+                                                stream)
+               : launchCompressed<WV, WS, false>(a, raw, wire, Kw, rawPos, head, nvec, tail,
+                                                 numCus, stream);
+  }
+  // element-wise: pointers that cannot be brought to 16-byte boundaries by one
+  // common head, or fewer elements than a group
+  return a.out_dtype == FRG_F32
+             ? launchCompressed<WS, WS, true>(a, raw, wire, Kw, rawPos, 0, a.n, 0, numCus, stream)
+             : launchCompressed<WS, WS, false>(a, raw, wire, Kw, rawPos, 0, a.n, 0, numCus, stream);
+}
+
+}  // namespace
+
+int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::string* err) {
+  auto fail = [&](int code, const std::string& msg) {
+    if (err) *err = msg;
+    return code;
+  };
+  if (a.wire_dtype != FRG_BF16 && a.wire_dtype != FRG_F16) {
+    return fail(FRG_ERR_UNSUPPORTED, "the wire type must be bf16 or fp16");
+  }
+  if (a.out_dtype != FRG_F32 && a.out_dtype != a.wire_dtype) {
+    return fail(FRG_ERR_UNSUPPORTED, "the output must be fp32 or of the wire type");
+  }
+  if (a.K < 1 || a.K > kMaxContribsPerLaunch) {
+    return fail(FRG_ERR_INVALID, "K must be in [1, 64], got " + std::to_string(a.K));
+  }
+  if (a.raw_index < -1 || a.raw_index >= a.K) {
+    return fail(FRG_ERR_INVALID, "raw_index out of range");
+  }
+  if (a.n < 0) return fail(FRG_ERR_INVALID, "negative element count");
+  if (a.scale_mode < FRG_SCALE_NONE || a.scale_mode > FRG_SCALE_DIV) {
+    return fail(FRG_ERR_INVALID, "bad scale mode (NONE, MUL or DIV on the raw contribution)");
+  }
+  if (a.contribs == nullptr) return fail(FRG_ERR_INVALID, "null contribution table");
+  if (a.n == 0) return FRG_OK;
+  if (a.out == nullptr) return fail(FRG_ERR_INVALID, "null output");
+
+  // Every pointer asks for a head h (elements before its first 16-byte
+  // boundary): h mod 8 for a 2-byte type, h mod 4 for fp32. One h must do.
+  const uintptr_t o = reinterpret_cast<uintptr_t>(a.out);
+  const uintptr_t outElsize = a.out_dtype == FRG_F32 ? 4 : 2;
+  if (o % outElsize != 0) return fail(FRG_ERR_INVALID, "output not element-aligned");
+  const uintptr_t outBytes = static_cast<uintptr_t>(a.n) * outElsize;
+  bool vectorOk = true;
+  int64_t headWire = -1, headF32 = -1;
+  auto want = [&](uintptr_t p, uintptr_t elsize) {
+    const int64_t h = static_cast<int64_t>(((16 - (p & 15)) & 15) / elsize);
+    int64_t& slot = elsize == 2 ? headWire : headF32;
+    if (slot < 0) {
+      slot = h;
+    } else if (slot != h) {
+      vectorOk = false;
+    }
+  };
+  want(o, outElsize);
+
+  Ptrs<0> wire;
+  int Kw = 0;
+  const float* raw = nullptr;
+  for (int k = 0; k < a.K; ++k) {
+    const uintptr_t p = reinterpret_cast<uintptr_t>(a.contribs[k]);
+    if (p == 0) return fail(FRG_ERR_INVALID, "null contribution " + std::to_string(k));
+    const uintptr_t elsize = k == a.raw_index ? 4 : 2;
+    if (p % elsize != 0) {
+      return fail(FRG_ERR_INVALID, "contribution " + std::to_string(k) + " not element-aligned");
+    }
+    const uintptr_t bytes = static_cast<uintptr_t>(a.n) * elsize;
+    // the output may be a contribution of its own element size, exactly in place
+    const bool inPlace = p == o && elsize == outElsize;
+    if (!inPlace && p < o + outBytes && o < p + bytes) {
+      return fail(FRG_ERR_INVALID, "output overlaps contribution " + std::to_string(k));
+    }
+    want(p, elsize);
+    if (k == a.raw_index) {
+      raw = static_cast<const float*>(a.contribs[k]);
+    } else {
+      wire.p[Kw++] = a.contribs[k];
+    }
+  }
+  for (int k = Kw; k < kMaxContribsPerLaunch; ++k) wire.p[k] = a.contribs[0];
+  // the own term goes in ahead of wire contribution rawPos
+  const int rawPos = a.raw_index;
+
+  int64_t head = 0, nvec = 0, tail = 0;
+  if (headWire >= 0 && headF32 >= 0 && headWire % 4 != headF32) vectorOk = false;
+  if (vectorOk) {
+    head = headWire >= 0 ? headWire : headF32;
+    if (head > a.n) head = a.n;
+    nvec = (a.n - head) / 8;
+    tail = a.n - head - nvec * 8;
+  }
+
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return fail(FRG_ERR_HIP, "hipGetDevice failed");
+  const int numCus = computeUnits(device);
+  hipError_t e;
+  if (a.wire_dtype == FRG_BF16) {
+    e = dispatchOut<Bf16Vec, Bf16Scalar>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus, stream);
+  } else {
+    e = dispatchOut<F16Vec, F16Scalar>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus, stream);
+  }
+  if (e != hipSuccess) {
+    return fail(FRG_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString(e));
+  }
+  return FRG_OK;
+}
+
+}  // namespace frg

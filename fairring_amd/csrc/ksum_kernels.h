@@ -38,4 +38,35 @@ int launchReduce(const ReduceArgs& args, hipStream_t stream, std::string* err);
 // Launch-shape knobs (process-wide); 0 keeps the default.
 void setTuning(int blocksPerCu);
 
+// Compute units of a device (cached).
+int computeUnits(int device);
+
+// The persistent grid for `nvec` 16-byte vectors per contribution: `grid`
+// blocks, `roundTiles` full tiles dealt in whole rounds of the grid, and what
+// is left dealt in `pieces` smaller pieces.
+struct GridPlan {
+  int64_t grid = 1;
+  int64_t roundTiles = 0;
+  int64_t pieces = 0;
+};
+GridPlan planGrid(int64_t nvec, int numContribs, int numCus);
+
+// The reduction around torch's gradient-compression hooks: peers' tensors in
+// the wire type (bf16 or fp16), this rank's own fp32 buffer compressed in
+// registers, the result stored in the wire type or widened into fp32.
+struct CompressedArgs {
+  void* out = nullptr;
+  int out_dtype = 0;                      // FRG_F32 or the wire dtype
+  const void* const* contribs = nullptr;  // host array of K device pointers
+  int K = 0;
+  int raw_index = -1;  // which contribution is raw fp32 (-1: none)
+  int64_t n = 0;
+  int wire_dtype = 0;  // FRG_BF16 / FRG_F16
+  int scale_mode = 0;  // applied to the raw contribution after the cast: NONE / MUL / DIV
+  float scale = 1.0f;
+  hipEvent_t startEvent = nullptr;
+  hipEvent_t stopEvent = nullptr;
+};
+int launchCompressedReduce(const CompressedArgs& args, hipStream_t stream, std::string* err);
+
 }  // namespace frg

@@ -295,16 +295,44 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     return FRG_ERR_INVALID;
   }
   if (req.op == FRG_MAX && req.scaleMode != FRG_SCALE_NONE) {
-    *err = "MAX takes no post-scale";
+    *err = "MAX takes no scale";
     return FRG_ERR_INVALID;
   }
-  if (req.scaleMode < FRG_SCALE_NONE || req.scaleMode > FRG_SCALE_DIV) {
+  if (req.scaleMode < FRG_SCALE_NONE || req.scaleMode > FRG_SCALE_PRE_DIV) {
     *err = "bad scale mode";
     return FRG_ERR_INVALID;
   }
   if (req.scaleMode != FRG_SCALE_NONE && !isFloating(req.dtype)) {
-    *err = "integer types take no post-scale";
+    *err = "integer types take no scale";
     return FRG_ERR_INVALID;
+  }
+  if (req.fromHost && req.scaleMode >= FRG_SCALE_PRE_MUL) {
+    // a server does not rescale what the machines deliver
+    *err = "host-staged contributions take no pre-scale";
+    return FRG_ERR_UNSUPPORTED;
+  }
+  if (req.compressed) {
+    if (req.dtype != FRG_BF16 && req.dtype != FRG_F16) {
+      *err = "the wire type must be bf16 or fp16";
+      return FRG_ERR_UNSUPPORTED;
+    }
+    if (req.outDtype != FRG_F32 && req.outDtype != req.dtype) {
+      *err = "the output must be fp32 or of the wire type";
+      return FRG_ERR_UNSUPPORTED;
+    }
+    if (req.scaleMode > FRG_SCALE_DIV) {
+      *err = "bad scale mode (NONE, MUL or DIV on the raw contribution)";
+      return FRG_ERR_INVALID;
+    }
+    const int K = static_cast<int>(req.contribs.size());
+    if (K > kMaxContribsPerLaunch) {
+      *err = "at most 64 contributions with compression folded in";
+      return FRG_ERR_INVALID;
+    }
+    if (req.rawIndex < -1 || req.rawIndex >= K) {
+      *err = "raw_index out of range";
+      return FRG_ERR_INVALID;
+    }
   }
   if (kAlignment % elementSize(req.dtype) != 0) {  // fairring/device.cc:316
     *err = "element size must divide 8";
@@ -377,6 +405,37 @@ void Context::launch(const ReduceArgs& args, hipStream_t stream) {
   if (rc != FRG_OK) throw ContractFailure(rc, err);
 }
 
+void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
+  CompressedArgs a = args;
+  const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
+  if (prof) {
+    FRG_HIP_CHECK(hipEventCreate(&a.startEvent));
+    FRG_HIP_CHECK(hipEventCreate(&a.stopEvent));
+  }
+  std::string err;
+  const int rc = launchCompressedReduce(a, stream, &err);
+  if (rc == FRG_OK && args.n > 0) {
+    for (size_t i = 0; i < reduceStreams_.size(); ++i) {
+      if (reduceStreams_[i] == stream) {
+        streamLaunches_[i] += 1;
+        streamElems_[i] += args.n;
+      }
+    }
+    lastContribs_ = args.K;
+  }
+  if (prof) {
+    if (rc == FRG_OK) {
+      std::lock_guard<std::mutex> g(profMu_);
+      profEvents_.push_back(ProfRecord{a.startEvent, a.stopEvent, a.n, a.K, stream, 1});
+    } else {
+      (void)hipEventDestroy(a.startEvent);
+      (void)hipEventDestroy(a.stopEvent);
+    }
+  }
+  if (rc == FRG_ERR_HIP) throw HipFailure(err);
+  if (rc != FRG_OK) throw ContractFailure(rc, err);
+}
+
 // Device-resident contributions: every slice (the slicing of
 // fairring/device.cc:315-326) is reduced by one launch, or by several when it
 // is larger than the launch size; launches are dealt round-robin to the reduce
@@ -409,7 +468,8 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     int64_t sliceOff, sliceLen;
     sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &sliceOff, &sliceLen);
     nextStagingSlot_++;  // a slice still takes its turn in the slot rotation (device.cc:482)
-    if (total == 1 && req.contribs[0] == req.out && req.scaleMode == FRG_SCALE_NONE) {
+    if (!req.compressed && total == 1 && req.contribs[0] == req.out &&
+        req.scaleMode == FRG_SCALE_NONE) {
       // A lone contribution reduced in place is the identity (what the
       // reference does for one machine and one device: device.cc:523,569).
       continue;
@@ -443,7 +503,23 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
         waited[si] = 1;
       }
       for (size_t k = 0; k < ptrs.size(); ++k) {
-        ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * elsize;
+        const int64_t es = (req.compressed && static_cast<int>(k) == req.rawIndex) ? 4 : elsize;
+        ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * es;
+      }
+      if (req.compressed) {
+        CompressedArgs a;
+        a.out = static_cast<char*>(req.out) + off * elementSize(req.outDtype);
+        a.out_dtype = req.outDtype;
+        a.contribs = ptrs.data();
+        a.K = total;
+        a.raw_index = req.rawIndex;
+        a.n = len;
+        a.wire_dtype = req.dtype;
+        a.scale_mode = req.scaleMode;
+        a.scale = req.scale;
+        launchCompressed(a, s);
+        lastIdx = si;
+        continue;
       }
       // More contributions than one launch takes: chain launches, carrying the
       // partial result in `out`; the post-scale goes on the last one only.
@@ -457,7 +533,9 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
         a.n = len;
         a.dtype = req.dtype;
         a.op = req.op;
-        a.scale_mode = lastLaunch ? req.scaleMode : FRG_SCALE_NONE;
+        // a post-scale goes on the last launch only, a pre-scale on every one
+        a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
+                                                                          : FRG_SCALE_NONE;
         a.scale = req.scale;
         a.carry = k0 > 0;
         launch(a, s);

@@ -75,6 +75,11 @@ class Context {
     float scale = 1.0f;
     bool fromHost = false;
     bool carry = false;  // host-staged only: `out` already holds the first term
+    // Compression hooks folded in: `dtype` is the wire type, contribution
+    // `rawIndex` is raw fp32, the output is of `outDtype`.
+    bool compressed = false;
+    int outDtype = FRG_F32;
+    int rawIndex = -1;
     hipStream_t producerStream = nullptr;
     frg_done_fn done = nullptr;
     void* user = nullptr;
@@ -108,6 +113,7 @@ class Context {
   // Makes `stream` wait for `initialEvent` unless that event has already fired.
   void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
   void launch(const struct ReduceArgs& args, hipStream_t stream);
+  void launchCompressed(const struct CompressedArgs& args, hipStream_t stream);
   hipEvent_t takeEvent();
   void giveEvent(hipEvent_t e);
 

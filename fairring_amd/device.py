@@ -11,7 +11,7 @@ import sys
 
 from . import _capi
 from ._capi import (BF16, F16, F32, F64, I8, I32, I64, MAX, SCALE_DIV, SCALE_MUL,
-                    SCALE_NONE, SUM, U8, FairringError)
+                    SCALE_NONE, SCALE_PRE_DIV, SCALE_PRE_MUL, SUM, U8, FairringError)
 
 MiB = 1024 * 1024
 
@@ -101,6 +101,52 @@ def reduce_slice(out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, carry=
         scale, 1 if carry else 0, stream.cuda_stream))
 
 
+def _check_compressed(out, contribs, raw_index):
+    """Shapes and types of the reduction with compression folded in; returns
+    the wire dtype code."""
+    import torch
+    if not -1 <= raw_index < len(contribs):
+        raise FairringError(_capi.ERR_INVALID, "raw_index out of range")
+    wire = None
+    for k, c in enumerate(contribs):
+        if c.numel() != out.numel():
+            raise FairringError(_capi.ERR_INVALID, "contribution shape mismatch")
+        if k == raw_index:
+            if c.dtype != torch.float32:
+                raise FairringError(_capi.ERR_INVALID, "the raw contribution must be float32")
+        elif wire is None:
+            wire = c.dtype
+        elif c.dtype != wire:
+            raise FairringError(_capi.ERR_INVALID, "peers' contributions differ in dtype")
+    if wire is None:
+        wire = out.dtype if out.dtype != torch.float32 else torch.bfloat16
+    if wire not in (torch.bfloat16, torch.float16):
+        raise FairringError(_capi.ERR_UNSUPPORTED, "the wire type must be bfloat16 or float16")
+    if out.dtype not in (torch.float32, wire):
+        raise FairringError(_capi.ERR_UNSUPPORTED, "the output must be float32 or of the wire type")
+    return BF16 if wire == torch.bfloat16 else F16
+
+
+def reduce_slice_compressed(out, contribs, raw_index=-1, scale_mode=SCALE_NONE, scale=1.0,
+                            wire_dtype=None, stream=None):
+    """One launch of the reduction with torch's bf16 / fp16 compression hooks
+    folded in (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:57-93):
+    contribs[raw_index] is this rank's float32 bucket, cast to the wire type and
+    scaled there in registers; the others are peers' tensors in the wire type;
+    `out` is of the wire type, or float32 to receive the result widened (it may
+    be the raw bucket itself). `wire_dtype` is only needed when there is no
+    peer tensor to take it from."""
+    import torch
+    stream = torch.cuda.current_stream(out.device) if stream is None else stream
+    wire = _check_compressed(out, contribs, raw_index)
+    if wire_dtype is not None:
+        wire = BF16 if wire_dtype == torch.bfloat16 else F16
+    tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+    _capi.check(_capi.lib().frg_reduce_slice_compressed(
+        out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index, out.numel(), wire,
+        scale_mode, scale, stream.cuda_stream))
+
+
 class Work:
     """Handle on a submitted operation (WorkFairring, process_group.cc:35-75)."""
 
@@ -180,6 +226,26 @@ class DeviceFairring:
         for c in contribs:
             _check_dense(c, "contribution")
         return self._submit(out, contribs, op, scale_mode, scale, stream, host=False)
+
+    def allreduce_compressed(self, out, contribs, raw_index=-1, scale_mode=SCALE_NONE, scale=1.0,
+                             wire_dtype=None, stream=None):
+        """reduce_slice_compressed through the slice pipeline (sliced by the
+        wire type's element size). Returns at once."""
+        import torch
+        _check_dense(out, "output")
+        for c in contribs:
+            _check_dense(c, "contribution")
+        wire = _check_compressed(out, contribs, raw_index)
+        if wire_dtype is not None:
+            wire = BF16 if wire_dtype == torch.bfloat16 else F16
+        stream = torch.cuda.current_stream(out.device) if stream is None else stream
+        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        wh = ctypes.c_void_p()
+        _capi.check(_capi.lib().frg_allreduce_compressed(
+            self._h, out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index,
+            out.numel(), wire, scale_mode, scale, stream.cuda_stream, _capi.DONE_FN(), None,
+            ctypes.byref(wh)))
+        return Work(wh, (out, list(contribs)))
 
     def allreduce_host(self, out, host_contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0,
                        carry=False, stream=None):

@@ -50,12 +50,21 @@ enum {
 /* reduction ops accepted by MachineFairring::allReduce (machine.cc:181) */
 enum { FRG_SUM = 0, FRG_MAX = 1 };
 
-/* fused post-scale applied once to the accumulated value before the store */
+/* Fused scale, floating-point types only. The post-scales are applied once to
+ * the accumulated value before the store. The pre-scales are applied to every
+ * contribution before it is folded in, each product rounded to the storage
+ * type, which is bit for bit what DDP leaves in every rank's bucket ahead of
+ * the allreduce (tensor.div_(world) in torch's allreduce_hook,
+ * torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:18-32; the
+ * reducer's own mul_out by 1/world when no hook is registered). ATen divides
+ * by a scalar as written on the CPU and multiplies by its reciprocal on the
+ * GPU: DIV and MUL exist for both. A carried-in term is never pre-scaled. */
 enum {
-  /* floating-point types only */
-  FRG_SCALE_NONE = 0, /* out = acc                                     */
-  FRG_SCALE_MUL = 1,  /* out = acc * scale  (scale = 1/K; exact for K = 2^p) */
-  FRG_SCALE_DIV = 2   /* out = acc / scale  (scale = K; IEEE division, at::div) */
+  FRG_SCALE_NONE = 0,    /* out = acc                                     */
+  FRG_SCALE_MUL = 1,     /* out = acc * scale  (scale = 1/K; exact for K = 2^p) */
+  FRG_SCALE_DIV = 2,     /* out = acc / scale  (scale = K; IEEE division, at::div) */
+  FRG_SCALE_PRE_MUL = 3, /* term k = x[k] * scale, then the fold */
+  FRG_SCALE_PRE_DIV = 4  /* term k = x[k] / scale, then the fold */
 };
 
 /* ---- layout and slicing (pure integer functions, no GPU) ---------------- */
@@ -100,6 +109,24 @@ FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
 FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);
+
+/* The same reduction with torch's gradient-compression hooks folded in
+ * (bf16_compress_hook / fp16_compress_hook,
+ * torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:57-134, wrapped
+ * around the allreduce of fairring/process_group.cc:131-155). `wire_dtype` is
+ * FRG_BF16 or FRG_F16. contribs[raw_index] (raw_index -1: none) is this rank's
+ * own fp32 bucket: it is cast to the wire type and scaled there
+ * (FRG_SCALE_MUL: * scale, FRG_SCALE_DIV: / scale, each rounded to the wire
+ * type; FRG_SCALE_NONE: the cast alone), in registers. Every other contribution
+ * is a peer's tensor already in the wire type. The fold runs in fp32 in
+ * contribution order with one rounding to the wire type. `out_dtype` is the
+ * wire type, or FRG_F32 to store the result widened (the hook's decompress
+ * step); `out` may be the raw contribution itself (the bucket, in place).
+ * K <= 64. Per element 4 + 2 (K - 1) + 4 bytes cross HBM instead of the
+ * 14 + 2 K of the three separate passes. */
+FRG_API int frg_reduce_slice_compressed(void* out, int out_dtype, const void* const* contribs,
+                                        int K, int raw_index, int64_t n, int wire_dtype,
+                                        int scale_mode, float scale, void* stream);
 
 /* ---- the per-GPU slice pipeline ----------------------------------------- */
 
@@ -161,6 +188,15 @@ FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
                           int K, int64_t numel, int dtype, int op,
                           int scale_mode, float scale, void* producer_stream,
                           frg_done_fn done, void* user, frg_work** work);
+
+/* frg_reduce_slice_compressed through the pipeline: sliced by the wire type's
+ * element size (the tensor the reference would be handed is the compressed
+ * one), launches dealt to the reduce streams like frg_allreduce's. */
+FRG_API int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype,
+                                     const void* const* contribs, int K, int raw_index,
+                                     int64_t numel, int wire_dtype, int scale_mode, float scale,
+                                     void* producer_stream, frg_done_fn done, void* user,
+                                     frg_work** work);
 
 /* Server-side accumulation with contributions in pinned host memory
  * (device.cc:543-589: collect into a staging slot, then reduce): contribution

@@ -19,6 +19,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 SCALE_NONE, SCALE_MUL, SCALE_DIV = 0, 1, 2
+SCALE_PRE_MUL, SCALE_PRE_DIV = 3, 4  # every contribution scaled (and rounded) before the fold
 
 _lib = None
 
@@ -48,6 +49,8 @@ def lib():
                      "orc_sum_u8", "orc_max_u8", "orc_sum_i8", "orc_max_i8"):
             getattr(L, name).argtypes = [vp, vp, i32, i64]
             getattr(L, name).restype = None
+        L.orc_compressed_sum.argtypes = [vp, i32, vp, i32, i32, i64, i32, i32, f32]
+        L.orc_compressed_sum.restype = None
         L.orc_ceil_of_ratio.argtypes = [i64, i64]
         L.orc_ceil_of_ratio.restype = i64
         L.orc_round_down.argtypes = [i64, i64]
@@ -135,6 +138,27 @@ def reduce(kind, contribs, op="sum", scale_mode=SCALE_NONE, scale=1.0):
     else:
         assert scale_mode == SCALE_NONE
         fn(out.ctypes.data, _ptr_table(arrs), len(arrs), n)
+    return out
+
+
+def compressed_sum(contribs, raw_index, wire="bf16", scale_mode=SCALE_NONE, scale=1.0,
+                   out_f32=True, threads=1):
+    """torch's compress hook + allreduce + decompress for one rank's bucket.
+
+    contribs[raw_index] is this rank's float32 buffer (raw_index -1: none), the
+    others are uint16 arrays of wire-type bit patterns. Returns float32 (the
+    decompressed bucket) or uint16 wire bits."""
+    arrs = []
+    for k, c in enumerate(contribs):
+        dt = np.float32 if k == raw_index else np.uint16
+        arrs.append(np.ascontiguousarray(c, dtype=dt).reshape(-1))
+    n = arrs[0].size
+    assert all(a.size == n for a in arrs)
+    out = np.empty(n, np.float32 if out_f32 else np.uint16)
+    L = lib()
+    L.orc_set_threads(threads)
+    L.orc_compressed_sum(out.ctypes.data, 1 if out_f32 else 0, _ptr_table(arrs), len(arrs),
+                         raw_index, n, {"bf16": 0, "f16": 1}[wire], scale_mode, scale)
     return out
 
 

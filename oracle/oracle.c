@@ -17,6 +17,11 @@
  *   orc_readme_layout                        -> README.md:61-62 (the
  *       FAIRRING_TOTAL_MEMORY / FAIRRING_SLICE_SIZE pair)
  *
+ *   orc_compressed_sum and the PRE_MUL / PRE_DIV scale modes follow torch's DDP
+ *       hooks on either side of the allreduce the reference serves
+ *       (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:18-93);
+ *       pinned against those very expressions run by the installed torch.
+ *
  * Pinned by (see tests/test_oracle.py): the installed ATen's add chain and
  * sum(dim=0) (K <= 17) bit for bit, ATen's bf16 sum over dim 0, an exact
  * rational-arithmetic brute force with explicit round-to-nearest-even on tiny
@@ -32,6 +37,11 @@
 #define ORC_SCALE_NONE 0 /* out = acc */
 #define ORC_SCALE_MUL 1  /* out = acc * scale   (scale = 1/K, exact for K=2^p) */
 #define ORC_SCALE_DIV 2  /* out = acc / scale   (scale = K, at::div semantics) */
+/* Pre-scale: every contribution is scaled, and rounded to its storage type,
+ * before the fold; what DDP does to each rank's bucket ahead of the
+ * allreduce (tensor.div_(world) in torch's allreduce_hook). */
+#define ORC_SCALE_PRE_MUL 3 /* term = x[k] * scale */
+#define ORC_SCALE_PRE_DIV 4 /* term = x[k] / scale */
 
 static inline float apply_scale(float acc, int mode, float scale) {
   if (mode == ORC_SCALE_MUL) return acc * scale;
@@ -39,13 +49,19 @@ static inline float apply_scale(float acc, int mode, float scale) {
   return acc;
 }
 
+static inline float pre_scale(float x, int mode, float scale) {
+  if (mode == ORC_SCALE_PRE_MUL) return x * scale;
+  if (mode == ORC_SCALE_PRE_DIV) return x / scale;
+  return x;
+}
+
 /* fp32: left fold in contribution order starting from x[0] (not from 0). */
 void orc_sum_f32(float* out, const float* const* in, int K, int64_t n,
                  int scale_mode, float scale) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
-    float acc = in[0][i];
-    for (int k = 1; k < K; ++k) acc = acc + in[k][i];
+    float acc = pre_scale(in[0][i], scale_mode, scale);
+    for (int k = 1; k < K; ++k) acc = acc + pre_scale(in[k][i], scale_mode, scale);
     out[i] = apply_scale(acc, scale_mode, scale);
   }
 }
@@ -61,10 +77,11 @@ void orc_sum_f32_chain(float* out, const float* const* in, int K, int64_t n,
 #pragma omp for schedule(static)
     for (int64_t b = 0; b < (n + B - 1) / B; ++b) {
       int64_t lo = b * B, hi = lo + B < n ? lo + B : n;
-      for (int64_t i = lo; i < hi; ++i) out[i] = in[0][i];
+      for (int64_t i = lo; i < hi; ++i) out[i] = pre_scale(in[0][i], scale_mode, scale);
       for (int k = 1; k < K; ++k)
-        for (int64_t i = lo; i < hi; ++i) out[i] = out[i] + in[k][i];
-      if (scale_mode != ORC_SCALE_NONE)
+        for (int64_t i = lo; i < hi; ++i)
+          out[i] = out[i] + pre_scale(in[k][i], scale_mode, scale);
+      if (scale_mode == ORC_SCALE_MUL || scale_mode == ORC_SCALE_DIV)
         for (int64_t i = lo; i < hi; ++i)
           out[i] = apply_scale(out[i], scale_mode, scale);
     }
@@ -93,8 +110,14 @@ void orc_sum_bf16(uint16_t* out, const uint16_t* const* in, int K, int64_t n,
                   int scale_mode, float scale) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
-    float acc = bf16_to_f32(in[0][i]);
-    for (int k = 1; k < K; ++k) acc = acc + bf16_to_f32(in[k][i]);
+    const int pre = scale_mode >= ORC_SCALE_PRE_MUL;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) {
+      float t = bf16_to_f32(in[k][i]);
+      /* a pre-scaled term is a bf16 tensor of its own: rounded before the fold */
+      if (pre) t = bf16_to_f32(f32_to_bf16_rne(pre_scale(t, scale_mode, scale)));
+      acc = k == 0 ? t : acc + t;
+    }
     out[i] = f32_to_bf16_rne(apply_scale(acc, scale_mode, scale));
   }
 }
@@ -256,8 +279,13 @@ void orc_sum_f16(uint16_t* out, const uint16_t* const* in, int K, int64_t n, int
                  float scale) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
-    float acc = f16_to_f32(in[0][i]);
-    for (int k = 1; k < K; ++k) acc = acc + f16_to_f32(in[k][i]);
+    const int pre = scale_mode >= ORC_SCALE_PRE_MUL;
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) {
+      float t = f16_to_f32(in[k][i]);
+      if (pre) t = f16_to_f32(f32_to_f16_rne(pre_scale(t, scale_mode, scale)));
+      acc = k == 0 ? t : acc + t;
+    }
     out[i] = f32_to_f16_rne(apply_scale(acc, scale_mode, scale));
   }
 }
@@ -274,8 +302,13 @@ void orc_sum_f64(double* out, const double* const* in, int K, int64_t n, int sca
                  float scale) {
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) {
-    double acc = in[0][i];
-    for (int k = 1; k < K; ++k) acc = acc + in[k][i];
+    double acc = 0.0;
+    for (int k = 0; k < K; ++k) {
+      double t = in[k][i];
+      if (scale_mode == ORC_SCALE_PRE_MUL) t = t * (double)scale;
+      if (scale_mode == ORC_SCALE_PRE_DIV) t = t / (double)scale;
+      acc = k == 0 ? t : acc + t;
+    }
     if (scale_mode == ORC_SCALE_MUL) acc = acc * (double)scale;
     if (scale_mode == ORC_SCALE_DIV) acc = acc / (double)scale;
     out[i] = acc;
@@ -313,3 +346,48 @@ ORC_INT_REDUCE(i32, int32_t, uint32_t)
 ORC_INT_REDUCE(i64, int64_t, uint64_t)
 ORC_INT_REDUCE(u8, uint8_t, uint8_t)
 ORC_INT_REDUCE(i8, int8_t, uint8_t)
+
+/* ---- gradient compression around the reduction ---------------------------
+ * What torch's bf16/fp16 compress hooks do on every rank on either side of the
+ * allreduce that fairring/process_group.cc:131-155 serves
+ * (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:57-93):
+ *   compressed = buffer.to(wire).div_(world)      -- two roundings to wire
+ *   allreduce(compressed)                         -- fp32 fold, one rounding
+ *   buffer.copy_(result)                          -- exact widening
+ * Contribution raw_index (if >= 0) is this rank's fp32 buffer and goes through
+ * the compress step here; the others are peers' tensors, already in the wire
+ * type. scale_mode MUL computes x * scale (ATen on the GPU multiplies by the
+ * reciprocal of a scalar divisor), DIV computes x / scale (ATen on the CPU).
+ * wire: 0 = bf16, 1 = fp16. out_f32: store the result widened to fp32. */
+static inline float wire_to_f32(uint16_t w, int wire) {
+  return wire ? f16_to_f32(w) : bf16_to_f32(w);
+}
+
+static inline uint16_t f32_to_wire(float f, int wire) {
+  return wire ? f32_to_f16_rne(f) : f32_to_bf16_rne(f);
+}
+
+void orc_compressed_sum(void* out, int out_f32, const void* const* in, int K, int raw_index,
+                        int64_t n, int wire, int scale_mode, float scale) {
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = 0.0f;
+    for (int k = 0; k < K; ++k) {
+      float t;
+      if (k == raw_index) {
+        const float x = ((const float*)in[k])[i];
+        const float cast = wire_to_f32(f32_to_wire(x, wire), wire);
+        t = wire_to_f32(f32_to_wire(apply_scale(cast, scale_mode, scale), wire), wire);
+      } else {
+        t = wire_to_f32(((const uint16_t*)in[k])[i], wire);
+      }
+      acc = k == 0 ? t : acc + t;
+    }
+    const uint16_t r = f32_to_wire(acc, wire);
+    if (out_f32) {
+      ((float*)out)[i] = wire_to_f32(r, wire);
+    } else {
+      ((uint16_t*)out)[i] = r;
+    }
+  }
+}

@@ -2,9 +2,11 @@
 // pipeline is compiled against the fake HIP runtime. The "kernel" is a plain
 // fp32 fold run as one unit of work on the fake stream, so the choreography
 // around it (ordering, slot reuse, carry chains) decides whether results come
-// out right. fp32 only.
+// out right. fp32 only, plus a bf16 stand-in of the reduction with compression
+// folded in.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <vector>
 
 #include "../../fairring_amd/csrc/ksum_kernels.h"
@@ -52,10 +54,15 @@ struct Job {
 void runJob(void* p) {
   Job* j = static_cast<Job*>(p);
   for (int64_t i = 0; i < j->n; ++i) {
+    const bool preMul = j->scaleMode == FRG_SCALE_PRE_MUL, preDiv = j->scaleMode == FRG_SCALE_PRE_DIV;
+    auto term = [&](size_t kk) {
+      const float x = j->in[kk][i];
+      return preMul ? x * j->scale : (preDiv ? x / j->scale : x);
+    };
     size_t k = 0;
-    float acc = j->carry ? j->out[i] : j->in[k++][i];
+    float acc = j->carry ? j->out[i] : term(k++);
     for (; k < j->in.size(); ++k) {
-      const float b = j->in[k][i];
+      const float b = term(k);
       if (j->op == FRG_SUM) {
         acc = acc + b;
       } else {
@@ -69,7 +76,71 @@ void runJob(void* p) {
   delete j;
 }
 
+// bf16 helpers of the compressed stand-in
+float widen(uint16_t b) {
+  const uint32_t u = static_cast<uint32_t>(b) << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+uint16_t narrow(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+  return static_cast<uint16_t>((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+struct CompressedJob {
+  void* out;
+  bool out32;
+  std::vector<const void*> in;
+  int rawIndex;
+  int64_t n;
+  int scaleMode;
+  float scale;
+};
+
+void runCompressedJob(void* p) {
+  CompressedJob* j = static_cast<CompressedJob*>(p);
+  for (int64_t i = 0; i < j->n; ++i) {
+    float acc = 0.0f;
+    for (size_t k = 0; k < j->in.size(); ++k) {
+      float t;
+      if (static_cast<int>(k) == j->rawIndex) {
+        t = widen(narrow(static_cast<const float*>(j->in[k])[i]));
+        if (j->scaleMode == FRG_SCALE_MUL) t = widen(narrow(t * j->scale));
+        if (j->scaleMode == FRG_SCALE_DIV) t = widen(narrow(t / j->scale));
+      } else {
+        t = widen(static_cast<const uint16_t*>(j->in[k])[i]);
+      }
+      acc = k == 0 ? t : acc + t;
+    }
+    if (j->out32) {
+      static_cast<float*>(j->out)[i] = widen(narrow(acc));
+    } else {
+      static_cast<uint16_t*>(j->out)[i] = narrow(acc);
+    }
+  }
+  delete j;
+}
+
 }  // namespace
+
+int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::string* err) {
+  auto fail = [&](int code, const char* msg) {
+    if (err) *err = msg;
+    return code;
+  };
+  if (a.wire_dtype != FRG_BF16) return fail(FRG_ERR_UNSUPPORTED, "host test build: bf16 wire only");
+  if (a.K < 1 || a.K > kMaxContribsPerLaunch) return fail(FRG_ERR_INVALID, "K out of range");
+  if (a.n == 0) return FRG_OK;
+  CompressedJob* j = new CompressedJob{a.out, a.out_dtype == FRG_F32, {}, a.raw_index,
+                                       a.n,   a.scale_mode,          a.scale};
+  for (int k = 0; k < a.K; ++k) j->in.push_back(a.contribs[k]);
+  fake_hip_enqueue(stream, &runCompressedJob, j);
+  return FRG_OK;
+}
 
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   auto fail = [&](int code, const char* msg) {

@@ -42,9 +42,14 @@ std::vector<Vec> randomContribs(int k, int64_t n, unsigned seed) {
 Vec fold(const std::vector<Vec>& c, int scaleMode, float scale, const Vec* carry = nullptr) {
   Vec out(c[0].size());
   for (size_t i = 0; i < out.size(); ++i) {
+    auto term = [&](size_t kk) {
+      const float x = c[kk][i];
+      return scaleMode == FRG_SCALE_PRE_MUL ? x * scale
+                                            : (scaleMode == FRG_SCALE_PRE_DIV ? x / scale : x);
+    };
     size_t k = 0;
-    float acc = carry ? (*carry)[i] : c[k++][i];
-    for (; k < c.size(); ++k) acc = acc + c[k][i];
+    float acc = carry ? (*carry)[i] : term(k++);
+    for (; k < c.size(); ++k) acc = acc + term(k);
     if (scaleMode == FRG_SCALE_MUL) acc = acc * scale;
     if (scaleMode == FRG_SCALE_DIV) acc = acc / scale;
     out[i] = acc;
@@ -100,6 +105,76 @@ void scenarioResident() {
       CHECK(frg_destroy(ctx) == FRG_OK);
     }
   }
+}
+
+float widenBf16(uint16_t b) {
+  const uint32_t u = static_cast<uint32_t>(b) << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+uint16_t narrowBf16(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+  return static_cast<uint16_t>((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+void scenarioPreScaleAndCompressed() {
+  std::puts("pre-scaled chains and the compressed reduction: offsets per element size");
+  frg_ctx* ctx = makeCtx(16384, 4096, 2, 1024);
+  frg_work* w = nullptr;
+  // a pre-scale goes on every launch of a chain, never on the carried term
+  auto big = randomContribs(150, 3001, 21);
+  Vec out(3001);
+  auto t = table(big);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 150, 3001, FRG_F32, FRG_SUM, FRG_SCALE_PRE_DIV,
+                      150.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  CHECK(same(out, fold(big, FRG_SCALE_PRE_DIV, 150.f)));
+  frg_work_release(w);
+  CHECK(frg_allreduce_host(ctx, out.data(), t.data(), 3, 3001, FRG_F32, FRG_SUM,
+                           FRG_SCALE_PRE_MUL, .5f, 0, nullptr, nullptr, nullptr,
+                           nullptr) == FRG_ERR_UNSUPPORTED);
+  // compressed: 5 contributions, the raw fp32 one third in the chain, reduced in place into it;
+  // slices are 2048 wire elements, so the fp32 side advances by 8 KiB per slice
+  const int64_t n = 10007;
+  const int K = 5, rawIndex = 2;
+  auto raw = randomContribs(1, n, 22)[0];
+  std::vector<std::vector<uint16_t>> peers(K, std::vector<uint16_t>(static_cast<size_t>(n)));
+  auto src = randomContribs(K, n, 23);
+  for (int k = 0; k < K; ++k) {
+    for (int64_t i = 0; i < n; ++i) peers[k][i] = narrowBf16(src[k][i]);
+  }
+  Vec want(static_cast<size_t>(n));
+  for (int64_t i = 0; i < n; ++i) {
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) {
+      float term = k == rawIndex ? widenBf16(narrowBf16(widenBf16(narrowBf16(raw[i])) * 0.2f))
+                                 : widenBf16(peers[k][i]);
+      acc = k == 0 ? term : acc + term;
+    }
+    want[i] = widenBf16(narrowBf16(acc));
+  }
+  std::vector<const void*> tab;
+  for (int k = 0; k < K; ++k) tab.push_back(k == rawIndex ? (const void*)raw.data() : peers[k].data());
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, rawIndex, n, FRG_BF16,
+                                 FRG_SCALE_MUL, 0.2f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  CHECK(same(raw, want));
+  frg_work_release(w);
+  // contract violations of the compressed entry point
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, 7, n, FRG_BF16, 0, 1.f,
+                                 nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, rawIndex, n, FRG_F32, 0,
+                                 1.f, nullptr, nullptr, nullptr, nullptr) == FRG_ERR_UNSUPPORTED);
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F64, tab.data(), K, rawIndex, n, FRG_BF16, 0,
+                                 1.f, nullptr, nullptr, nullptr, nullptr) == FRG_ERR_UNSUPPORTED);
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, rawIndex, n, FRG_BF16,
+                                 FRG_SCALE_PRE_MUL, 1.f, nullptr, nullptr, nullptr,
+                                 nullptr) == FRG_ERR_INVALID);
+  CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
 void scenarioBusyProducer() {
@@ -353,6 +428,7 @@ void scenarioConcurrentSubmitters() {
 
 int main() {
   scenarioResident();
+  scenarioPreScaleAndCompressed();
   scenarioBusyProducer();
   scenarioProducerOrdering();
   scenarioHostStaged();

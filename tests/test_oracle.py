@@ -247,6 +247,105 @@ def test_f64_and_integer_types_vs_numpy_and_aten():
     assert (m == d.max(axis=0)).all()
 
 
+# ---- DDP hook arithmetic on either side of the reduction ---------------------------------
+# Pinned against the very expressions of torch's hooks
+# (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:18-93) run by the installed torch.
+
+def _wide_f32(rng, shape):
+    x = (rng.standard_normal(shape) * np.exp(rng.uniform(-30, 30, shape))).astype(np.float32)
+    x.reshape(-1)[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-42]   # special lanes, a subnormal
+    return x
+
+
+@pytest.mark.parametrize("world", [2, 3, 6, 7, 8, 48])
+def test_pre_scale_matches_torch_allreduce_hook(world):
+    rng = np.random.default_rng(300 + world)
+    x = _wide_f32(rng, (world, 4099))
+    # allreduce_hook: every rank runs tensor.div_(world) on its bucket, then the buckets are summed
+    terms = [torch.from_numpy(r.copy()).div_(world) for r in x]
+    acc = terms[0].clone()
+    for t in terms[1:]:
+        acc = torch.add(acc, t)
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_PRE_DIV, float(world)), acc.numpy(),
+                      "fp32 pre-div")
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_PRE_DIV, float(world), chain=True,
+                                     threads=3), acc.numpy(), "fp32 pre-div, blocked chain")
+    # ATen on the GPU multiplies by the reciprocal of a scalar divisor instead
+    s = np.float32(1) / np.float32(world)
+    terms = [torch.from_numpy(r.copy()).mul_(torch.tensor(s)) for r in x]
+    acc = terms[0].clone()
+    for t in terms[1:]:
+        acc = torch.add(acc, t)
+    assert_bits_equal(oracle.sum_f32(list(x), oracle.SCALE_PRE_MUL, float(s)), acc.numpy(),
+                      "fp32 pre-mul")
+    # half types: the scaled bucket is a tensor of the half type, so every term is rounded
+    for kind, dt in (("bf16", torch.bfloat16), ("f16", torch.float16)):
+        h = [torch.from_numpy(r.copy()).to(dt) for r in x]
+        bits = [t.view(torch.int16).numpy().view(np.uint16) for t in h]
+        terms = [t.clone().div_(world) for t in h]
+        acc = terms[0].float()
+        for t in terms[1:]:
+            acc = acc + t.float()
+        want = acc.to(dt).view(torch.int16).numpy().view(np.uint16)
+        got = oracle.reduce(kind, bits, "sum", oracle.SCALE_PRE_DIV, float(world))
+        assert_bits_equal(got, want, kind + " pre-div", half=True)
+    d = x.astype(np.float64)
+    with np.errstate(all="ignore"):
+        acc = d[0] / world
+        for k in range(1, world):
+            acc = acc + d[k] / world
+    assert_bits_equal(oracle.reduce("f64", list(d), "sum", oracle.SCALE_PRE_DIV, float(world)), acc,
+                      "f64 pre-div")
+
+
+@pytest.mark.parametrize("wire,dt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+@pytest.mark.parametrize("world", [1, 2, 3, 8, 64])
+def test_compressed_sum_matches_torch_compress_hook(wire, dt, world):
+    rng = np.random.default_rng(400 + world)
+    x = _wide_f32(rng, (world, 3001))
+    # _compress_hook on every rank: buffer.to(dtype).div_(world_size)
+    comp = [torch.from_numpy(r.copy()).to(dt).div_(world) for r in x]
+    # the allreduce of the compressed tensors: fp32 fold in rank order, one rounding
+    acc = comp[0].float()
+    for c in comp[1:]:
+        acc = acc + c.float()
+    reduced = acc.to(dt)
+    # decompress: buffer.copy_(value)
+    buffer = torch.from_numpy(x[0].copy())
+    buffer.copy_(reduced)
+    peers = [c.view(torch.int16).numpy().view(np.uint16) for c in comp]
+    wire_bits = reduced.view(torch.int16).numpy().view(np.uint16)
+    for raw in sorted({0, world // 2, world - 1}):
+        contribs = list(peers)
+        contribs[raw] = x[raw]
+        got = oracle.compressed_sum(contribs, raw, wire, oracle.SCALE_DIV, float(world))
+        assert_bits_equal(got, buffer.numpy(), "%s raw %d -> fp32" % (wire, raw))
+        got = oracle.compressed_sum(contribs, raw, wire, oracle.SCALE_DIV, float(world),
+                                    out_f32=False)
+        assert_bits_equal(got, wire_bits, "%s raw %d -> wire" % (wire, raw), half=True)
+    # no raw contribution: the plain reduction of the wire type, widened or not
+    got = oracle.compressed_sum(peers, -1, wire, out_f32=False)
+    assert_bits_equal(got, oracle.reduce(wire, peers), wire + " all peers", half=True)
+    assert_bits_equal(got, wire_bits, wire + " all peers vs torch", half=True)
+
+
+def test_compressed_sum_bf16_numpy_twin():
+    rng = np.random.default_rng(55)
+    x = _wide_f32(rng, (5, 2000))
+    peers = [oracle.np_f32_to_bf16_rne(r) for r in x]
+    s = np.float32(1) / np.float32(5)
+    with np.errstate(all="ignore"):
+        own = oracle.np_bf16_to_f32(oracle.np_f32_to_bf16_rne(x[3]))
+        own = oracle.np_bf16_to_f32(oracle.np_f32_to_bf16_rne(own * s))
+        acc = oracle.np_bf16_to_f32(peers[0])
+        for k in range(1, 5):
+            acc = acc + (own if k == 3 else oracle.np_bf16_to_f32(peers[k]))
+        want = oracle.np_bf16_to_f32(oracle.np_f32_to_bf16_rne(acc))
+    contribs = list(peers)
+    contribs[3] = x[3]
+    assert_bits_equal(oracle.compressed_sum(contribs, 3, "bf16", oracle.SCALE_MUL, float(s)), want)
+
+
 # ---- layout and slicing ---------------------------------------------------------------
 
 MiB = 1024 * 1024
