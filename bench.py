@@ -18,6 +18,9 @@ Other workloads (the remaining configurations of the benchmark definition, for t
   c5    DDP backward stream: the 1.37 G gradient as 25 MiB buckets (first one
         1 MiB) released in reverse order, one allreduce call per bucket
   copy  K = 1 (a plain copy of known size), the calibration for HBM counters
+  hook  torch's bf16 compression hook folded into the reduction: own fp32
+        gradient compressed in registers + 7 peers' bf16 tensors, result
+        decompressed in place (22 algorithmic bytes per element)
 
 Prints one JSON line with the whole-job GB/s, the roofline of the reduction
 kernel (algorithmic bytes per launch / average launch duration from HIP events
@@ -42,7 +45,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy", "hook"])
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
     ap.add_argument("--k", type=int, default=0, help="override the number of contributions")
     ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
@@ -436,6 +439,65 @@ def run_c5(args, np, torch, fa, oracle):
     return value, elapsed, cfg, roof, checked, None, "f32"
 
 
+def run_hook(args, np, torch, fa, oracle):
+    """The reduction with torch's bf16 compression hook folded in: this rank's
+    fp32 gradient is compressed in registers, K - 1 peers' bf16 tensors are read,
+    the result is decompressed in place into the fp32 gradient. 4 + 2 (K - 1) + 4
+    algorithmic bytes per element."""
+    k, numel = args.k or 8, args.numel or 1_370_000_000
+    slice_elems = args.slice_bytes // 2          # sliced as the bf16 tensor the hook hands over
+    n_slices = (numel + slice_elems - 1) // slice_elems
+    raw = 0
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams,
+                            max_launch_bytes=args.launch_bytes)
+    peers = synth(torch, numel, k, "bf16", 20240)
+    bucket = synth(torch, numel, 1, "f32", 777)[0]
+    contribs = list(peers)
+    contribs[raw] = bucket
+    del peers
+    torch.cuda.synchronize()
+    inv = float(np.float32(1) / np.float32(k))
+
+    def step(d):
+        return d.allreduce_compressed(bucket, contribs, raw, scale_mode=fa.SCALE_MUL, scale=inv)
+
+    elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
+    bytes_per_elem = 4 + 2 * (k - 1) + 4
+    value = bytes_per_elem * numel * args.steps / elapsed / 1e9
+    roof = roofline_from_records(recs, bytes_per_elem, launch_elems(args, slice_elems, 2), SPAN_HOW)
+    roof["kernel"] = "compressedKernel<Bf16Vec, out fp32>, K=%d" % k
+    # parity on a fresh bucket (the timed steps reduced in place)
+    fresh = synth(torch, numel, 1, "f32", 777)[0]
+    bucket.copy_(fresh)
+    step(dev).wait()
+    checked = []
+    for idx in sorted({0, n_slices // 2, n_slices - 1}):
+        lo, hi = idx * slice_elems, min(numel, (idx + 1) * slice_elems)
+        host = [to_host(np, torch, c[lo:hi]) for c in contribs]
+        host[raw] = fresh[lo:hi].cpu().numpy()
+        want = oracle.compressed_sum(host, raw, "bf16", oracle.SCALE_MUL, inv,
+                                     threads=os.cpu_count() or 1)
+        got = bucket[lo:hi].cpu().numpy()
+        if not (got.view(np.uint32) == want.view(np.uint32)).all():
+            raise SystemExit("parity FAILED on slice %d" % idx)
+        checked.append(idx)
+    layout = dev.layout
+    dev.close()
+    cfg = {
+        "workload": "bf16 compression hook folded into the reduction: own fp32 gradient of %d "
+                    "elements + %d peers' bf16 tensors, %d slices of %d B (bf16), x1/%d on the own "
+                    "term, result decompressed in place into the fp32 gradient" % (
+                        numel, k - 1, n_slices, args.slice_bytes, k),
+        "k": k, "numel": numel, "slice_bytes": args.slice_bytes,
+        "staging_total_bytes": args.total_memory, "layout": layout,
+        "reduce_streams": args.streams or "default",
+        "launch_bytes_per_contribution": args.launch_bytes or "default",
+    }
+    return value, elapsed, cfg, roof, checked, None, "bf16"
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -464,6 +526,8 @@ def main():
                                                                        oracle, "bf16")
     elif args.workload == "c3":
         value, elapsed, cfg, roof, checked, base, dtype = run_c3(args, np, torch, fa, oracle)
+    elif args.workload == "hook":
+        value, elapsed, cfg, roof, checked, base, dtype = run_hook(args, np, torch, fa, oracle)
     else:
         value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle)
 
@@ -485,6 +549,7 @@ def main():
         "c3": "reduce GB/s (bytes read+written at HBM level), 64-way fp32 host-staged, one slice",
         "c5": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream",
         "copy": "copy GB/s (bytes read+written), 25 MiB slices",
+        "hook": "reduce GB/s (bytes read+written), 8-way with the bf16 compression hook folded in",
     }[args.workload]
     result = {
         "metric": metric,
