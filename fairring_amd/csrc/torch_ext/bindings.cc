@@ -48,6 +48,11 @@ void bind(py::module& m) {
             py::arg("peers"), py::call_guard<py::gil_scoped_release>());
   group.def("_set_fused_divide", &PG::setFusedDivide, py::arg("on"));
   group.def("_layout", &PG::layout);
+  // the allreduce with one of torch's DDP communication hooks folded in
+  group.def("_allreduce_pre_divided", &PG::allreducePreDivided, py::arg("bucket"),
+            py::call_guard<py::gil_scoped_release>());
+  group.def("_allreduce_compressed", &PG::allreduceCompressed, py::arg("bucket"),
+            py::arg("wire_dtype"), py::call_guard<py::gil_scoped_release>());
 }
 
 }  // namespace

@@ -256,7 +256,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduce_scatter(
 // input (peerNumel == size*n), or its n elements when it hands in just that.
 c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     c10d::OpType opType, const c10d::ReduceOp& reduceOp, at::Tensor own, at::Tensor out,
-    int64_t chunkOffset, int64_t peerNumel, std::vector<at::Tensor> keepAlive) {
+    int64_t chunkOffset, int64_t peerNumel, std::vector<at::Tensor> keepAlive, bool preDivide) {
   // fairring/machine.cc:181: SUM and MAX only
   const c10d::ReduceOp::RedOpType op = reduceOp.op_;
   FRG_CHECK(op == c10d::ReduceOp::SUM || op == c10d::ReduceOp::MAX);
@@ -330,9 +330,18 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
 
   const bool divide = fusedDivide_ && op == c10d::ReduceOp::SUM && size > 1;
   const bool pow2 = (size & (size - 1)) == 0;
-  const int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
-  const float scale = !divide ? 1.0f : (pow2 ? 1.0f / static_cast<float>(size)
-                                              : static_cast<float>(size));
+  int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
+  float scale = !divide ? 1.0f : (pow2 ? 1.0f / static_cast<float>(size)
+                                        : static_cast<float>(size));
+  if (preDivide) {
+    // tensor.div_(size) on every rank ahead of the sum; ATen on the GPU
+    // multiplies by the reciprocal of a scalar divisor
+    TORCH_CHECK(op == c10d::ReduceOp::SUM && at::isFloatingType(out.scalar_type()),
+                "fairring: a pre-divided allreduce is a SUM of a floating-point tensor");
+    TORCH_CHECK(!fromHost, "fairring: a pre-divided allreduce takes GPU-resident peers");
+    scaleMode = FRG_SCALE_PRE_MUL;
+    scale = 1.0f / static_cast<float>(size);
+  }
   const int frgOp = op == c10d::ReduceOp::SUM ? FRG_SUM : FRG_MAX;
 
   if (fromHost) {
@@ -363,6 +372,77 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     TORCH_CHECK(false, "fairring: ", frg_last_error());
   }
   return c10::make_intrusive<WorkFairring>(opType, std::move(future));
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreducePreDivided(at::Tensor bucket) {
+  FRG_CHECK(bucket.layout() == at::kStrided);
+  FRG_CHECK(bucket.is_cuda());
+  FRG_CHECK(bucket.is_non_overlapping_and_dense());
+  at::Tensor t = viewAsFlat(bucket);
+  return reduceCommon(c10d::OpType::ALLREDUCE, c10d::ReduceOp(c10d::ReduceOp::SUM), t, t,
+                      /*chunkOffset=*/0, /*peerNumel=*/t.numel(), {}, /*preDivide=*/true);
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Tensor bucket,
+                                                                         at::ScalarType wire) {
+  FRG_CHECK(bucket.layout() == at::kStrided);
+  FRG_CHECK(bucket.is_cuda());
+  FRG_CHECK(bucket.is_non_overlapping_and_dense());
+  TORCH_CHECK(bucket.scalar_type() == at::kFloat,
+              "fairring: the compression hooks take a float32 bucket, got ", bucket.scalar_type());
+  TORCH_CHECK(wire == at::kBFloat16 || wire == at::kHalf,
+              "fairring: the wire type must be bfloat16 or float16, got ", wire);
+  at::Tensor t = viewAsFlat(bucket);
+
+  std::lock_guard<std::mutex> g(mutex_);
+  const c10::DeviceIndex device = t.device().index();
+  frg_ctx* ctx = contextFor(device);
+  const int size = getSize();
+  const int rank = getRank();
+  const int64_t n = t.numel();
+  std::vector<at::Tensor> peers = peers_;
+  TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
+              "fairring: this build runs on one GPU without a transport; a group of size ",
+              size, " needs ", size - 1, " simulated peer contributions, got ", peers.size());
+  for (at::Tensor& p : peers) {
+    TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense() && p.is_cuda() &&
+                    p.device() == t.device(),
+                "fairring: a compressed peer contribution must be a dense tensor on the bucket's "
+                "device");
+    TORCH_CHECK(p.scalar_type() == wire && p.numel() == n,
+                "fairring: a compressed peer contribution must hold ", n, " elements of ", wire);
+    p = viewAsFlat(p);
+  }
+  std::vector<const void*> table;
+  table.reserve(size);
+  for (int r = 0, pi = 0; r < size; ++r) {
+    table.push_back(r == rank ? t.data_ptr() : peers[pi].data_ptr());
+    if (r != rank) ++pi;
+  }
+  void* streams[16];
+  int nStreams = 0;
+  TORCH_CHECK(frg_get_streams(ctx, streams, 16, &nStreams) == FRG_OK, frg_last_error());
+  for (int i = 0; i < nStreams && i < 16; ++i) {
+    c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
+        static_cast<hipStream_t>(streams[i]), device);
+    t.record_stream(s);
+    for (at::Tensor& p : peers) p.record_stream(s);
+  }
+  auto future = c10::make_intrusive<c10::ivalue::Future>(
+      c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
+  hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
+  auto* pending = new Pending{future, t, std::move(peers), device};
+  // buffer.to(wire).div_(size): on the GPU a multiply by the reciprocal, in
+  // the wire type's arithmetic
+  const int rc = frg_allreduce_compressed(
+      ctx, t.data_ptr(), FRG_F32, table.data(), size, rank, n,
+      wire == at::kBFloat16 ? FRG_BF16 : FRG_F16, size > 1 ? FRG_SCALE_MUL : FRG_SCALE_NONE,
+      1.0f / static_cast<float>(size), current, &onDone, pending, nullptr);
+  if (rc != FRG_OK) {
+    delete pending;
+    TORCH_CHECK(false, "fairring: ", frg_last_error());
+  }
+  return c10::make_intrusive<WorkFairring>(c10d::OpType::ALLREDUCE, std::move(future));
 }
 
 }  // namespace fairring

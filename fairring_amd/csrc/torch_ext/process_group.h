@@ -103,6 +103,20 @@ class ProcessGroupFairring : public c10d::Backend {
   // inside the reduction (DDP otherwise pre-divides each gradient).
   void setFusedDivide(bool on);
 
+  // Not in the reference: the allreduce with one of torch's DDP communication
+  // hooks folded in (torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py).
+  //
+  // allreducePreDivided: allreduce_hook (:18-54). Every rank's bucket is scaled
+  // by 1/size before the sum; here the scaling of all contributions happens
+  // inside the reduction and the peers hand in their unscaled buckets.
+  c10::intrusive_ptr<c10d::Work> allreducePreDivided(at::Tensor bucket);
+  // allreduceCompressed: bf16_compress_hook / fp16_compress_hook (:57-134).
+  // `bucket` is this rank's fp32 gradient bucket, the simulated peers hand in
+  // their buckets already compressed (tensors of `wire`, scaled by 1/size);
+  // this rank's bucket is compressed in registers, the sum is rounded to
+  // `wire` once and written back widened into `bucket`.
+  c10::intrusive_ptr<c10d::Work> allreduceCompressed(at::Tensor bucket, at::ScalarType wire);
+
   // {slot size, slice size, padding slots, staging slots} once initialised.
   std::vector<int64_t> layout();
 
@@ -112,7 +126,8 @@ class ProcessGroupFairring : public c10d::Backend {
                                               const c10d::ReduceOp& reduceOp, at::Tensor own,
                                               at::Tensor out, int64_t chunkOffset,
                                               int64_t peerNumel,
-                                              std::vector<at::Tensor> keepAlive);
+                                              std::vector<at::Tensor> keepAlive,
+                                              bool preDivide = false);
 
   c10::intrusive_ptr<c10d::Store> store_;
   c10::intrusive_ptr<OptionsFairring> options_;
