@@ -534,9 +534,11 @@ def main():
     # HBM bytes per launch as measured with rocprofv3 --pmc (two counter runs,
     # scaled by a copy of known size); the summary that holds the figure names
     # the commands that produced it.
-    if (args.workload == "c2" and args.slice_bytes == 25 * MiB and not args.k
+    traffic_file = {"c2": "ksum_f32_k8_c2_hbm_traffic.md",
+                    "hook": "compressed_bf16_k8_hook_hbm_traffic.md"}.get(args.workload)
+    if (traffic_file and args.slice_bytes == 25 * MiB and not args.k and not args.numel
             and not args.launch_bytes):
-        tpath = os.path.join(ROOT, "profiles", "ksum_f32_k8_c2_hbm_traffic.md")
+        tpath = os.path.join(ROOT, "profiles", traffic_file)
         if os.path.exists(tpath):
             import re
             m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", open(tpath).read())
