@@ -27,59 +27,6 @@
 namespace frg {
 namespace {
 
-// The fp32 side of a lane's elements: 8 floats as two vectors, or one float in
-// the element-wise variant.
-template <int LANES>
-struct Fp32Side;
-
-template <>
-struct Fp32Side<8> {
-  struct regs_t {
-    f32x4 a, b;
-  };
-  __device__ static regs_t load(const float* base, unsigned int lane) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(base) + lane * 32u);
-    regs_t r;
-    r.a = ldStream(p);
-    r.b = ldStream(p + 1);
-    return r;
-  }
-  __device__ static void unpack(const regs_t& r, float (&f)[8]) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      f[j] = r.a[j];
-      f[4 + j] = r.b[j];
-    }
-  }
-  __device__ static void store(float* base, unsigned int lane, const float (&f)[8]) {
-    f32x4* p = reinterpret_cast<f32x4*>(reinterpret_cast<char*>(base) + lane * 32u);
-    f32x4 a, b;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      a[j] = f[j];
-      b[j] = f[4 + j];
-    }
-    stStream(a, p);
-    stStream(b, p + 1);
-  }
-};
-
-template <>
-struct Fp32Side<1> {
-  struct regs_t {
-    float a;
-  };
-  __device__ static regs_t load(const float* base, unsigned int lane) {
-    regs_t r;
-    r.a = ldStream(base + lane);
-    return r;
-  }
-  __device__ static void unpack(const regs_t& r, float (&f)[1]) { f[0] = r.a; }
-  __device__ static void store(float* base, unsigned int lane, const float (&f)[1]) {
-    stStream(f[0], base + lane);
-  }
-};
-
 // State of one lane's fold: the accumulator, whether it holds a term yet, and
 // this rank's own term (compressed once the loads that follow it are issued).
 template <typename W>

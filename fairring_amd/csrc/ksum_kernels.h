@@ -23,7 +23,13 @@ struct ReduceArgs {
   int op = 0;     // FRG_SUM / FRG_MAX
   int scale_mode = 0;
   float scale = 1.0f;
-  bool carry = false;  // out is read first and takes part as term "-1"
+  bool carry = false;  // a carried-in term is read first and takes part as term "-1"
+  const void* carry_src = nullptr;  // where it is read from; null = `out` itself
+  // bf16 / fp16 SUM only: the carried-in term is read from, or the result is
+  // left in, a buffer of fp32 accumulators (unrounded, unscaled), so that a
+  // chain of launches rounds once, at its end.
+  bool carry_acc = false;
+  bool out_acc = false;
   // Optional timing events (created with timing enabled) that receive the
   // begin and end timestamps of this launch.
   hipEvent_t startEvent = nullptr;

@@ -79,6 +79,13 @@ __device__ __forceinline__ void foldChunk(typename TR::acc_t (&acc)[TR::kLanes],
 // on the plain variants.
 constexpr int kPreMul = -2;
 constexpr int kPreDiv = -3;
+// SC value of the variant of the 2-byte floating types that can take the
+// carried-in term from, and leave its result in, a buffer of fp32 accumulators
+// (accFlags): a chain of launches over more contributions than one launch
+// takes then rounds once, at its end, like a single launch. Any scale mode.
+constexpr int kAccIo = -4;
+constexpr int kCarryIsAcc = 1;
+constexpr int kOutIsAcc = 2;
 
 // One vector of the output: out = scale(carry? (+) in[0] (+) ... (+) in[K-1]).
 // SC >= 0 fixes the scale mode at compile time and rules out a carry: the hot
@@ -87,11 +94,12 @@ constexpr int kPreDiv = -3;
 // starts it with a cold instruction cache).
 template <typename TR, int OP, int KT, int SC>
 __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
-                                          const Ptrs<KT>& in, int K, bool carry,
-                                          int scaleMode, float scale,
+                                          const Ptrs<KT>& in, int K,
+                                          const typename TR::elem_t* carrySrc,
+                                          int scaleMode, float scale, int accFlags,
                                           int64_t elemBase, unsigned int lane) {
   if (SC >= 0) {
-    carry = false;
+    carrySrc = nullptr;
     scaleMode = SC;
   }
   using vec_t = typename TR::vec_t;
@@ -99,18 +107,36 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
   vec_t* o = reinterpret_cast<vec_t*>(reinterpret_cast<char*>(out + elemBase) + laneBytes);
   typename TR::acc_t acc[TR::kLanes];
   bool first = true;
-  constexpr int pre = SC == kPreMul ? FRG_SCALE_PRE_MUL : (SC == kPreDiv ? FRG_SCALE_PRE_DIV : 0);
+  constexpr int preC = SC == kPreMul ? FRG_SCALE_PRE_MUL : (SC == kPreDiv ? FRG_SCALE_PRE_DIV : 0);
+  const int pre = SC == kAccIo ? (scaleMode >= FRG_SCALE_PRE_MUL ? scaleMode : 0) : preC;
   const typename TR::acc_t preScale = static_cast<typename TR::acc_t>(scale);
   vec_t c;
-  if (carry) c = *o;  // issued before the contribution loads, consumed first
+  const bool carry = carrySrc != nullptr;
+  // the carried-in term (normally `out` itself): issued before the contribution
+  // loads, consumed first
+  bool carryLoaded = false;
+  if constexpr (SC == kAccIo) {
+    if (carry && (accFlags & kCarryIsAcc)) {
+      using Side = Fp32Side<TR::kLanes>;
+      const typename Side::regs_t r =
+          Side::load(reinterpret_cast<const float*>(carrySrc) + elemBase, lane);
+      Side::unpack(r, acc);
+      first = false;
+      carryLoaded = true;
+    }
+  }
+  if (carry && !carryLoaded) {
+    c = *reinterpret_cast<const vec_t*>(reinterpret_cast<const char*>(carrySrc + elemBase) +
+                                        laneBytes);
+  }
   if (KT > 0) {
-    if (carry) {
+    if (carry && !carryLoaded) {
       TR::unpack(c, acc);
       first = false;
     }
     foldChunk<TR, OP, (KT > 0 ? KT : 1)>(acc, in, 0, elemBase, laneBytes, first, pre, preScale);
   } else {
-    if (carry) {
+    if (carry && !carryLoaded) {
       TR::unpack(c, acc);
       first = false;
     }
@@ -131,7 +157,14 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
       default: break;
     }
   }
-  if constexpr (TR::kFloating && pre == 0) {
+  if constexpr (SC == kAccIo) {
+    if (accFlags & kOutIsAcc) {
+      // parked unrounded and unscaled for the next launch of the chain
+      Fp32Side<TR::kLanes>::store(reinterpret_cast<float*>(out) + elemBase, lane, acc);
+      return;
+    }
+  }
+  if constexpr (TR::kFloating && preC == 0) {
     if (OP == FRG_SUM) {
       // in the accumulator's precision: fp32, or fp64 for fp64 data
       const typename TR::acc_t sc = static_cast<typename TR::acc_t>(scale);
@@ -157,8 +190,9 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
 // end on a few CUs finishing a whole extra tile.
 template <typename TRV, typename TRS, int OP, int KT, int SC>
 __global__ void __launch_bounds__(kBlock)
-    ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K, int carry,
-               int scaleMode, float scale, int64_t head, int64_t nvec,
+    ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K,
+               const typename TRV::elem_t* carrySrc,
+               int scaleMode, float scale, int accFlags, int64_t head, int64_t nvec,
                int64_t tail, int64_t roundTiles, int64_t pieces) {
   // roundTiles (tiles in whole rounds of the grid) and pieces (remainder pieces
   // of kBlock * FRG_REMAINDER_PIECE_UNROLL vectors) come from the host: a
@@ -168,10 +202,19 @@ __global__ void __launch_bounds__(kBlock)
   const int64_t grid = gridDim.x;
   for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
     const int64_t elemBase = head + t * kTile * TRV::kLanes;
+    if constexpr (SC == kAccIo) {
+      // the largest body (every scale mode, both kinds of carry and output) and
+      // the rarest: its two vectors per lane go one after the other
+      for (int u = 0; u < kUnroll; ++u) {
+        reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags, elemBase,
+                                   threadIdx.x + u * kBlock);
+      }
+    } else {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      reduceOne<TRV, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale, elemBase,
-                             threadIdx.x + u * kBlock);
+      for (int u = 0; u < kUnroll; ++u) {
+        reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags, elemBase,
+                                   threadIdx.x + u * kBlock);
+      }
     }
   }
   // remainder: pieces of kBlock * kPiece vectors, the last one possibly partial
@@ -184,7 +227,7 @@ __global__ void __launch_bounds__(kBlock)
     for (int u = 0; u < kPiece; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
       if (v0 + lane < nvec) {
-        reduceOne<TRV, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale,
+        reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags,
                                head + v0 * TRV::kLanes, lane);
       }
     }
@@ -194,7 +237,7 @@ __global__ void __launch_bounds__(kBlock)
     const int64_t e = threadIdx.x < head
                           ? static_cast<int64_t>(threadIdx.x)
                           : head + nvec * TRV::kLanes + (threadIdx.x - head);
-    reduceOne<TRS, OP, KT, SC>(out, in, K, carry != 0, scaleMode, scale, e, 0u);
+    reduceOne<TRS, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags, e, 0u);
   }
 }
 
@@ -208,17 +251,22 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   }
   const GridPlan plan = planGrid(nvec, a.K, numCus);
   const int64_t grid = plan.grid, roundTiles = plan.roundTiles, pieces = plan.pieces;
+  using elem_t = typename TRV::elem_t;
+  const elem_t* carrySrc =
+      !a.carry ? nullptr
+               : static_cast<const elem_t*>(a.carry_src != nullptr ? a.carry_src : a.out);
+  const int accFlags = (a.carry && a.carry_acc ? kCarryIsAcc : 0) | (a.out_acc ? kOutIsAcc : 0);
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
     // Timed launch: the events take the dispatch's own begin/end timestamps.
     hipExtLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
                           dim3(kBlock), 0, stream, a.startEvent, a.stopEvent, 0,
                           static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                          a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, roundTiles, pieces);
+                          carrySrc, a.scale_mode, a.scale, accFlags, head, nvec, tail, roundTiles, pieces);
   } else {
     hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
                        dim3(kBlock), 0, stream,
                        static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                       a.carry ? 1 : 0, a.scale_mode, a.scale, head, nvec, tail, roundTiles, pieces);
+                       carrySrc, a.scale_mode, a.scale, accFlags, head, nvec, tail, roundTiles, pieces);
   }
   return hipGetLastError();
 }
@@ -230,6 +278,13 @@ hipError_t dispatchK(const ReduceArgs& a, int64_t head, int64_t nvec,
                      int64_t tail, int numCus, hipStream_t stream) {
   if (a.op == FRG_MAX) {
     return launchVariant<TRV, TRS, FRG_MAX, 0>(a, head, nvec, tail, numCus, stream);
+  }
+  if ((a.carry && a.carry_acc) || a.out_acc) {
+    if constexpr (TRV::kFloating && sizeof(typename TRV::elem_t) == 2) {
+      return launchVariant<TRV, TRS, FRG_SUM, 0, kAccIo>(a, head, nvec, tail, numCus, stream);
+    } else {
+      return hipErrorInvalidValue;  // ruled out by launchReduce
+    }
   }
   if constexpr (FAST) {
     // the gradient shapes: 2, 4 or 8 contributions, nothing carried in, no
@@ -370,22 +425,53 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   if (a.n == 0) return FRG_OK;  // device.cc:120-122
   if (a.out == nullptr) return fail(FRG_ERR_INVALID, "null output");
 
+  const bool carryAcc = a.carry && a.carry_acc;
+  if (carryAcc || a.out_acc) {
+    if ((a.dtype != FRG_BF16 && a.dtype != FRG_F16) || a.op != FRG_SUM) {
+      return fail(FRG_ERR_INVALID, "fp32 accumulator buffers go with a SUM of bf16 or fp16");
+    }
+    if (carryAcc && a.carry_src == nullptr) {
+      return fail(FRG_ERR_INVALID, "null accumulator buffer to carry from");
+    }
+  }
   const int lanes = static_cast<int>(16 / elsize);
   const uintptr_t o = reinterpret_cast<uintptr_t>(a.out);
+  const uintptr_t outElsize = a.out_acc ? 4 : static_cast<uintptr_t>(elsize);
+  const uintptr_t outBytes = static_cast<uintptr_t>(a.n) * outElsize;
   const uintptr_t bytes = static_cast<uintptr_t>(a.n) * elsize;
-  if (o % elsize != 0) return fail(FRG_ERR_INVALID, "output not element-aligned");
+  if (o % outElsize != 0) return fail(FRG_ERR_INVALID, "output not element-aligned");
+  // Position within 16 bytes that every pointer of the storage type must share
+  // for the vector variant; fp32 accumulator buffers (of a 2-byte type) must
+  // reach a 16-byte boundary after the same number of head elements.
+  const uintptr_t ref = a.out_acc ? (reinterpret_cast<uintptr_t>(a.contribs[0]) & 15) : (o & 15);
+  const uintptr_t headElems = ((16 - ref) & 15) / static_cast<uintptr_t>(elsize);
   bool congruent = true;
+  auto accCongruent = [&](uintptr_t p) { return ((p + 4 * headElems) & 15) == 0; };
+  if (a.out_acc && !accCongruent(o)) congruent = false;
   for (int k = 0; k < a.K; ++k) {
     const uintptr_t p = reinterpret_cast<uintptr_t>(a.contribs[k]);
     if (p == 0) return fail(FRG_ERR_INVALID, "null contribution " + std::to_string(k));
     if (p % elsize != 0) {
       return fail(FRG_ERR_INVALID, "contribution " + std::to_string(k) + " not element-aligned");
     }
-    if (p != o && p < o + bytes && o < p + bytes) {
+    const bool inPlace = p == o && !a.out_acc;
+    if (!inPlace && p < o + outBytes && o < p + bytes) {
       return fail(FRG_ERR_INVALID,
                   "output partially overlaps contribution " + std::to_string(k));
     }
-    if ((p & 15) != (o & 15)) congruent = false;
+    if ((p & 15) != ref) congruent = false;
+  }
+  if (a.carry && a.carry_src != nullptr && a.carry_src != a.out) {
+    const uintptr_t c = reinterpret_cast<uintptr_t>(a.carry_src);
+    const uintptr_t cElsize = carryAcc ? 4 : static_cast<uintptr_t>(elsize);
+    if (c % cElsize != 0) return fail(FRG_ERR_INVALID, "carried-in term not element-aligned");
+    if (c < o + outBytes && o < c + static_cast<uintptr_t>(a.n) * cElsize) {
+      return fail(FRG_ERR_INVALID, "output partially overlaps the carried-in term");
+    }
+    if (carryAcc ? !accCongruent(c) : (c & 15) != ref) congruent = false;
+  } else if (a.carry && carryAcc != a.out_acc) {
+    // carried from `out` itself: both sides of one buffer must be of one kind
+    return fail(FRG_ERR_INVALID, "the carried-in term and the output share a buffer but not a type");
   }
 
   int device = 0;
@@ -396,7 +482,7 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
 
   int64_t head = 0, nvec = 0, tail = 0;
   if (congruent) {
-    head = static_cast<int64_t>(((16 - (o & 15)) & 15) / elsize);
+    head = static_cast<int64_t>(headElems);
     if (head > a.n) head = a.n;
     nvec = (a.n - head) / lanes;
     tail = a.n - head - nvec * lanes;

@@ -184,6 +184,7 @@ Context::~Context() {
   for (hipStream_t s : reduceStreams_) (void)hipStreamSynchronize(s);
   for (hipStream_t s : copyStreams_) (void)hipStreamSynchronize(s);
   if (stagingPool_) (void)hipFree(stagingPool_);
+  if (carryScratch_) (void)hipFree(carryScratch_);
   for (hipEvent_t e : slotFreeEvents_) (void)hipEventDestroy(e);
   for (hipEvent_t e : slotFilledEvents_) (void)hipEventDestroy(e);
   for (hipEvent_t e : freeEvents_) (void)hipEventDestroy(e);
@@ -405,6 +406,64 @@ void Context::launch(const ReduceArgs& args, hipStream_t stream) {
   if (rc != FRG_OK) throw ContractFailure(rc, err);
 }
 
+// The scratch region of a reduce stream (allocated on first use; reused in
+// stream order), placed so that the vector variant of the kernel still runs:
+// at the same position within 16 bytes as `like` for a buffer of the storage
+// type, or, for fp32 accumulators of a 2-byte type, such that it reaches a
+// 16-byte boundary after as many elements as `like` does.
+char* Context::scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize) {
+  if (carryScratch_ == nullptr) {
+    FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&carryScratch_),
+                            reduceStreams_.size() * static_cast<size_t>(kCarryScratchBytes + 16)));
+  }
+  char* base = carryScratch_ + streamIdx * static_cast<size_t>(kCarryScratchBytes + 16);
+  const uintptr_t pos = reinterpret_cast<uintptr_t>(like) & 15;
+  if (!acc) return base + pos;
+  const uintptr_t headElems = ((16 - pos) & 15) / static_cast<uintptr_t>(elsize);
+  return base + ((16 - (4 * headElems) % 16) % 16);
+}
+
+// One part of a slice with more contributions than a launch takes, chained
+// through a scratch buffer in pieces of that buffer's size; only the last
+// launch of each piece writes `out`. Needed where `out` is itself one of the
+// contributions beyond the first launch's (the partial result must not land in
+// it early), and for bf16 / fp16 sums (`acc`: the partial sums stay in fp32).
+void Context::chainThroughScratch(const Request& req, const std::vector<const void*>& ptrs,
+                                  int64_t off, int64_t len, size_t streamIdx, bool acc) {
+  const int64_t elsize = elementSize(req.dtype);
+  const int total = static_cast<int>(ptrs.size());
+  hipStream_t s = reduceStreams_[streamIdx];
+  char* outBase = static_cast<char*>(req.out) + off * elsize;
+  char* scratch = scratchFor(streamIdx, acc ? ptrs[0] : outBase, acc, elsize);
+  const int64_t pieceLen = kCarryScratchBytes / (acc ? 4 : elsize);
+  std::vector<const void*> shifted(ptrs.size());
+  for (int64_t q = 0; q < len; q += pieceLen) {
+    const int64_t qlen = len - q < pieceLen ? len - q : pieceLen;
+    for (size_t k = 0; k < ptrs.size(); ++k) {
+      shifted[k] = static_cast<const char*>(ptrs[k]) + q * elsize;
+    }
+    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
+      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
+      const bool lastLaunch = k0 + kn == total;
+      ReduceArgs a;
+      a.out = lastLaunch ? outBase + q * elsize : scratch;
+      a.out_acc = acc && !lastLaunch;
+      a.contribs = shifted.data() + k0;
+      a.K = kn;
+      a.n = qlen;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
+                                                                        : FRG_SCALE_NONE;
+      a.scale = req.scale;
+      a.carry = k0 > 0;
+      a.carry_src = scratch;
+      a.carry_acc = acc;
+      launch(a, s);
+    }
+  }
+}
+
 void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
   CompressedArgs a = args;
   const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
@@ -463,6 +522,16 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   const int total = static_cast<int>(ptrs.size());
   size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
   bool initialFired = false;
+  // Reduced in place into a contribution that only a later launch of the chain
+  // reads: the partial result must not land in `out` before that.
+  bool lateAlias = false;
+  for (int k = kMaxContribsPerLaunch; k < total && !req.compressed; ++k) {
+    if (req.contribs[k] == req.out) lateAlias = true;
+  }
+  // A chain over bf16 / fp16 contributions keeps its partial sums in fp32
+  // between launches, so that it rounds once like a single launch.
+  const bool accChain = !req.compressed && total > kMaxContribsPerLaunch && req.op == FRG_SUM &&
+                        (req.dtype == FRG_BF16 || req.dtype == FRG_F16);
 
   for (int64_t i = 0; i < nSlices; ++i) {
     int64_t sliceOff, sliceLen;
@@ -521,6 +590,11 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
         lastIdx = si;
         continue;
       }
+      if (lateAlias || accChain) {
+        chainThroughScratch(req, ptrs, off, len, si, accChain);
+        lastIdx = si;
+        continue;
+      }
       // More contributions than one launch takes: chain launches, carrying the
       // partial result in `out`; the post-scale goes on the last one only.
       for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
@@ -566,9 +640,8 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
 std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   // A staged slice must fit a slot as well as the slice size.
-  const int64_t sliceBytes =
+  int64_t sliceBytes =
       layout_.sliceSizeInBytes < slotBytes_ ? layout_.sliceSizeInBytes : slotBytes_;
-  const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
   const int K = static_cast<int>(req.contribs.size());
   hipStream_t s = reduceStreams_[0];
   bool initialFired = false;
@@ -578,6 +651,15 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
   int64_t batch = numSlots_ / 2;
   if (batch < 1) batch = 1;
   if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
+  // bf16 / fp16 sums folded in more than one batch keep their partial sums in
+  // fp32 between the launches (one rounding, like a single launch); the slices
+  // are then as short as the scratch buffer that holds those partial sums.
+  const bool accChain = req.op == FRG_SUM && (req.dtype == FRG_BF16 || req.dtype == FRG_F16) &&
+                        K - (req.carry ? 0 : 1) > batch;
+  if (accChain && sliceBytes > kCarryScratchBytes / 4 * elsize) {
+    sliceBytes = kCarryScratchBytes / 4 * elsize;
+  }
+  const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
 
   for (int64_t i = 0; i < nSlices; ++i) {
     int64_t off, len;
@@ -615,6 +697,8 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
 
     std::vector<const void*> staged;
     std::vector<int64_t> slots;
+    char* accBuf = accChain ? scratchFor(0, outp, /*acc=*/true, elsize) : nullptr;
+    bool inAcc = false;  // the partial sum sits in accBuf (fp32), not in `out`
     for (int k = firstStaged; k < K;) {
       staged.clear();
       slots.clear();
@@ -647,6 +731,15 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       a.scale_mode = k == K ? req.scaleMode : FRG_SCALE_NONE;
       a.scale = req.scale;
       a.carry = true;
+      if (accChain) {
+        a.carry_src = inAcc ? accBuf : outp;
+        a.carry_acc = inAcc;
+        if (k < K) {  // more batches follow
+          a.out = accBuf;
+          a.out_acc = true;
+          inAcc = true;
+        }
+      }
       launch(a, s);
       for (int64_t slot : slots) {
         FRG_HIP_CHECK(hipEventRecord(slotFreeEvents_[slot], s));

@@ -114,6 +114,9 @@ class Context {
   void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
   void launch(const struct ReduceArgs& args, hipStream_t stream);
   void launchCompressed(const struct CompressedArgs& args, hipStream_t stream);
+  void chainThroughScratch(const Request& req, const std::vector<const void*>& ptrs, int64_t off,
+                           int64_t len, size_t streamIdx, bool acc);
+  char* scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize);
   hipEvent_t takeEvent();
   void giveEvent(hipEvent_t e);
 
@@ -131,6 +134,11 @@ class Context {
   std::vector<hipStream_t> copyStreams_;
 
   char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
+  // Allocated on first use, one region per reduce stream: carries the partial
+  // result of a chain of launches that must not, or not yet, land in `out`
+  // (reduced in place into a late contribution; bf16 / fp16 sums, kept in fp32).
+  static constexpr int64_t kCarryScratchBytes = 1024 * 1024;
+  char* carryScratch_ = nullptr;
   std::vector<hipEvent_t> slotFreeEvents_;    // recorded after a slot's last consumer
   std::vector<hipEvent_t> slotFilledEvents_;  // recorded after the copy into a slot
   std::vector<char> slotUsed_;

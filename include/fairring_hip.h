@@ -104,8 +104,12 @@ FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
  * folded left to right in fp32 in exactly that order. `out` may be the same
  * pointer as one of the contributions (in-place, as the reference reduces into
  * the caller's own shard); partial overlaps are rejected. 1 <= K <= 64 per
- * launch; chain launches with carry = 1 for more. n == 0 is a no-op
- * (device.cc:120-122). Asynchronous: returns after enqueueing. */
+ * launch; chain launches with carry = 1 for more. Such a chain carries its
+ * partial result in `out`, in the storage type: exact for fp32, fp64, the
+ * integer types and MAX, but a bf16 / fp16 SUM then rounds once per launch.
+ * frg_allreduce chains those through fp32 accumulators instead and rounds once
+ * for any K. n == 0 is a no-op (device.cc:120-122). Asynchronous: returns
+ * after enqueueing. */
 FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);

@@ -43,6 +43,7 @@ namespace {
 
 struct Job {
   float* out;
+  const float* carrySrc;
   std::vector<const float*> in;
   int64_t n;
   int op;
@@ -60,7 +61,7 @@ void runJob(void* p) {
       return preMul ? x * j->scale : (preDiv ? x / j->scale : x);
     };
     size_t k = 0;
-    float acc = j->carry ? j->out[i] : term(k++);
+    float acc = j->carry ? j->carrySrc[i] : term(k++);
     for (; k < j->in.size(); ++k) {
       const float b = term(k);
       if (j->op == FRG_SUM) {
@@ -153,7 +154,14 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   if (a.n < 0) return fail(FRG_ERR_INVALID, "negative element count");
   if (a.n == 0) return FRG_OK;
   if (a.out == nullptr || a.contribs == nullptr) return fail(FRG_ERR_INVALID, "null pointer");
-  Job* j = new Job{static_cast<float*>(a.out), {}, a.n, a.op, a.scale_mode, a.scale, a.carry};
+  Job* j = new Job{static_cast<float*>(a.out),
+                   static_cast<const float*>(a.carry_src ? a.carry_src : a.out),
+                   {},
+                   a.n,
+                   a.op,
+                   a.scale_mode,
+                   a.scale,
+                   a.carry};
   for (int k = 0; k < a.K; ++k) j->in.push_back(static_cast<const float*>(a.contribs[k]));
   if (a.startEvent) hipEventRecord(a.startEvent, stream);
   fake_hip_enqueue(stream, &runJob, j);

@@ -102,6 +102,14 @@ void scenarioResident() {
       CHECK(frg_work_wait(w) == FRG_OK);
       CHECK(same(out2, fold(big, FRG_SCALE_DIV, 150.f)));
       frg_work_release(w);
+      // the same reduced in place into contribution 100, which only the second
+      // launch of the chain reads: the partial result must not land there early
+      Vec want = fold(big, FRG_SCALE_DIV, 150.f);
+      CHECK(frg_allreduce(ctx, big[100].data(), t2.data(), 150, 3001, FRG_F32, FRG_SUM,
+                          FRG_SCALE_DIV, 150.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(big[100], want));
+      frg_work_release(w);
       CHECK(frg_destroy(ctx) == FRG_OK);
     }
   }
