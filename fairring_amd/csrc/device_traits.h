@@ -152,6 +152,24 @@ struct Bf16Scalar {
   __device__ static acc_t roundStorage(acc_t f) { return bitsToFloat(f32ToBf16Rne(f) << 16); }
 };
 
+// Conversions between fp16 storage and fp32 accumulators go through here. The
+// value is made opaque on the fp32 side, which keeps the compiler from folding a
+// neighbouring multiply into the conversion as a mixed-precision fma with a +0
+// addend (v_fma_mix*): that instruction turns a product of -0 into +0, where
+// ATen, and the multiply followed by the conversion, keep the sign.
+template <typename A, typename E>
+__device__ __forceinline__ A widenElem(E e) {
+  A a = static_cast<A>(e);
+  if constexpr (sizeof(E) == 2 && sizeof(A) == 4) asm("" : "+v"(a));
+  return a;
+}
+
+template <typename E, typename A>
+__device__ __forceinline__ E narrowElem(A a) {
+  if constexpr (sizeof(E) == 2 && sizeof(A) == 4) asm("" : "+v"(a));
+  return static_cast<E>(a);
+}
+
 // Element-wise traits for types whose vector is an ext_vector of the element:
 // convert up on unpack, down (round to nearest even for fp16, wrap-around for
 // integers) on pack.
@@ -164,15 +182,15 @@ struct PlainVec {
   static constexpr bool kFloating = FLOATING;
   __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) {
 #pragma unroll
-    for (int j = 0; j < LANES; ++j) f[j] = static_cast<A>(v[j]);
+    for (int j = 0; j < LANES; ++j) f[j] = widenElem<A, E>(v[j]);
   }
   __device__ static vec_t pack(const acc_t (&f)[kLanes]) {
     vec_t v;
 #pragma unroll
-    for (int j = 0; j < LANES; ++j) v[j] = static_cast<E>(f[j]);
+    for (int j = 0; j < LANES; ++j) v[j] = narrowElem<E, A>(f[j]);
     return v;
   }
-  __device__ static acc_t roundStorage(acc_t f) { return static_cast<A>(static_cast<E>(f)); }
+  __device__ static acc_t roundStorage(acc_t f) { return widenElem<A, E>(narrowElem<E, A>(f)); }
 };
 
 template <typename E, typename A, bool FLOATING>
@@ -182,9 +200,9 @@ struct PlainScalar {
   using acc_t = A;
   static constexpr int kLanes = 1;
   static constexpr bool kFloating = FLOATING;
-  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) { f[0] = static_cast<A>(v); }
-  __device__ static vec_t pack(const acc_t (&f)[kLanes]) { return static_cast<E>(f[0]); }
-  __device__ static acc_t roundStorage(acc_t f) { return static_cast<A>(static_cast<E>(f)); }
+  __device__ static void unpack(const vec_t& v, acc_t (&f)[kLanes]) { f[0] = widenElem<A, E>(v); }
+  __device__ static vec_t pack(const acc_t (&f)[kLanes]) { return narrowElem<E, A>(f[0]); }
+  __device__ static acc_t roundStorage(acc_t f) { return widenElem<A, E>(narrowElem<E, A>(f)); }
 };
 
 using F16Vec = PlainVec<_Float16, float, 8, true>;

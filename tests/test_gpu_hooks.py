@@ -292,3 +292,29 @@ def test_compressed_error_paths():
     e = torch.zeros(0, device=DEV)
     fa.reduce_slice_compressed(e, [e, torch.zeros(0, dtype=torch.bfloat16, device=DEV)], 0)
     torch.cuda.synchronize()
+
+
+def test_fp16_products_of_negative_zero_keep_their_sign():
+    # -0 * s is -0. A mixed-precision fma with a +0 addend, which a compiler may pick for
+    # "multiply, then convert to fp16", gives +0; every scaled fp16 path is held to -0.
+    _print_case("fp16 negative zero")
+    n = 4099
+    neg0 = np.full(n, -0.0, np.float32)
+    tiny = np.full(n, -1e-9, np.float32)          # underflows to -0 in fp16
+    h = neg0.astype(np.float16).view(np.uint16)
+    assert (h == 0x8000).all()
+    xs = [gpu_wire(h, torch.float16)]
+    out = torch.empty_like(xs[0])
+    for mode, s in ((fa.SCALE_MUL, 0.5), (fa.SCALE_DIV, 3.0), (fa.SCALE_PRE_MUL, 0.5),
+                    (fa.SCALE_PRE_DIV, 3.0)):
+        out.fill_(1.0)
+        fa.reduce_slice(out, xs, scale_mode=mode, scale=s)
+        torch.cuda.synchronize()
+        assert (bits_of(out) == 0x8000).all(), mode
+    for src in (neg0, tiny):
+        for mode, s in ((fa.SCALE_NONE, 1.0), (fa.SCALE_MUL, 0.5), (fa.SCALE_DIV, 3.0)):
+            bucket = gpu_f32(src)
+            fa.reduce_slice_compressed(bucket, [bucket], 0, scale_mode=mode, scale=s,
+                                       wire_dtype=torch.float16)
+            torch.cuda.synchronize()
+            assert (bucket.cpu().numpy().view(np.uint32) == 0x80000000).all(), (mode, src[0])

@@ -131,3 +131,117 @@ def test_random_case(seed):
     if guard is not None:   # nothing outside the output range was written
         assert int(torch.count_nonzero(guard[:shift].view(torch.uint8))) == 0
         assert int(torch.count_nonzero(guard[shift + n:].view(torch.uint8))) == 0
+
+
+def draw_host_case(seed):
+    rng = np.random.default_rng(seed)
+    kind = list(KINDS)[rng.integers(len(KINDS))]
+    floating = oracle.TYPES[kind][1]
+    op = "max" if rng.random() < 0.25 else "sum"
+    scale = "none"
+    if floating and op == "sum":
+        scale = ["none", "mul", "div"][rng.integers(3)]
+    return dict(seed=seed, kind=kind, op=op, scale=scale, k=int(rng.integers(1, 14)),
+                n=int(rng.choice([1, 17, 4099, 65537, 300_011])),
+                slots=int(rng.integers(1, 7)), carry=bool(rng.random() < 0.4),
+                slice_bytes=int(rng.choice([16 * 1024, 256 * 1024, 1024 * 1024])),
+                copy_streams=int(rng.integers(1, 4)))
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_host_staged_case(seed):
+    # contributions in pinned host memory, staged through 1 to 6 slots and folded in order
+    c = draw_host_case(zlib.crc32(b"fairring-host-matrix") + seed)
+    print("[case]", c, flush=True)
+    kind, tdt, k, n = c["kind"], KINDS[c["kind"]], c["k"], c["n"]
+    rng = np.random.default_rng(c["seed"] + 1)
+    x = random_values(kind, rng, k, n)
+
+    def pinned(a):
+        t = torch.from_numpy(np.ascontiguousarray(a))
+        if tdt in (torch.float16, torch.bfloat16):
+            t = t.view(torch.int16).view(tdt)
+        return t.pin_memory()
+
+    fmode, omode = SCALES[c["scale"]]
+    sval = {"none": 1.0, "mul": float(np.float32(1) / np.float32(k)), "div": float(k)}[c["scale"]]
+    fop = fa.SUM if c["op"] == "sum" else fa.MAX
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=c["slice_bytes"],
+                            max_memory_allocated_in_bytes=c["slots"] * c["slice_bytes"],
+                            num_copy_streams=c["copy_streams"])
+    if c["carry"]:
+        out = to_gpu(x[0], tdt)
+        dev.allreduce_host(out, [pinned(r) for r in x[1:]], op=fop, scale_mode=fmode, scale=sval,
+                           carry=True).wait()
+    else:
+        out = torch.empty(n, dtype=tdt, device=DEV)
+        dev.allreduce_host(out, [pinned(r) for r in x], op=fop, scale_mode=fmode,
+                           scale=sval).wait()
+    dev.close()
+    if oracle.TYPES[kind][1] and c["op"] == "sum":
+        want = oracle.reduce(kind, list(x), "sum", omode, sval)
+    else:
+        want = oracle.reduce(kind, list(x), c["op"])
+    got = to_np(out)
+    if c["op"] == "max" and kind in ("f32", "bf16", "f16", "f64"):
+        zero = (want == 0) if kind in ("f32", "f64") else ((want & 0x7FFF) == 0)
+        got, want = got[~zero], want[~zero]
+    assert_bits_equal(got, want, str(c), half=kind == "f16")
+
+
+def draw_compressed_case(seed):
+    rng = np.random.default_rng(seed)
+    k = int(rng.choice([1, 2, 3, 5, 8, 9, 16, 31, 64]))
+    return dict(seed=seed, wire=["bf16", "f16"][rng.integers(2)], k=k,
+                raw=int(rng.integers(-1, k)),
+                n=int(rng.choice([1, 7, 8, 9, 1000, 4099, 65537, 300_011, 1_048_577])),
+                shift=int(rng.integers(0, 9)), out_f32=bool(rng.random() < 0.7),
+                in_place=bool(rng.random() < 0.5),
+                mode=["none", "mul", "div"][rng.integers(3)], pipeline=bool(rng.random() < 0.5),
+                slice_bytes=int(rng.choice([8 * 1024, 64 * 1024, 1024 * 1024])),
+                streams=int(rng.integers(1, 4)), launch_div=int(rng.choice([1, 2, 3])))
+
+
+@pytest.mark.parametrize("seed", range(100))
+def test_random_compressed_case(seed):
+    # the reduction with a compression hook folded in: raw fp32 bucket at a random rank
+    c = draw_compressed_case(zlib.crc32(b"fairring-compressed-matrix") + seed)
+    print("[case]", c, flush=True)
+    wire, tdt, k, n, shift, raw = c["wire"], KINDS[c["wire"]], c["k"], c["n"], c["shift"], c["raw"]
+    rng = np.random.default_rng(c["seed"] + 1)
+    xf = random_values("f32", rng, k, n + shift)
+    if wire == "bf16":
+        bits = oracle.np_f32_to_bf16_rne(xf).reshape(xf.shape)
+    else:
+        with np.errstate(over="ignore"):
+            bits = xf.astype(np.float16).view(np.uint16)
+    contribs = [to_gpu(bits[i], tdt)[shift:] for i in range(k)]
+    contribs_np = [bits[i, shift:] for i in range(k)]
+    if raw >= 0:
+        contribs[raw] = to_gpu(xf[raw], torch.float32)[shift:]
+        contribs_np[raw] = xf[raw, shift:]
+    out_dt = torch.float32 if c["out_f32"] else tdt
+    # a float32 output may be the raw bucket itself, a wire-type output any peer's tensor
+    if c["out_f32"]:
+        alias = [raw] if raw >= 0 else []
+    else:
+        alias = [i for i in range(k) if i != raw]
+    if c["in_place"] and alias:
+        out = contribs[alias[int(rng.integers(len(alias)))]]
+    else:
+        out = torch.empty(n + shift, dtype=out_dt, device=DEV)[shift:]
+    fmode, omode = SCALES[c["mode"]]
+    sval = {"none": 1.0, "mul": float(np.float32(1) / np.float32(k)), "div": float(k)}[c["mode"]]
+    if c["pipeline"]:
+        dev = fa.DeviceFairring(0, slice_size_in_bytes=c["slice_bytes"],
+                                max_memory_allocated_in_bytes=2 * c["slice_bytes"],
+                                num_reduce_streams=c["streams"],
+                                max_launch_bytes=max(16, c["slice_bytes"] // c["launch_div"]))
+        dev.allreduce_compressed(out, contribs, raw, scale_mode=fmode, scale=sval,
+                                 wire_dtype=tdt).wait()
+        dev.close()
+    else:
+        fa.reduce_slice_compressed(out, contribs, raw, scale_mode=fmode, scale=sval, wire_dtype=tdt)
+        torch.cuda.synchronize()
+    want = oracle.compressed_sum(contribs_np, raw, wire, omode, sval, out_f32=c["out_f32"])
+    assert_bits_equal(to_np(out), want, str(c), half=(wire == "f16" and not c["out_f32"]))
