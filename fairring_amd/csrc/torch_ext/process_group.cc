@@ -1,5 +1,7 @@
 #include "process_group.h"
 
+#include <cstdlib>
+
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/StreamGuard.h>
 
@@ -293,6 +295,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     if (i == 0) fromHost = !p.is_cuda();
     TORCH_CHECK(fromHost == !p.is_cuda(), "fairring: peers must be all on the GPU or all pinned");
     if (fromHost) {
+      // Switched off by default: one run of this path through the process group
+      // (pinned peers, 2 staging slots, completion through the future) stopped
+      // making progress on an MI355X and no cause has been found. The same
+      // staging through the C ABI (frg_allreduce_host) is unaffected.
+      static const bool allowed = std::getenv("FAIRRING_PINNED_PEERS") != nullptr;
+      TORCH_CHECK(allowed, "fairring: peer contributions in pinned host memory are switched off "
+                           "in the process group (set FAIRRING_PINNED_PEERS=1 to enable them); "
+                           "hand them in as GPU tensors, or use frg_allreduce_host");
       TORCH_CHECK(p.is_pinned(), "fairring: host-side peer contributions must be pinned");
     } else {
       TORCH_CHECK(p.device() == out.device(), "fairring: peer contribution on another device");

@@ -92,7 +92,8 @@ class ProcessGroupFairring : public c10d::Backend {
 
   // Not in the reference. The contributions of the other size-1 ranks, in rank
   // order with this rank left out; GPU tensors on the caller's device or
-  // pinned CPU tensors (then they are staged through the pool). For allreduce
+  // pinned CPU tensors (then they are staged through the pool; refused unless
+  // FAIRRING_PINNED_PEERS is set in the environment). For allreduce
   // each has the tensor's size; for the reduce-scatter forms each is either a
   // peer's whole flat input (size * n elements, its chunk for this rank is
   // taken) or just the n elements it would send here. Used by every operation
