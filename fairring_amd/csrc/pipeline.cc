@@ -1,7 +1,6 @@
 #include "pipeline.h"
 
 #include <cstdio>
-#include <cstdlib>
 #include <stdexcept>
 
 #include "ksum_kernels.h"
@@ -120,10 +119,6 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
-  if (const char* q = std::getenv("FAIRRING_LAUNCH_QUANTUM")) {
-    const long long v = std::atoll(q);
-    if (v >= 16 && v % 16 == 0) c->launchQuantumBytes_ = v;
-  }
   try {
     DeviceGuard g(device);
     int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams : 2;
@@ -220,10 +215,7 @@ void Context::giveEvent(hipEvent_t e) {
 }
 
 void Context::releaseWork(Work* w) {
-  if (w->refs.fetch_sub(1) == 1) {
-
-    delete w;
-  }
+  if (w->refs.fetch_sub(1) == 1) delete w;
 }
 
 bool Context::workEnqueued(Work* w) {
@@ -375,15 +367,20 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   return FRG_OK;
 }
 
-void Context::launch(const ReduceArgs& args, hipStream_t stream) {
-  ReduceArgs a = args;
+// Enqueues one launch and keeps the books around it: the running totals per
+// reduce stream and, with per-launch profiling on, the timing events of the
+// dispatch. Failures become exceptions that run() turns into the work's status.
+template <typename Args>
+void Context::launchAndCount(const Args& args, hipStream_t stream,
+                             int (*enqueue)(const Args&, hipStream_t, std::string*)) {
+  Args a = args;
   const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
   if (prof) {
     FRG_HIP_CHECK(hipEventCreate(&a.startEvent));
     FRG_HIP_CHECK(hipEventCreate(&a.stopEvent));
   }
   std::string err;
-  const int rc = launchReduce(a, stream, &err);
+  const int rc = enqueue(a, stream, &err);
   if (rc == FRG_OK && args.n > 0) {
     for (size_t i = 0; i < reduceStreams_.size(); ++i) {
       if (reduceStreams_[i] == stream) {
@@ -404,6 +401,14 @@ void Context::launch(const ReduceArgs& args, hipStream_t stream) {
   }
   if (rc == FRG_ERR_HIP) throw HipFailure(err);
   if (rc != FRG_OK) throw ContractFailure(rc, err);
+}
+
+void Context::launch(const ReduceArgs& args, hipStream_t stream) {
+  launchAndCount<ReduceArgs>(args, stream, &launchReduce);
+}
+
+void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
+  launchAndCount<CompressedArgs>(args, stream, &launchCompressedReduce);
 }
 
 // The scratch region of a reduce stream (allocated on first use; reused in
@@ -464,37 +469,6 @@ void Context::chainThroughScratch(const Request& req, const std::vector<const vo
   }
 }
 
-void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
-  CompressedArgs a = args;
-  const bool prof = profiling_.load(std::memory_order_relaxed) && args.n > 0;
-  if (prof) {
-    FRG_HIP_CHECK(hipEventCreate(&a.startEvent));
-    FRG_HIP_CHECK(hipEventCreate(&a.stopEvent));
-  }
-  std::string err;
-  const int rc = launchCompressedReduce(a, stream, &err);
-  if (rc == FRG_OK && args.n > 0) {
-    for (size_t i = 0; i < reduceStreams_.size(); ++i) {
-      if (reduceStreams_[i] == stream) {
-        streamLaunches_[i] += 1;
-        streamElems_[i] += args.n;
-      }
-    }
-    lastContribs_ = args.K;
-  }
-  if (prof) {
-    if (rc == FRG_OK) {
-      std::lock_guard<std::mutex> g(profMu_);
-      profEvents_.push_back(ProfRecord{a.startEvent, a.stopEvent, a.n, a.K, stream, 1});
-    } else {
-      (void)hipEventDestroy(a.startEvent);
-      (void)hipEventDestroy(a.stopEvent);
-    }
-  }
-  if (rc == FRG_ERR_HIP) throw HipFailure(err);
-  if (rc != FRG_OK) throw ContractFailure(rc, err);
-}
-
 // Device-resident contributions: every slice (the slicing of
 // fairring/device.cc:315-326) is reduced by one launch, or by several when it
 // is larger than the launch size; launches are dealt round-robin to the reduce
@@ -546,10 +520,10 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     // Launches of about the launch size whose boundaries fall on multiples of
     // the kernel's 4 KiB tile from the start of the slice (a launch that starts
     // off a tile boundary measured 8 % slower). The last launch takes what is
-    // left. FAIRRING_LAUNCH_QUANTUM overrides the boundary multiple.
+    // left.
     int64_t parts = 1;
     int64_t partLen = sliceLen;
-    const int64_t quantum = launchQuantumBytes_ / elsize;
+    const int64_t quantum = kLaunchQuantumBytes / elsize;
     if (maxLaunchElems > 0 && 2 * sliceLen > 3 * maxLaunchElems) {
       parts = (sliceLen + maxLaunchElems / 2) / maxLaunchElems;  // nearest
       partLen = roundDownToNearestMultiple(sliceLen / parts, quantum);

@@ -112,6 +112,9 @@ class Context {
   std::vector<hipStream_t> runHostStaged(const Request& req, hipEvent_t initialEvent);
   // Makes `stream` wait for `initialEvent` unless that event has already fired.
   void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
+  template <typename Args>
+  void launchAndCount(const Args& args, hipStream_t stream,
+                      int (*enqueue)(const Args&, hipStream_t, std::string*));
   void launch(const struct ReduceArgs& args, hipStream_t stream);
   void launchCompressed(const struct CompressedArgs& args, hipStream_t stream);
   void chainThroughScratch(const Request& req, const std::vector<const void*>& ptrs, int64_t off,
@@ -125,7 +128,6 @@ class Context {
   int64_t numSlots_ = 0;
   int64_t slotBytes_ = 0;
   int64_t maxLaunchBytes_ = 0;   // per contribution and launch; 0 = whole slice
-  int64_t launchQuantumBytes_ = kLaunchQuantumBytes;  // launch boundaries within a slice
   int64_t nextLaunch_ = 0;       // deals launches to the reduce streams
 
   std::vector<hipStream_t> reduceStreams_;
