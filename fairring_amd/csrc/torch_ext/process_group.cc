@@ -1,3 +1,5 @@
+#include <Python.h>
+
 #include "process_group.h"
 
 #include <cstdlib>
@@ -147,7 +149,15 @@ ProcessGroupFairring::ProcessGroupFairring(const c10::intrusive_ptr<c10d::Store>
 }
 
 ProcessGroupFairring::~ProcessGroupFairring() {
+  // Destroying a context drains its command thread, whose completion callbacks
+  // may run Python code (future.then) or drop the last reference to a tensor
+  // that Python created: both take the GIL. When this destructor runs from
+  // Python's deallocation of the group, the GIL is held here, so let go of it
+  // for the duration.
+  PyThreadState* saved = nullptr;
+  if (Py_IsInitialized() && PyGILState_Check()) saved = PyEval_SaveThread();
   for (auto& kv : contexts_) frg_destroy(kv.second);
+  if (saved != nullptr) PyEval_RestoreThread(saved);
 }
 
 const std::string ProcessGroupFairring::getBackendName() const { return kPgName; }

@@ -148,6 +148,25 @@ def test_allreduce_server_side_from_pinned_host():
     assert_bits_equal(own.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_MUL, 1.0 / 16))
 
 
+def test_group_destroyed_while_python_callbacks_are_pending():
+    # the group's destructor drains the command thread, whose completion callbacks run Python
+    # code here (future.then): it must not hold the GIL while it waits for them
+    print("[case] pg destroyed with callbacks pending", flush=True)
+    n = 1 << 20
+    pg = make_pg(0, 2)
+    own = torch.ones(n, device=DEV)
+    pg._set_simulated_peer_contributions([torch.ones(n, device=DEV)])
+    seen = []
+    futs = [pg.allreduce([own]).get_future().then(lambda f: seen.append(f.value()[0].numel()))
+            for _ in range(40)]
+    del pg
+    for f in futs:
+        f.wait()
+    torch.cuda.synchronize()
+    assert seen == [n] * 40
+    assert float(own[0]) == 41.0 and float(own[-1]) == 41.0   # 1, plus the peer's 1 forty times
+
+
 def test_missing_peers_is_a_loud_error():
     print("[case] pg missing peers", flush=True)
     pg = make_pg(0, 2)
