@@ -56,7 +56,7 @@ def parse_args():
     ap.add_argument("--copy-streams", type=int, default=0, help="host-staged path (0 = default)")
     ap.add_argument("--blocks-per-cu", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-slices", type=int, default=8)
+    ap.add_argument("--cpu-slices", type=int, default=16)
     return ap.parse_args()
 
 
@@ -96,11 +96,15 @@ def check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale
     return checked
 
 
+TORCH_PASSES = 150   # timed passes of the CPU baseline (about ten seconds of CPU work in all)
+ORACLE_PASSES = 30
+
+
 def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
     """The contract's reduction on this host's cores: torch's at::add chain
     (acc = x0; acc += xk; acc /= K; bf16: fp32 accumulator, one final cast) over
-    `n_sample` distinct 25 MiB slices copied back from the GPU; 3 warm-up and 10
-    timed passes, median. The repository's C restatement (OpenMP) is timed
+    `n_sample` distinct 25 MiB slices copied back from the GPU; 3 warm-up and
+    TORCH_PASSES timed passes, median. The repository's C restatement (OpenMP) is timed
     beside it. GB/s uses the same algorithmic-bytes formula as the GPU figure."""
     host = [[x[i * slice_elems:(i + 1) * slice_elems].cpu() for x in xs]
             for i in range(n_sample)]
@@ -120,7 +124,7 @@ def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
     for _ in range(3):
         one_pass()
     times = []
-    for _ in range(10):
+    for _ in range(TORCH_PASSES):
         t0 = time.perf_counter()
         one_pass()
         times.append(time.perf_counter() - t0)
@@ -136,7 +140,7 @@ def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
     for sl in hnp[:2]:
         fn(sl, oracle.SCALE_DIV, float(k), threads=cores, **kw)
     times = []
-    for _ in range(5):
+    for _ in range(ORACLE_PASSES):
         t0 = time.perf_counter()
         for sl in hnp:
             fn(sl, oracle.SCALE_DIV, float(k), threads=cores, **kw)
@@ -145,8 +149,8 @@ def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
     return {
         "value": round(torch_gbps, 2), "unit": "GB/s", "cores": threads, "kind": "port",
         "sample": "%d distinct 25 MiB slices x K=%d %s, torch CPU at::add chain + div, median of "
-                  "10 passes, %d torch threads of %d host cpus" % (n_sample, k, dtype, threads,
-                                                                    cores),
+                  "%d passes, %d torch threads of %d host cpus" % (n_sample, k, dtype, TORCH_PASSES,
+                                                                    threads, cores),
         "c_oracle_gbps": round(c_gbps, 2), "c_oracle_threads": cores,
     }
 

@@ -179,6 +179,14 @@ frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
     std::terminate();
   }
   TORCH_CHECK(rc == FRG_OK, "fairring: ", frg_last_error());
+  // the layout in force, once per device (the reference logs it from
+  // computeLayout, fairring/utils.h:314-319)
+  frg_layout l = {};
+  if (frg_get_layout(ctx, &l) == FRG_OK) {
+    std::fprintf(stderr, "[fairring] device %d: %lld staging slots, slice size %lld bytes\n",
+                 static_cast<int>(device), static_cast<long long>(l.num_staging_slots),
+                 static_cast<long long>(l.slice_size_in_bytes));
+  }
   contexts_.emplace(device, ctx);
   return ctx;
 }
