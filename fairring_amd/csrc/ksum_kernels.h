@@ -49,13 +49,14 @@ int computeUnits(int device);
 
 // The persistent grid for `nvec` 16-byte vectors per contribution: `grid`
 // blocks, `roundTiles` full tiles dealt in whole rounds of the grid, and what
-// is left dealt in `pieces` smaller pieces.
+// is left dealt in `pieces` smaller pieces. A positive hint fixes the blocks per
+// CU unless the process-wide tuning knob is set.
 struct GridPlan {
   int64_t grid = 1;
   int64_t roundTiles = 0;
   int64_t pieces = 0;
 };
-GridPlan planGrid(int64_t nvec, int numContribs, int numCus);
+GridPlan planGrid(int64_t nvec, int numContribs, int numCus, int blocksPerCuHint = 0);
 
 // The reduction around torch's gradient-compression hooks: peers' tensors in
 // the wire type (bf16 or fp16), this rank's own fp32 buffer compressed in
