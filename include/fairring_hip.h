@@ -183,8 +183,12 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
  * contributions that peers would have delivered passed in explicitly.
  * Device-resident contributions: `contribs[k]` are device pointers to `numel`
  * elements each; the tensor is cut into slices of the layout's slice size and
- * each slice is reduced by one kernel launch, slices rotating over the
- * reduce streams / staging slots. `producer_stream` is the stream the caller's
+ * each slice is reduced by one kernel launch, or by a few when it is much
+ * larger than frg_options.max_launch_bytes, the launches rotating over the
+ * reduce streams. More than 64 contributions are folded by a chain of
+ * launches per range; the result is that of one fold over all of them, with
+ * one rounding (bf16 / fp16 partial sums travel as fp32), also when `out` is
+ * one of the contributions. `producer_stream` is the stream the caller's
  * producer work was enqueued on (the reference records its initial event on
  * the current stream, device.cc:294-295). Returns immediately; `*work`
  * (optional) receives a handle to wait on. */
