@@ -129,6 +129,45 @@ def test_c4_full_size_bf16(dev):
                           oracle.sum_bf16(host, oracle.SCALE_MUL, 0.125, threads=16), "slice %d" % idx)
 
 
+def test_hook_full_size_bf16_compression_folded_in(dev):
+    # the 1.37 G fp32 gradient with torch's bf16 compression hook folded into the reduction:
+    # own bucket compressed in registers, 7 peers' bf16 tensors, result widened in place
+    print("[case] hook full size", flush=True)
+    numel, k, raw = 1_370_000_000, 8, 3
+    g = torch.Generator(device=DEV)
+    g.manual_seed(6)
+    inv = float(np.float32(1) / np.float32(k))
+    bucket = torch.empty(numel, device=DEV).normal_(0, 0.01, generator=g)
+    # (1) peers all zero, no scale: the bucket comes back rounded to bf16, nothing else
+    zeros = torch.zeros(numel, dtype=torch.bfloat16, device=DEV)
+    contribs = [zeros] * k
+    contribs[raw] = bucket
+    want = bucket.to(torch.bfloat16).float()
+    dev.allreduce_compressed(bucket, contribs, raw).wait()
+    assert bool(torch.equal(bucket, want))
+    # (2) the same again is the identity (the values are bf16 already), also with x 1/8:
+    #     a bf16 value times a power of two is exact
+    dev.allreduce_compressed(bucket, contribs, raw, scale_mode=fa.SCALE_MUL, scale=inv).wait()
+    assert bool(torch.equal(bucket, want * inv))
+    del zeros, want
+    # (3) random peers, oracle on sampled slices (sliced as the bf16 tensor: 13,107,200 elements)
+    bucket.normal_(0, 0.01, generator=g)
+    fresh = bucket.clone()
+    peers = [torch.empty(numel, device=DEV).normal_(0, 0.01, generator=g).to(torch.bfloat16)
+             for _ in range(k)]
+    contribs = list(peers)
+    contribs[raw] = bucket
+    dev.allreduce_compressed(bucket, contribs, raw, scale_mode=fa.SCALE_MUL, scale=inv).wait()
+    for idx, lo, hi in sampled_slices(numel, SLICE // 2):
+        host = [bits16(p[lo:hi]) for p in peers]
+        host[raw] = fresh[lo:hi].cpu().numpy()
+        assert_bits_equal(bucket[lo:hi].cpu().numpy(),
+                          oracle.compressed_sum(host, raw, "bf16", oracle.SCALE_MUL, inv, threads=16),
+                          "slice %d" % idx)
+    # every value of the result is a bf16 value
+    assert bool(torch.equal(bucket, bucket.to(torch.bfloat16).float()))
+
+
 def test_c3_full_size_server_side_from_pinned_host(dev):
     # configs[2]: K = 64 contributions of one 25 MiB fp32 slice in pinned host memory
     print("[case] c3 full size", flush=True)
