@@ -402,6 +402,68 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
   return c10::make_intrusive<WorkFairring>(opType, std::move(future));
 }
 
+// ---- a group of one: collectives that only move data ------------------------
+
+void ProcessGroupFairring::requireGroupOfOne(const char* what) const {
+  TORCH_CHECK(getSize() == 1, "fairring: ", what, " needs a transport between ranks; this build "
+              "runs on one GPU and supports it for a group of size 1 only (got size ", getSize(),
+              ")");
+}
+
+// A finished Work whose future is marked under the caller's current stream, so
+// that whatever was enqueued there (a copy) is what consumers are ordered after.
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::completedWork(
+    c10d::OpType opType, std::vector<at::Tensor> tensors) {
+  std::vector<c10::Device> devices;
+  for (const at::Tensor& t : tensors) {
+    if (t.is_cuda() && (devices.empty() || devices.back() != t.device())) {
+      devices.push_back(t.device());
+    }
+  }
+  auto future =
+      c10::make_intrusive<c10::ivalue::Future>(c10::ListType::ofTensors(), std::move(devices));
+  future->markCompleted(std::move(tensors));
+  return c10::make_intrusive<WorkFairring>(opType, std::move(future));
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::broadcast(
+    std::vector<at::Tensor>& data, const c10d::BroadcastOptions& /*opts*/) {
+  requireGroupOfOne("broadcast");
+  return completedWork(c10d::OpType::BROADCAST, data);  // the root already holds its own data
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allgather(
+    std::vector<std::vector<at::Tensor>>& outputTensors, std::vector<at::Tensor>& inputTensors,
+    const c10d::AllgatherOptions& /*opts*/) {
+  requireGroupOfOne("allgather");
+  TORCH_CHECK(outputTensors.size() == inputTensors.size(),
+              "fairring: allgather takes one output list per input tensor");
+  std::vector<at::Tensor> outs;
+  for (size_t i = 0; i < inputTensors.size(); ++i) {
+    TORCH_CHECK(outputTensors[i].size() == 1, "fairring: allgather output list must hold ",
+                getSize(), " tensor(s)");
+    outputTensors[i][0].copy_(inputTensors[i], /*non_blocking=*/true);
+    outs.push_back(outputTensors[i][0]);
+  }
+  return completedWork(c10d::OpType::ALLGATHER, std::move(outs));
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::_allgather_base(
+    at::Tensor& outputBuffer, at::Tensor& inputBuffer, const c10d::AllgatherOptions& /*opts*/) {
+  requireGroupOfOne("_allgather_base");
+  TORCH_CHECK(outputBuffer.numel() == inputBuffer.numel(),
+              "fairring: _allgather_base output must hold size * input elements");
+  FRG_CHECK(outputBuffer.is_non_overlapping_and_dense());
+  FRG_CHECK(inputBuffer.is_non_overlapping_and_dense());
+  viewAsFlat(outputBuffer).copy_(viewAsFlat(inputBuffer), /*non_blocking=*/true);
+  return completedWork(c10d::OpType::_ALLGATHER_BASE, {outputBuffer});
+}
+
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::barrier(const c10d::BarrierOptions& /*opts*/) {
+  requireGroupOfOne("barrier");
+  return completedWork(c10d::OpType::BARRIER, {});
+}
+
 c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreducePreDivided(at::Tensor bucket) {
   FRG_CHECK(bucket.layout() == at::kStrided);
   FRG_CHECK(bucket.is_cuda());

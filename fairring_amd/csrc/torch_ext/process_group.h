@@ -90,6 +90,23 @@ class ProcessGroupFairring : public c10d::Backend {
       at::Tensor& outputBuffer, at::Tensor& inputBuffer,
       const c10d::ReduceScatterOptions& opts = c10d::ReduceScatterOptions()) override;
 
+  // The collectives that move data without reducing it need a transport (the
+  // reference runs them on NCCL: fairring/process_group.cc:124-129,173-251,
+  // 423-440). Here they exist for a group of one, where nothing moves, so that
+  // DistributedDataParallel can be built on the backend as it is; for a larger
+  // group they raise.
+  c10::intrusive_ptr<c10d::Work> broadcast(
+      std::vector<at::Tensor>& data,
+      const c10d::BroadcastOptions& opts = c10d::BroadcastOptions()) override;
+  c10::intrusive_ptr<c10d::Work> allgather(
+      std::vector<std::vector<at::Tensor>>& outputTensors, std::vector<at::Tensor>& inputTensors,
+      const c10d::AllgatherOptions& opts = c10d::AllgatherOptions()) override;
+  c10::intrusive_ptr<c10d::Work> _allgather_base(
+      at::Tensor& outputBuffer, at::Tensor& inputBuffer,
+      const c10d::AllgatherOptions& opts = c10d::AllgatherOptions()) override;
+  c10::intrusive_ptr<c10d::Work> barrier(
+      const c10d::BarrierOptions& opts = c10d::BarrierOptions()) override;
+
   // Not in the reference. The contributions of the other size-1 ranks, in rank
   // order with this rank left out; GPU tensors on the caller's device or
   // pinned CPU tensors (then they are staged through the pool; refused unless
@@ -123,6 +140,9 @@ class ProcessGroupFairring : public c10d::Backend {
 
  private:
   frg_ctx* contextFor(c10::DeviceIndex device);
+  void requireGroupOfOne(const char* what) const;
+  c10::intrusive_ptr<c10d::Work> completedWork(c10d::OpType opType,
+                                               std::vector<at::Tensor> tensors);
   c10::intrusive_ptr<c10d::Work> reduceCommon(c10d::OpType opType,
                                               const c10d::ReduceOp& reduceOp, at::Tensor own,
                                               at::Tensor out, int64_t chunkOffset,

@@ -123,7 +123,7 @@ def grads(hook):
     torch.manual_seed(0)
     model = nn.Sequential(nn.Linear(512, 1024), nn.GELU(), nn.Linear(1024, 1024), nn.GELU(),
                           nn.Linear(1024, 10)).to("cuda:0")
-    ddp = DDP(model, device_ids=[0], bucket_cap_mb=1, init_sync=False)
+    ddp = DDP(model, device_ids=[0], bucket_cap_mb=1)   # init_sync: broadcast + allgather, group of one
     if hook is not None:
         ddp.register_comm_hook(None, hook)
     x = torch.randn(64, 512, device="cuda:0", generator=torch.Generator("cuda:0").manual_seed(1))

@@ -167,6 +167,28 @@ def test_group_destroyed_while_python_callbacks_are_pending():
     assert float(own[0]) == 41.0 and float(own[-1]) == 41.0   # 1, plus the peer's 1 forty times
 
 
+def test_data_moving_collectives_exist_for_a_group_of_one_only():
+    print("[case] pg broadcast/allgather/barrier", flush=True)
+    pg = make_pg(0, 1)
+    x = torch.arange(1000, dtype=torch.float32, device=DEV)
+    w = pg.broadcast([x])
+    assert w.wait() and w.is_completed() and w.result()[0].data_ptr() == x.data_ptr()
+    out = torch.zeros(1000, device=DEV)
+    pg.allgather([[out]], [x]).wait()
+    torch.cuda.synchronize()
+    assert bool(torch.equal(out, x))
+    out2 = torch.zeros(2, 500, device=DEV)
+    pg._allgather_base(out2, x).wait()
+    torch.cuda.synchronize()
+    assert bool(torch.equal(out2.reshape(-1), x))
+    assert pg.barrier().wait()
+    pg2 = make_pg(0, 2)
+    for call in (lambda: pg2.broadcast([x]), lambda: pg2.allgather([[out, out]], [x]),
+                 lambda: pg2._allgather_base(torch.zeros(2000, device=DEV), x), pg2.barrier):
+        with pytest.raises(RuntimeError, match="needs a transport"):
+            call()
+
+
 def test_missing_peers_is_a_loud_error():
     print("[case] pg missing peers", flush=True)
     pg = make_pg(0, 2)
