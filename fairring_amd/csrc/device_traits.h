@@ -70,11 +70,25 @@ __device__ __forceinline__ float bitsToFloat(unsigned int u) {
   return __builtin_bit_cast(float, u);
 }
 
-// fp32 -> bf16 bits, round to nearest even, NaN -> 0x7FC0.
+// fp32 -> bf16 bits, round to nearest even, NaN -> 0x7FC0 (as ATen). gfx950
+// converts in hardware (v_cvt_pk_bf16_f32, two values per instruction); the NaN
+// pattern is fixed up afterwards.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ unsigned int f32PairToBf16Rne(float lo, float hi) {
+  f32x2 v;
+  v[0] = lo;
+  v[1] = hi;
+  unsigned int r = __builtin_bit_cast(unsigned int, __builtin_convertvector(v, bf16x2));
+  if (lo != lo) r = (r & 0xFFFF0000u) | 0x7FC0u;
+  if (hi != hi) r = (r & 0x0000FFFFu) | 0x7FC00000u;
+  return r;
+}
+
 __device__ __forceinline__ unsigned int f32ToBf16Rne(float f) {
-  unsigned int u = __builtin_bit_cast(unsigned int, f);
-  unsigned int r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? 0x7FC0u : r;
+  const unsigned short r = __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
+  return (f != f) ? 0x7FC0u : static_cast<unsigned int>(r);
 }
 
 // ---- storage traits: how a "vector" of elements is loaded and unpacked ------
@@ -130,7 +144,7 @@ struct Bf16Vec {  // 8 bf16 in 16 bytes
     vec_t v;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      v[j] = f32ToBf16Rne(f[2 * j]) | (f32ToBf16Rne(f[2 * j + 1]) << 16);
+      v[j] = f32PairToBf16Rne(f[2 * j], f[2 * j + 1]);
     }
     return v;
   }

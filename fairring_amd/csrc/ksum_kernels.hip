@@ -501,7 +501,7 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
       e = dispatchType<Bf16Vec, Bf16Scalar, true>(a, head, nvec, tail, numCus, stream);
       break;
     case FRG_F16:
-      e = dispatchType<F16Vec, F16Scalar, false>(a, head, nvec, tail, numCus, stream);
+      e = dispatchType<F16Vec, F16Scalar, true>(a, head, nvec, tail, numCus, stream);
       break;
     case FRG_F64:
       e = dispatchType<F64Vec, F64Scalar, false>(a, head, nvec, tail, numCus, stream);
