@@ -186,23 +186,22 @@ DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch target per 
 LAUNCH_QUANTUM_BYTES = 4096
 
 
-def launch_elems(args, slice_elems, elsize):
-    """Elements of the commonest launch: a slice much larger than the launch
-    target is cut on 4 KiB boundaries into parts of about that size (what the
-    pipeline does); the last part of a slice takes the rest."""
+def launch_elems(args, op_elems, slice_elems, elsize):
+    """Elements of the commonest launch of an operation over `op_elems` elements:
+    the pipeline cuts the tensor into launches of the launch target, on 4 KiB
+    boundaries from its start and whatever the slice size; the last launch takes
+    up to one and a half times that. A negative target means one launch per
+    slice."""
     lb = args.launch_bytes or DEFAULT_LAUNCH_BYTES
     if lb < 0:
-        return slice_elems
+        return min(slice_elems, op_elems)
     max_elems = (lb - lb % 16) // elsize
-    if 2 * slice_elems <= 3 * max_elems:
-        return slice_elems
-    parts = (slice_elems + max_elems // 2) // max_elems
     quantum = LAUNCH_QUANTUM_BYTES // elsize
-    per = (slice_elems // parts) // quantum * quantum
+    per = max_elems // quantum * quantum
     if per < quantum:
         lanes = 16 // elsize
-        per = -(-(-(-slice_elems // parts)) // lanes) * lanes
-    return per
+        per = -(-max_elems // lanes) * lanes
+    return per if 2 * op_elems > 3 * per else op_elems
 
 
 def roofline_from_records(recs, bytes_per_elem, full_launch_elems, how):
@@ -306,7 +305,8 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     step_bytes = (k + 1) * numel * elsize
     value = step_bytes * args.steps / elapsed / 1e9
-    roof = roofline_from_records(recs, (k + 1) * elsize, launch_elems(args, slice_elems, elsize),
+    roof = roofline_from_records(recs, (k + 1) * elsize,
+                                 launch_elems(args, numel, slice_elems, elsize),
                                  SPAN_HOW)
     roof["kernel"] = "ksumKernel<%s, SUM, K=%d>" % ("F32Vec" if dtype == "f32" else "Bf16Vec", k)
     step(dev).wait()
@@ -426,7 +426,8 @@ def run_c5(args, np, torch, fa, oracle):
     elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     step_bytes = (k + 1) * numel * 4
     value = step_bytes * args.steps / elapsed / 1e9
-    roof = roofline_from_records(recs, (k + 1) * 4, launch_elems(args, slice_elems, 4), SPAN_HOW)
+    roof = roofline_from_records(recs, (k + 1) * 4,
+                                 launch_elems(args, slice_elems, slice_elems, 4), SPAN_HOW)
     roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
     step(dev).wait()
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)
@@ -470,7 +471,8 @@ def run_hook(args, np, torch, fa, oracle):
     elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     bytes_per_elem = 4 + 2 * (k - 1) + 4
     value = bytes_per_elem * numel * args.steps / elapsed / 1e9
-    roof = roofline_from_records(recs, bytes_per_elem, launch_elems(args, slice_elems, 2), SPAN_HOW)
+    roof = roofline_from_records(recs, bytes_per_elem, launch_elems(args, numel, slice_elems, 2),
+                                 SPAN_HOW)
     roof["kernel"] = "compressedKernel<Bf16Vec, out fp32>, K=%d" % k
     # parity on a fresh bucket (the timed steps reduced in place)
     fresh = synth(torch, numel, 1, "f32", 777)[0]

@@ -147,12 +147,12 @@ typedef struct frg_options {
   int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
   int32_t num_reduce_streams;             /* 0 = default (2) */
   int32_t num_copy_streams;               /* host-staged path; 0 = default (2), at most 4 */
-  int64_t max_launch_bytes;               /* target bytes of one contribution that a single
-                                             reduction launch covers; a slice much larger than
-                                             this is reduced by several launches (cut on 4 KiB
-                                             boundaries from the slice start) dealt round-robin
-                                             to the reduce streams. 0 = default (12.5 MiB), < 0
-                                             = one launch per slice */
+  int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
+                                             launch covers: device-resident tensors are cut into
+                                             launches of this size on 4 KiB boundaries (the last
+                                             one up to 1.5 times as long), dealt round-robin to the
+                                             reduce streams. 0 = default (12.5 MiB), < 0 = one
+                                             launch per slice */
 } frg_options;
 
 /* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,
@@ -182,10 +182,11 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
 /* DeviceFairring::allReduce: fairring/device.cc:291-353, with the
  * contributions that peers would have delivered passed in explicitly.
  * Device-resident contributions: `contribs[k]` are device pointers to `numel`
- * elements each; the tensor is cut into slices of the layout's slice size and
- * each slice is reduced by one kernel launch, or by a few when it is much
- * larger than frg_options.max_launch_bytes, the launches rotating over the
- * reduce streams. More than 64 contributions are folded by a chain of
+ * elements each. The slices of the layout only count here (they advance the
+ * slot cursor): resident contributions need no slot, so the tensor is reduced
+ * by launches of frg_options.max_launch_bytes per contribution, cut on 4 KiB
+ * boundaries from its start and rotating over the reduce streams, whatever
+ * the slice size (max_launch_bytes < 0: one launch per slice). More than 64 contributions are folded by a chain of
  * launches per range; the result is that of one fold over all of them, with
  * one rounding (bf16 / fp16 partial sums travel as fp32), also when `out` is
  * one of the contributions. `producer_stream` is the stream the caller's

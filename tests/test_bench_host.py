@@ -34,17 +34,19 @@ def test_defaults_are_the_headline_configuration():
     assert a.steps >= 1 and a.warmup >= 1
 
 
-@pytest.mark.parametrize("slice_elems,elsize,lb,want", [
-    (6_553_600, 4, 0, 3_276_800),          # 25 MiB fp32 slice: two launches of 12.5 MiB
-    (13_107_200, 2, 0, 6_553_600),         # 25 MiB bf16 slice
-    (6_553_600, 4, -1, 6_553_600),         # one launch per slice
-    (819_196, 4, 0, 819_196),              # default-layout slice (3,276,784 B): below the target
-    (6_553_600, 4, 6 * MiB, 1_638_400),    # 4 launches, cut on 4 KiB boundaries
-    (297_600, 4, 0, 297_600),              # the ragged last slice
+@pytest.mark.parametrize("op_elems,slice_elems,elsize,lb,want", [
+    (1_370_000_000, 6_553_600, 4, 0, 3_276_800),   # 12.5 MiB launches, whatever the slice size
+    (1_300_000_000, 13_107_200, 2, 0, 6_553_600),  # bf16
+    (1_370_000_000, 819_196, 4, 0, 3_276_800),     # default layout (3,276,784 B slices): the same
+    (1_370_000_000, 6_553_600, 4, -1, 6_553_600),  # one launch per slice
+    (6_553_600, 6_553_600, 4, 0, 3_276_800),       # one 25 MiB bucket: two launches
+    (262_144, 6_553_600, 4, 0, 262_144),           # the 1 MiB bucket: one launch
+    (4_000_000, 6_553_600, 4, 0, 4_000_000),       # up to 1.5 x the target: still one launch
+    (1_370_000_000, 6_553_600, 4, 6 * MiB, 1_572_864),
 ])
-def test_launch_elems_follows_the_pipeline_rule(slice_elems, elsize, lb, want):
+def test_launch_elems_follows_the_pipeline_rule(op_elems, slice_elems, elsize, lb, want):
     args = types.SimpleNamespace(launch_bytes=lb)
-    assert bench.launch_elems(args, slice_elems, elsize) == want
+    assert bench.launch_elems(args, op_elems, slice_elems, elsize) == want
 
 
 def test_ddp_bucket_schedule():
