@@ -227,6 +227,21 @@ int frg_work_wait(frg_work* work) {
   return FRG_OK;
 }
 
+int frg_set_wait_timeout(double seconds) {
+  frg::setWaitTimeout(seconds);
+  return FRG_OK;
+}
+
+int frg_get_progress(frg_ctx* ctx, frg_progress* out) {
+  if (ctx == nullptr || out == nullptr) return fail(FRG_ERR_INVALID, "null argument");
+  const frg::Progress& p = asCtx(ctx)->progress();
+  out->submitted = p.submitted.load();
+  out->started = p.started.load();
+  out->enqueued = p.enqueued.load();
+  out->launches = p.launches.load();
+  return FRG_OK;
+}
+
 int frg_work_is_completed(frg_work* work) {
   if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
   return Context::workEnqueued(asWork(work)) ? FRG_OK : FRG_ERR_NOT_READY;

@@ -1,6 +1,8 @@
 #include "pipeline.h"
 
+#include <chrono>
 #include <cstdio>
+#include <cstdlib>
 #include <stdexcept>
 
 #include "ksum_kernels.h"
@@ -223,10 +225,57 @@ bool Context::workEnqueued(Work* w) {
   return w->enqueued;
 }
 
+namespace {
+
+// Seconds after which a wait gives up and reports where the pipeline stands
+// instead of blocking for good; 0 = wait without limit, as the reference does
+// (fairring/process_group.cc:64-68). Starts from FAIRRING_WAIT_TIMEOUT_S.
+std::atomic<double>& waitTimeout() {
+  static std::atomic<double> seconds{[] {
+    const char* v = std::getenv("FAIRRING_WAIT_TIMEOUT_S");
+    const double s = v ? std::atof(v) : 0.0;
+    return s > 0.0 ? s : 0.0;
+  }()};
+  return seconds;
+}
+
+double waitTimeoutSeconds() { return waitTimeout().load(); }
+
+std::string progressReport(const Work* w) {
+  const Progress& p = *w->progress;
+  return "operation #" + std::to_string(w->seq) + "; context: " +
+         std::to_string(p.submitted.load()) + " submitted, " + std::to_string(p.started.load()) +
+         " started by the command thread, " + std::to_string(p.enqueued.load()) +
+         " fully enqueued, " + std::to_string(p.launches.load()) + " kernel launches issued";
+}
+
+}  // namespace
+
+void setWaitTimeout(double seconds) { waitTimeout().store(seconds > 0.0 ? seconds : 0.0); }
+
 int Context::waitWork(Work* w, std::string* err) {
+  const double limit = waitTimeoutSeconds();
+  const auto deadline = std::chrono::steady_clock::now() +
+                        std::chrono::duration_cast<std::chrono::steady_clock::duration>(
+                            std::chrono::duration<double>(limit));
   {
     std::unique_lock<std::mutex> lock(w->mu);
-    w->cv.wait(lock, [&] { return w->enqueued; });
+    if (limit > 0.0) {
+      // against the system clock: that is pthread_cond_timedwait, which
+      // ThreadSanitizer models (the steady-clock wait is not intercepted by
+      // older versions of it, which then report a double lock)
+      const auto wallDeadline =
+          std::chrono::system_clock::now() +
+          std::chrono::duration_cast<std::chrono::system_clock::duration>(
+              std::chrono::duration<double>(limit));
+      if (!w->cv.wait_until(lock, wallDeadline, [&] { return w->enqueued; })) {
+        *err = "gave up after " + std::to_string(limit) +
+               " s waiting for the command thread to enqueue " + progressReport(w);
+        return FRG_ERR_NOT_READY;
+      }
+    } else {
+      w->cv.wait(lock, [&] { return w->enqueued; });
+    }
     if (w->status != FRG_OK) {
       *err = w->error;
       return w->status;
@@ -234,7 +283,28 @@ int Context::waitWork(Work* w, std::string* err) {
   }
   try {
     DeviceGuard g(w->device);
-    for (hipStream_t s : w->doneStreams) FRG_HIP_CHECK(hipStreamSynchronize(s));
+    for (size_t i = 0; i < w->doneStreams.size(); ++i) {
+      hipStream_t s = w->doneStreams[i];
+      if (limit <= 0.0) {
+        FRG_HIP_CHECK(hipStreamSynchronize(s));
+        continue;
+      }
+      // poll, so that a stream that never drains ends in a message, not a stall
+      int64_t spins = 0;
+      for (;;) {
+        const hipError_t q = hipStreamQuery(s);
+        if (q == hipSuccess) break;
+        if (q != hipErrorNotReady) FRG_HIP_CHECK(q);
+        (void)hipGetLastError();
+        if (std::chrono::steady_clock::now() > deadline) {
+          *err = "gave up after " + std::to_string(limit) + " s waiting for stream " +
+                 std::to_string(i) + " of " + std::to_string(w->doneStreams.size()) +
+                 " to drain after " + progressReport(w);
+          return FRG_ERR_NOT_READY;
+        }
+        if (++spins > 2000) std::this_thread::sleep_for(std::chrono::microseconds(50));
+      }
+    }
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;
@@ -346,6 +416,8 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
 
   Work* work = new Work();
   work->device = device_;
+  work->progress = progress_;
+  work->seq = progress_->submitted.fetch_add(1);
   hipEvent_t initial = nullptr;
   try {
     DeviceGuard g(device_);
@@ -389,6 +461,7 @@ void Context::launchAndCount(const Args& args, hipStream_t stream,
       }
     }
     lastContribs_ = args.K;
+    progress_->launches.fetch_add(1);
   }
   if (prof) {
     if (rc == FRG_OK) {
@@ -736,6 +809,7 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
 
 void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
   const int64_t seq = nextSeq_++;
+  progress_->started.fetch_add(1);
   int status = FRG_OK;
   std::string error;
   hipStream_t lastStream = reduceStreams_[0];
@@ -769,6 +843,7 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
                  static_cast<long long>(seq), error.c_str());
   }
   giveEvent(initialEvent);
+  progress_->enqueued.fetch_add(1);
   {
     std::lock_guard<std::mutex> g(work->mu);
     work->status = status;

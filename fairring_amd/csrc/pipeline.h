@@ -9,6 +9,7 @@
 #include <condition_variable>
 #include <deque>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <thread>
@@ -33,6 +34,16 @@ class CommandQueue {
   std::deque<std::function<void()>> fns_;
 };
 
+// Progress counters of a context, shared with the works it hands out so that a
+// wait that gives up can say where things stand (a work may outlive its
+// context's handle).
+struct Progress {
+  std::atomic<int64_t> submitted{0};  // operations accepted by submit()
+  std::atomic<int64_t> started{0};    // operations the command thread has begun
+  std::atomic<int64_t> enqueued{0};   // operations whose GPU work is all enqueued
+  std::atomic<int64_t> launches{0};   // kernel launches issued
+};
+
 // Completion state of one submitted operation (what the reference keeps in an
 // ivalue::Future, fairring/device.cc:303-307,337-348).
 struct Work {
@@ -49,6 +60,8 @@ struct Work {
   std::vector<hipStream_t> doneStreams;
   hipStream_t lastStream = nullptr;
   int device = 0;
+  int64_t seq = 0;  // position among the context's operations
+  std::shared_ptr<Progress> progress;
   std::atomic<int> refs{1};
 };
 
@@ -59,6 +72,7 @@ class Context {
 
   const Layout& layout() const { return layout_; }
   int device() const { return device_; }
+  const Progress& progress() const { return *progress_; }
   std::vector<hipStream_t> streams() const {
     std::vector<hipStream_t> v = reduceStreams_;
     v.insert(v.end(), copyStreams_.begin(), copyStreams_.end());
@@ -146,6 +160,7 @@ class Context {
   std::vector<char> slotUsed_;
   int64_t nextStagingSlot_ = 0;  // round-robin cursor (fairring/device.cc:482)
   int64_t nextSeq_ = 0;          // operation counter for log lines
+  std::shared_ptr<Progress> progress_ = std::make_shared<Progress>();
 
   std::mutex eventMu_;
   std::vector<hipEvent_t> freeEvents_;
@@ -175,6 +190,9 @@ class Context {
   CommandQueue queue_;
   std::thread thread_;
 };
+
+// Process-wide limit of frg_work_wait in seconds (0: none).
+void setWaitTimeout(double seconds);
 
 void setLastError(const std::string& msg);
 const char* lastError();

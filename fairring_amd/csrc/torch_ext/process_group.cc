@@ -2,7 +2,9 @@
 
 #include "process_group.h"
 
+#include <chrono>
 #include <cstdlib>
+#include <thread>
 
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/core/StreamGuard.h>
@@ -84,8 +86,12 @@ void onDone(void* user, int status, void* lastStream) {
 // ---- WorkFairring ---------------------------------------------------------
 
 ProcessGroupFairring::WorkFairring::WorkFairring(
-    c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future)
-    : c10d::Work(/*rank=*/-1, opType), future_(std::move(future)) {}
+    c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future,
+    c10::intrusive_ptr<c10d::Backend> group, frg_ctx* ctx)
+    : c10d::Work(-1, opType),
+      future_(std::move(future)),
+      group_(std::move(group)),
+      ctx_(ctx) {}
 
 ProcessGroupFairring::WorkFairring::~WorkFairring() = default;
 
@@ -98,15 +104,47 @@ std::exception_ptr ProcessGroupFairring::WorkFairring::exception() const {
 }
 
 std::vector<at::Tensor> ProcessGroupFairring::WorkFairring::result() {
-  future_->wait();
+  awaitCompletion();
   return future_->value().toTensorVector();
 }
 
-void ProcessGroupFairring::WorkFairring::synchronize() { future_->wait(); }
+// FAIRRING_WAIT_TIMEOUT_S (seconds, unset or 0: no limit, as in the reference):
+// a wait that sees no completion for that long raises with a report of where
+// the pipeline stands, instead of blocking for good.
+void ProcessGroupFairring::WorkFairring::awaitCompletion() {
+  static const double limit = [] {
+    const char* v = std::getenv("FAIRRING_WAIT_TIMEOUT_S");
+    const double s = v ? std::atof(v) : 0.0;
+    return s > 0.0 ? s : 0.0;
+  }();
+  if (limit > 0.0) {
+    const auto deadline = std::chrono::steady_clock::now() +
+                          std::chrono::duration_cast<std::chrono::steady_clock::duration>(
+                              std::chrono::duration<double>(limit));
+    while (!future_->completed()) {
+      if (std::chrono::steady_clock::now() > deadline) {
+        std::string where = "no context";
+        frg_progress p = {};
+        if (ctx_ != nullptr && frg_get_progress(ctx_, &p) == FRG_OK) {
+          where = std::to_string(p.submitted) + " operations submitted, " +
+                  std::to_string(p.started) + " started by the command thread, " +
+                  std::to_string(p.enqueued) + " fully enqueued, " + std::to_string(p.launches) +
+                  " kernel launches issued";
+        }
+        TORCH_CHECK(false, "fairring: gave up after ", limit,
+                    " s waiting for an operation to complete (", where, ")");
+      }
+      std::this_thread::sleep_for(std::chrono::microseconds(100));
+    }
+  }
+  future_->wait();
+}
+
+void ProcessGroupFairring::WorkFairring::synchronize() { awaitCompletion(); }
 
 // The timeout is ignored, as in the reference (process_group.cc:64-68).
 bool ProcessGroupFairring::WorkFairring::wait(std::chrono::milliseconds /*timeout*/) {
-  future_->wait();
+  awaitCompletion();
   return true;
 }
 
@@ -399,7 +437,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     delete pending;
     TORCH_CHECK(false, "fairring: ", frg_last_error());
   }
-  return c10::make_intrusive<WorkFairring>(opType, std::move(future));
+  return c10::make_intrusive<WorkFairring>(
+      opType, std::move(future),
+      c10::intrusive_ptr<c10d::Backend>::unsafe_reclaim_from_nonowning(this), ctx);
 }
 
 // ---- a group of one: collectives that only move data ------------------------
@@ -532,7 +572,9 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
     delete pending;
     TORCH_CHECK(false, "fairring: ", frg_last_error());
   }
-  return c10::make_intrusive<WorkFairring>(c10d::OpType::ALLREDUCE, std::move(future));
+  return c10::make_intrusive<WorkFairring>(
+      c10d::OpType::ALLREDUCE, std::move(future),
+      c10::intrusive_ptr<c10d::Backend>::unsafe_reclaim_from_nonowning(this), ctx);
 }
 
 }  // namespace fairring

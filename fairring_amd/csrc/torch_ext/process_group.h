@@ -27,7 +27,10 @@ class ProcessGroupFairring : public c10d::Backend {
   // fairring/process_group.h:24-50, fairring/process_group.cc:35-75
   class WorkFairring : public c10d::Work {
    public:
-    WorkFairring(c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future);
+    // `group` and `ctx` (optional) let a wait that gives up say where the
+    // pipeline stands; the work keeps the group, and so the context, alive.
+    WorkFairring(c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future,
+                 c10::intrusive_ptr<c10d::Backend> group = {}, frg_ctx* ctx = nullptr);
     ~WorkFairring() override;
 
     bool isCompleted() override;
@@ -40,7 +43,10 @@ class ProcessGroupFairring : public c10d::Backend {
     c10::intrusive_ptr<c10::ivalue::Future> getFuture() override;
 
    private:
+    void awaitCompletion();
     const c10::intrusive_ptr<c10::ivalue::Future> future_;
+    const c10::intrusive_ptr<c10d::Backend> group_;
+    frg_ctx* const ctx_;
   };
 
   // fairring/process_group.h:52-77, plus the README's slice size

@@ -147,6 +147,13 @@ def reduce_slice_compressed(out, contribs, raw_index=-1, scale_mode=SCALE_NONE, 
         scale_mode, scale, stream.cuda_stream))
 
 
+def set_wait_timeout(seconds):
+    """Process-wide limit of Work.wait() in seconds; 0 = none. A wait that gives
+    up raises FairringError (ERR_NOT_READY) with a report of where the pipeline
+    stands, and can be repeated."""
+    _capi.check(_capi.lib().frg_set_wait_timeout(float(seconds)))
+
+
 class Work:
     """Handle on a submitted operation (WorkFairring, process_group.cc:35-75)."""
 
@@ -287,6 +294,13 @@ class DeviceFairring:
             return Work(wh, keep)
 
         return submit
+
+    def progress(self):
+        """Operations submitted / started by the command thread / fully
+        enqueued, and kernel launches issued, so far."""
+        out = (ctypes.c_int64 * 4)()
+        _capi.check(_capi.lib().frg_get_progress(self._h, ctypes.byref(out)))
+        return dict(submitted=out[0], started=out[1], enqueued=out[2], launches=out[3])
 
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))

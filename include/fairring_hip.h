@@ -228,6 +228,24 @@ FRG_API int frg_allreduce_host(frg_ctx* ctx, void* out,
  * until the operation has been enqueued and its GPU work has finished. */
 FRG_API int frg_work_wait(frg_work* work);
 
+/* Not in the reference, whose wait ignores its timeout (process_group.cc:64-68):
+ * a process-wide limit, in seconds, after which frg_work_wait gives up with
+ * FRG_ERR_NOT_READY and a message that says where the pipeline stands
+ * (operations submitted / started / fully enqueued, launches issued, which
+ * stream has not drained). The work stays valid and can be waited on again.
+ * 0 = no limit (the default, unless FAIRRING_WAIT_TIMEOUT_S is set). */
+FRG_API int frg_set_wait_timeout(double seconds);
+
+/* Where the pipeline stands, for such reports: operations accepted, begun by
+ * the command thread and fully enqueued, and kernel launches issued so far. */
+typedef struct frg_progress {
+  int64_t submitted;
+  int64_t started;
+  int64_t enqueued;
+  int64_t launches;
+} frg_progress;
+FRG_API int frg_get_progress(frg_ctx* ctx, frg_progress* out);
+
 /* WorkFairring::isCompleted (process_group.cc:43-45): FRG_OK once the command
  * thread has enqueued the whole operation, FRG_ERR_NOT_READY before. */
 FRG_API int frg_work_is_completed(frg_work* work);

@@ -8,6 +8,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# A wait that sees no progress for a minute ends in an error that says where the
+# pipeline stands, instead of a silent stall (read when the libraries load).
+os.environ.setdefault("FAIRRING_WAIT_TIMEOUT_S", "60")
+
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")

@@ -103,6 +103,11 @@ struct FakeStream {
     const long target = submitted;
     cv.wait(lock, [&] { return finished >= target; });
   }
+
+  bool idle() {
+    std::lock_guard<std::mutex> lock(mu);
+    return finished >= submitted;
+  }
 };
 
 struct FakeEvent {
@@ -230,6 +235,11 @@ hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) {
     r->cv.notify_all();
   });
   return hipSuccess;
+}
+
+hipError_t hipStreamQuery(hipStream_t stream) {
+  enter("hipStreamQuery");
+  return resolve(stream)->idle() ? hipSuccess : ret(hipErrorNotReady);
 }
 
 hipError_t hipEventQuery(hipEvent_t event) {

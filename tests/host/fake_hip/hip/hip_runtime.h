@@ -48,6 +48,7 @@ const char* hipGetErrorString(hipError_t e);
 
 hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags);
 hipError_t hipStreamSynchronize(hipStream_t stream);
+hipError_t hipStreamQuery(hipStream_t stream);
 hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int flags);
 
 hipError_t hipEventCreate(hipEvent_t* event);

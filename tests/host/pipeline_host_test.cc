@@ -210,6 +210,27 @@ void scenarioBusyProducer() {
   CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
+void scenarioWaitGivesUp() {
+  std::puts("a wait with a time limit gives up with a report, and can be repeated");
+  frg_ctx* ctx = makeCtx(16384, 4096, 2, 1024);
+  auto c = randomContribs(4, 5000, 77);
+  Vec out(5000);
+  auto t = table(c);
+  frg_work* w = nullptr;
+  CHECK(frg_set_wait_timeout(0.2) == FRG_OK);
+  fake_hip_occupy(nullptr, 1500);  // the producer's stream is busy for a while
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 4, 5000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      /*producer=*/nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_ERR_NOT_READY);
+  CHECK(std::strstr(frg_last_error(), "gave up after") != nullptr);
+  CHECK(std::strstr(frg_last_error(), "submitted") != nullptr);
+  CHECK(frg_set_wait_timeout(0) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  frg_work_release(w);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
 void scenarioProducerOrdering() {
   std::puts("the pipeline waits for the producer stream");
   frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
@@ -438,6 +459,7 @@ int main() {
   scenarioResident();
   scenarioPreScaleAndCompressed();
   scenarioBusyProducer();
+  scenarioWaitGivesUp();
   scenarioProducerOrdering();
   scenarioHostStaged();
   scenarioCallback();

@@ -382,6 +382,34 @@ def test_pipeline_host_staged_bf16_default_layout():
     dev.close()
 
 
+def test_wait_with_a_time_limit_gives_up_with_a_report_and_can_be_repeated():
+    _print_case("wait time limit")
+    k, n = 4, 1_000_003
+    xs = [torch.full((n,), float(i + 1), device=DEV) for i in range(k)]
+    out = torch.empty(n, device=DEV)
+    dev = fa.DeviceFairring(0)
+    a = torch.randn(8192, 8192, device=DEV)
+    torch.cuda.synchronize()
+    before = dev.progress()
+    try:
+        fa.set_wait_timeout(0.02)
+        for _ in range(60):          # keeps the producer's stream busy for a few hundred ms
+            a = torch.mm(a, a).clamp_(-1, 1)
+        w = dev.allreduce(out, xs)
+        with pytest.raises(fa.FairringError, match="gave up after") as info:
+            w.wait()
+        assert info.value.code == 5   # FRG_ERR_NOT_READY
+        assert "submitted" in str(info.value)
+    finally:
+        fa.set_wait_timeout(60)
+    w.wait()
+    assert float(out.min()) == 10.0 and float(out.max()) == 10.0
+    after = dev.progress()
+    assert after["submitted"] == before["submitted"] + 1
+    assert after["enqueued"] == after["submitted"] and after["launches"] > before["launches"]
+    dev.close()
+
+
 def test_pipeline_many_small_operations_in_order():
     _print_case("pipeline many ops")
     dev = fa.DeviceFairring(0, slice_size_in_bytes=64 * 1024, max_memory_allocated_in_bytes=256 * 1024)
