@@ -186,13 +186,22 @@ DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch target per 
 LAUNCH_QUANTUM_BYTES = 4096
 
 
-def launch_elems(args, op_elems, slice_elems, elsize):
+def default_launch_bytes(k):
+    """The library's default launch size by number of contributions."""
+    if k <= 2:
+        return 50 * MiB
+    if k <= 8:
+        return DEFAULT_LAUNCH_BYTES
+    return max(100 * MiB // k, 25 * MiB // 8) // 4096 * 4096
+
+
+def launch_elems(args, op_elems, slice_elems, elsize, k=8):
     """Elements of the commonest launch of an operation over `op_elems` elements:
     the pipeline cuts the tensor into launches of the launch target, on 4 KiB
     boundaries from its start and whatever the slice size; the last launch takes
     up to one and a half times that. A negative target means one launch per
     slice."""
-    lb = args.launch_bytes or DEFAULT_LAUNCH_BYTES
+    lb = args.launch_bytes or default_launch_bytes(k)
     if lb < 0:
         return min(slice_elems, op_elems)
     max_elems = (lb - lb % 16) // elsize
@@ -306,7 +315,7 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     step_bytes = (k + 1) * numel * elsize
     value = step_bytes * args.steps / elapsed / 1e9
     roof = roofline_from_records(recs, (k + 1) * elsize,
-                                 launch_elems(args, numel, slice_elems, elsize),
+                                 launch_elems(args, numel, slice_elems, elsize, k),
                                  SPAN_HOW)
     roof["kernel"] = "ksumKernel<%s, SUM, K=%d>" % ("F32Vec" if dtype == "f32" else "Bf16Vec", k)
     step(dev).wait()
@@ -427,7 +436,7 @@ def run_c5(args, np, torch, fa, oracle):
     step_bytes = (k + 1) * numel * 4
     value = step_bytes * args.steps / elapsed / 1e9
     roof = roofline_from_records(recs, (k + 1) * 4,
-                                 launch_elems(args, slice_elems, slice_elems, 4), SPAN_HOW)
+                                 launch_elems(args, slice_elems, slice_elems, 4, k), SPAN_HOW)
     roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
     step(dev).wait()
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)

@@ -17,7 +17,19 @@ constexpr int64_t kAlignment = 8;
 constexpr int64_t kDefaultTotalMemory = 50ll * 1024 * 1024;   // fairring/__init__.py:26
 constexpr int64_t kDefaultPaddingMemory = 1024ll * 1024;      // fairring/__init__.py:30
 constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init__.py:34
-constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;  // per contribution and launch (target)
+// Default bytes of one contribution per launch, by number of contributions.
+// Measured on MI355X (fp32, two reduce streams, GB/s at 6.25 / 12.5 / 25 / 50 MiB):
+// K = 2: 4,530 / 5,990 / 6,290 / 6,340; K = 4: 5,370 / 6,565 / 6,460 / 6,280;
+// K = 8: 6,070 / 6,360 / 6,060 / - ; K = 16 (at 1.6 / 3.1 / 6.25 / 12.5 MiB): 4,930 /
+// 5,340 / 6,220 / 6,110; K = 64 (0.4 / 1.6 / 3.1 / 12.5 MiB): 3,180 / 6,100 / 6,125 / 6,055.
+constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;
+inline constexpr int64_t defaultLaunchBytes(int numContribs) {
+  if (numContribs <= 2) return 50ll * 1024 * 1024;
+  if (numContribs <= 8) return kDefaultMaxLaunchBytes;
+  const int64_t perContrib = 100ll * 1024 * 1024 / numContribs;
+  const int64_t floor = 25ll * 1024 * 1024 / 8;  // 3.125 MiB
+  return (perContrib > floor ? perContrib : floor) / 4096 * 4096;
+}
 constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {

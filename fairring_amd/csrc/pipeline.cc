@@ -118,6 +118,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   // the second stream fills the ramp and drain of the first. Shorter launches
   // still (6 to 8 MiB) gain another 2 % in a bare launch loop but lose it again
   // to per-launch costs here.
+  c->launchBytesByContribs_ = o.max_launch_bytes == 0;  // the default: see defaultLaunchBytes
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
@@ -563,10 +564,12 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   const int64_t elsize = elementSize(req.dtype);
   const int64_t nSlices = numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
   const size_t nStreams = reduceStreams_.size();
-  const int64_t maxLaunchElems = maxLaunchBytes_ > 0 ? maxLaunchBytes_ / elsize : 0;
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
   const int total = static_cast<int>(ptrs.size());
+  const int64_t launchBytes =
+      launchBytesByContribs_ && !req.compressed ? defaultLaunchBytes(total) : maxLaunchBytes_;
+  const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;
   size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
   bool initialFired = false;
   // Reduced in place into a contribution that only a later launch of the chain

@@ -142,6 +142,7 @@ class Context {
   int64_t numSlots_ = 0;
   int64_t slotBytes_ = 0;
   int64_t maxLaunchBytes_ = 0;   // per contribution and launch; 0 = whole slice
+  bool launchBytesByContribs_ = false;  // no size was asked for: it follows the contribution count
   int64_t nextLaunch_ = 0;       // deals launches to the reduce streams
 
   std::vector<hipStream_t> reduceStreams_;
