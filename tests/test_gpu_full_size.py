@@ -94,6 +94,14 @@ def test_c2_full_size_fp32(dev):
         host = [x[lo:hi].cpu().numpy() for x in xs]
         assert_bits_equal(out[lo:hi].cpu().numpy(),
                           oracle.sum_f32(host, oracle.SCALE_MUL, 0.125, threads=16), "slice %d" % idx)
+    # every one of the 1.37 G elements against the at::add chain itself, run by torch on the GPU
+    # (an elementwise fp32 add is the same IEEE operation there as on the CPU)
+    chain = xs[0].clone()
+    for x in xs[1:]:
+        chain.add_(x)
+    chain.mul_(0.125)
+    assert bool(torch.equal(out.view(torch.int32), chain.view(torch.int32)))
+    del chain
     # a checksum of checksums: per-slice sums of the output agree with torch's own reduction of
     # the same chain evaluated on the GPU in fp64 (loose, catches a dropped or duplicated slice)
     acc = torch.zeros((), dtype=torch.float64, device=DEV)
@@ -127,6 +135,12 @@ def test_c4_full_size_bf16(dev):
         host = [bits16(x[lo:hi]) for x in xs]
         assert_bits_equal(bits16(out[lo:hi]),
                           oracle.sum_bf16(host, oracle.SCALE_MUL, 0.125, threads=16), "slice %d" % idx)
+    # every element against the fp32 chain run by torch on the GPU, rounded once to bf16
+    chain = xs[0].float()
+    for x in xs[1:]:
+        chain.add_(x.float())
+    chain.mul_(0.125)
+    assert bool(torch.equal(out.view(torch.int16), chain.to(torch.bfloat16).view(torch.int16)))
 
 
 def test_hook_full_size_bf16_compression_folded_in(dev):
