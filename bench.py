@@ -320,6 +320,19 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     roof["kernel"] = "ksumKernel<%s, SUM, K=%d>" % ("F32Vec" if dtype == "f32" else "Bf16Vec", k)
     step(dev).wait()
     checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, dtype, scale)
+    # and every element against the at::add chain itself, run by torch on the GPU
+    chain = xs[0].float() if dtype != "f32" else xs[0].clone()
+    for x in xs[1:]:
+        chain.add_(x.float() if dtype != "f32" else x)
+    if scale:
+        chain.mul_(1.0 / k)
+    same = torch.equal(out.view(torch.int32 if dtype == "f32" else torch.int16),
+                       (chain if dtype == "f32" else chain.to(torch.bfloat16)).view(
+                           torch.int32 if dtype == "f32" else torch.int16))
+    del chain
+    if not same:
+        raise SystemExit("parity FAILED against the at::add chain on the GPU")
+    checked = "%s; every element equal to torch's at::add chain on the GPU" % checked
     layout = dev.layout
     dev.close()
     name = {"c2": "configs[1]", "c4": "configs[3]",
