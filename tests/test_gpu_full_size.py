@@ -209,6 +209,40 @@ def test_c3_full_size_server_side_from_pinned_host(dev):
     assert_bits_equal(out.cpu().numpy(), chain.numpy())
 
 
+def test_c5_ddp_bucket_stream_inputs_ready(dev):
+    # configs[4] with the inputs finished before the buckets are submitted (what bench.py
+    # --workload c5 times): the 1.37 G gradient as 25 MiB buckets (first one 1 MiB) released from
+    # the end to the start, one allreduce per bucket, 8 contributions each, pool = 2 x 25 MiB
+    print("[case] c5 bucket stream, inputs ready", flush=True)
+    numel, k = 1_370_000_000, 8
+    se = SLICE // 4
+    spans, hi, size = [], numel, MiB // 4
+    while hi > 0:
+        lo = max(0, hi - size)
+        spans.append((lo, hi))
+        hi, size = lo, se
+    assert len(spans) == 211
+    g = torch.Generator(device=DEV)
+    g.manual_seed(5)
+    xs = [torch.empty(numel, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    out = torch.zeros(numel, device=DEV)
+    torch.cuda.synchronize()
+    works = [dev.allreduce(out[lo:hi], [x[lo:hi] for x in xs], scale_mode=fa.SCALE_MUL, scale=0.125)
+             for lo, hi in spans]
+    for w in works:
+        w.wait()
+    chain = xs[0].clone()
+    for x in xs[1:]:
+        chain.add_(x)
+    chain.mul_(0.125)
+    assert bool(torch.equal(out.view(torch.int32), chain.view(torch.int32)))
+    for i in (0, 1, 105, 210):
+        lo, hi = spans[i]
+        host = [x[lo:hi].cpu().numpy() for x in xs]
+        assert_bits_equal(out[lo:hi].cpu().numpy(),
+                          oracle.sum_f32(host, oracle.SCALE_MUL, 0.125, threads=16), "bucket %d" % i)
+
+
 @pytest.mark.skip(reason="went silent for 180 s on its only GPU run (killed by the harness, GPU "
                          "still answering) while 211 operations were submitted with the producer "
                          "(default) stream still busy; no cause found by reading the code, so the "
