@@ -185,6 +185,52 @@ void scenarioPreScaleAndCompressed() {
   CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
+int64_t launchesSoFar(frg_ctx* ctx) {
+  frg_progress p = {};
+  CHECK(frg_get_progress(ctx, &p) == FRG_OK);
+  return p.launches;
+}
+
+void scenarioLaunchPartition() {
+  std::puts("launch partition: sizes cut from the tensor on tile boundaries, 1.5x rule, per slice");
+  struct Case {
+    int64_t launchBytes, sliceBytes, numel;
+    int64_t wantLaunches;
+  };
+  // 16 KiB launches = 4096 fp32 elements each (a multiple of the 1024-element tile)
+  const Case cases[] = {
+      {16384, 4096, 4096, 1},          // exactly one launch
+      {16384, 4096, 6144, 1},          // 1.5 x the launch size: still one
+      {16384, 4096, 6145, 2},          // a little more: 4096 + 2049
+      {16384, 4096, 40960 + 100, 10},  // nine of 4096, the last takes 4096 + 100
+      {16384, 65536, 40960 + 100, 10},  // the slice size does not matter
+      {-1, 4096, 10000, 10},           // one launch per slice: ceil(10000 / 1024)
+      {-1, 65536, 10000, 1},
+      {6000, 65536, 10000, 10},        // 1496 elements round down to one 1024-element tile: 9 + a rest of 784
+  };
+  for (const Case& cs : cases) {
+    frg_ctx* ctx = makeCtx(2 * cs.sliceBytes, cs.sliceBytes, 2, cs.launchBytes);
+    auto c = randomContribs(3, cs.numel, 5);
+    Vec out(static_cast<size_t>(cs.numel));
+    auto t = table(c);
+    frg_work* w = nullptr;
+    const int64_t before = launchesSoFar(ctx);
+    CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, cs.numel, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                        1.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+    CHECK(frg_work_wait(w) == FRG_OK);
+    CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+    const int64_t got = launchesSoFar(ctx) - before;
+    if (got != cs.wantLaunches) {
+      std::fprintf(stderr, "launch bytes %lld, slice %lld, numel %lld: %lld launches, expected %lld\n",
+                   (long long)cs.launchBytes, (long long)cs.sliceBytes, (long long)cs.numel,
+                   (long long)got, (long long)cs.wantLaunches);
+      std::abort();
+    }
+    frg_work_release(w);
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
 void scenarioBusyProducer() {
   std::puts("many operations submitted while the producer stream is busy");
   frg_ctx* ctx = makeCtx(2 * 65536, 65536, 2, 32768);
@@ -457,6 +503,7 @@ void scenarioConcurrentSubmitters() {
 
 int main() {
   scenarioResident();
+  scenarioLaunchPartition();
   scenarioPreScaleAndCompressed();
   scenarioBusyProducer();
   scenarioWaitGivesUp();
