@@ -102,3 +102,38 @@ dist.destroy_process_group()
     r = _run(code)
     assert r.returncode == 0, r.stderr
     assert "backend fairring 1" in r.stdout
+
+
+def test_data_moving_collectives_for_a_group_of_one_on_cpu_tensors():
+    # nothing moves in a group of one, so these need no GPU: enough to build DDP on the backend
+    pg = make_pg(0, 1)
+    x = torch.arange(100, dtype=torch.float32)
+    w = pg.broadcast([x])
+    assert w.wait() and w.is_completed() and w.is_success()
+    out = torch.zeros(100)
+    pg.allgather([[out]], [x]).wait()
+    assert torch.equal(out, x)
+    out2 = torch.zeros(4, 25)
+    pg._allgather_base(out2, x).wait()
+    assert torch.equal(out2.reshape(-1), x)
+    assert pg.barrier().wait()
+    pg2 = make_pg(1, 2)
+    for call in (lambda: pg2.broadcast([x]), lambda: pg2.allgather([[out, out]], [x]),
+                 lambda: pg2._allgather_base(torch.zeros(200), x), pg2.barrier):
+        with pytest.raises(RuntimeError, match="needs a transport"):
+            call()
+
+
+def test_hook_entry_points_exist_and_refuse_other_backends():
+    from fairring_amd import ddp_comm_hooks
+    pg = make_pg(0, 1)
+    assert hasattr(pg, "_allreduce_pre_divided") and hasattr(pg, "_allreduce_compressed")
+
+    class Bucket:
+        def buffer(self):
+            return torch.zeros(4)
+
+    for hook in (ddp_comm_hooks.allreduce_hook, ddp_comm_hooks.bf16_compress_hook,
+                 ddp_comm_hooks.fp16_compress_hook):
+        with pytest.raises(RuntimeError, match="'fairring' backend"):
+            hook(object(), Bucket())
