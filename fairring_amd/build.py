@@ -56,6 +56,22 @@ def build(extra_flags=(), output=LIB_PATH, verbose=False):
     return output
 
 
+def build_c_client(output=None):
+    """The plain-C client of the ABI used by the tests (tests/host/abi_client.c):
+    gcc, linked against the library above and the HIP runtime, no PyTorch."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "host", "abi_client.c")
+    output = output or os.path.join(root, "tests", "host", "abi_client")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c99", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__", "-I", os.path.join(rocm, "include"),
+           "-o", output, src, "-L", HERE, "-lfairring_hip", "-L", os.path.join(rocm, "lib"),
+           "-lamdhip64", "-Wl,-rpath,$ORIGIN/../../fairring_amd", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("gcc failed:\n" + proc.stdout)
+    return output
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
     sys.exit(0)

@@ -118,3 +118,37 @@ def test_dense_check():
     assert dense(torch.zeros(2, 3, 4).permute(2, 0, 1))
     assert not dense(torch.zeros(3, 4)[:, :2]) and not dense(torch.zeros(8)[::2])
     assert dense(torch.zeros(0))
+
+
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header must compile as strict C99 on its own
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not available")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "fairring_hip.h"\n'
+                   "int probe(void) { frg_options o = {0}; frg_progress p = {0};\n"
+                   "  return (int)(o.num_machines + p.launches) + FRG_SCALE_PRE_DIV + FRG_I8; }\n")
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                        "-I", os.path.join(ROOT, "include"), str(src)],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+
+
+def test_c_client_builds_and_fails_cleanly_without_a_gpu(tmp_path):
+    import shutil
+    import subprocess
+    import torch
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not available")
+    from fairring_amd import build as hip_build
+    exe = hip_build.build_c_client(str(tmp_path / "abi_client"))
+    # rpath of the copy does not reach the library: point the loader at it
+    env = dict(os.environ, LD_LIBRARY_PATH=os.path.join(ROOT, "fairring_amd") + ":" +
+               os.environ.get("LD_LIBRARY_PATH", ""))
+    r = subprocess.run([exe, "2", "100"], capture_output=True, text=True, timeout=120, env=env)
+    if torch.cuda.is_available():
+        assert r.returncode == 0 and "abi client ok" in r.stdout, r.stderr
+    else:
+        assert r.returncode == 2 and "abi 0.1" in r.stdout     # the HIP runtime finds no device
