@@ -236,6 +236,34 @@ def test_pipeline_resident_independent_of_slicing(slice_bytes, total, streams):
     dev.close()
 
 
+def test_block_stream_orders_a_consumer_behind_a_long_operation():
+    # hundreds of launches over three streams are still in flight when the consumer is enqueued
+    # on the caller's stream right behind block_stream(): it must see the finished result
+    _print_case("block_stream, long operation")
+    k, n = 8, 100_000_007
+    g = torch.Generator(device=DEV)
+    g.manual_seed(77)
+    xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    out = torch.zeros(n, device=DEV)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=4 * MiB, max_memory_allocated_in_bytes=8 * MiB,
+                            num_reduce_streams=3, max_launch_bytes=MiB)
+    torch.cuda.synchronize()
+    w = dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+    w.block_stream()
+    doubled = out * 2           # on torch's current stream, no host wait in between
+    nonzero = int(torch.count_nonzero(doubled))
+    w.wait()
+    chain = xs[0].clone()
+    for x in xs[1:]:
+        chain.add_(x)
+    chain.mul_(0.125)
+    assert bool(torch.equal(out.view(torch.int32), chain.view(torch.int32)))
+    assert bool(torch.equal(doubled.view(torch.int32), (chain * 2).view(torch.int32)))
+    assert nonzero > n - 100
+    assert dev.progress()["launches"] >= 380
+    dev.close()
+
+
 def test_pipeline_more_than_64_contributions():
     _print_case("pipeline K=100")
     k, n = 100, 50_003
