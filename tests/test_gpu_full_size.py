@@ -143,6 +143,25 @@ def test_c4_full_size_bf16(dev):
     assert bool(torch.equal(out.view(torch.int16), chain.to(torch.bfloat16).view(torch.int16)))
 
 
+def test_more_than_two_to_the_31_elements_in_one_launch_and_through_the_pipeline(dev):
+    # element indices beyond 32 bits: 3,000,000,017 uint8 elements per contribution, once as one
+    # launch and once through the pipeline, against torch's own wrap-around add on the GPU
+    print("[case] > 2^31 elements", flush=True)
+    n = 3_000_000_017
+    g = torch.Generator(device=DEV)
+    g.manual_seed(9)
+    xs = [torch.randint(0, 256, (n,), dtype=torch.uint8, device=DEV, generator=g) for _ in range(3)]
+    want = xs[0] + xs[1] + xs[2]            # uint8 arithmetic wraps modulo 256
+    out = torch.zeros(n + 64, dtype=torch.uint8, device=DEV)
+    fa.reduce_slice(out[32:32 + n], xs)
+    torch.cuda.synchronize()
+    assert bool(torch.equal(out[32:32 + n], want))
+    assert int(out[:32].sum()) == 0 and int(out[32 + n:].sum()) == 0
+    out.zero_()
+    dev.allreduce(out[32:32 + n], xs, op=fa.MAX).wait()
+    assert bool(torch.equal(out[32:32 + n], torch.maximum(torch.maximum(xs[0], xs[1]), xs[2])))
+
+
 def test_hook_full_size_bf16_compression_folded_in(dev):
     # the 1.37 G fp32 gradient with torch's bf16 compression hook folded into the reduction:
     # own bucket compressed in registers, 7 peers' bf16 tensors, result widened in place
