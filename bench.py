@@ -45,7 +45,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy", "hook"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy", "hook", "smallops"])
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
     ap.add_argument("--k", type=int, default=0, help="override the number of contributions")
     ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
@@ -526,6 +526,85 @@ def run_hook(args, np, torch, fa, oracle):
     return value, elapsed, cfg, roof, checked, None, "bf16"
 
 
+def run_small_ops(args, torch, fa):
+    """Per-operation cost at bucket sizes where the kernel is short (a DDP step's
+    first 1 MiB bucket and its small ones): what the caller's thread pays per
+    call, call -> wait -> device idle, and the sustained back-to-back rate,
+    through the ctypes mirror of the ABI and, when the torch extension is built,
+    through the process group. Prints its own JSON line (operations per second)."""
+    import datetime
+    import time
+    k = args.k or 8
+    sizes = [1024, 262144]
+    reps, burst = 200, max(args.steps, 1) * 100
+
+    def measure(submit, wait_last):
+        out = {}
+        for numel in sizes:
+            call = submit(numel)
+            wait_last(call())
+            torch.cuda.synchronize()
+            lat = []
+            for _ in range(reps):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                wait_last(call())
+                torch.cuda.synchronize()
+                lat.append(time.perf_counter() - t0)
+            lat.sort()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(burst):
+                w = call()
+            t1 = time.perf_counter()
+            wait_last(w)
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            out[str(numel)] = {"latency_us_median": round(lat[reps // 2] * 1e6, 1),
+                               "latency_us_p90": round(lat[reps * 9 // 10] * 1e6, 1),
+                               "caller_us_per_op": round((t1 - t0) / burst * 1e6, 1),
+                               "sustained_us_per_op": round((t2 - t0) / burst * 1e6, 1)}
+        return out
+
+    dev = fa.DeviceFairring(0)
+
+    def submit_abi(numel):
+        xs = [torch.zeros(numel, device="cuda:0") for _ in range(k)]
+        out = torch.empty(numel, device="cuda:0")
+        return lambda: dev.allreduce(out, xs)
+
+    report = {"abi_ctypes": measure(submit_abi, lambda w: w.wait())}
+    dev.close()
+    try:
+        import torch.distributed as dist
+
+        import fairring  # noqa: F401  (registers the backend, loads the extension)
+        from fairring_amd import _fairring
+    except ImportError:
+        _fairring = None
+    if _fairring is not None:
+        o = _fairring.ProcessGroup.Options(
+            max_memory_allocated_in_bytes=args.total_memory,
+            max_padding_allocated_in_bytes=MiB, min_parallelism=2, is_high_priority_stream=True,
+            timeout=datetime.timedelta(seconds=60), slice_size_in_bytes=args.slice_bytes)
+        pg = _fairring.ProcessGroup(dist.HashStore(), 0, k, o)
+
+        def submit_pg(numel):
+            own = torch.zeros(numel, device="cuda:0")
+            pg._set_simulated_peer_contributions(
+                [torch.zeros(numel, device="cuda:0") for _ in range(k - 1)])
+            return lambda: pg.allreduce([own])
+
+        report["process_group"] = measure(submit_pg, lambda w: w.wait())
+    best = report.get("process_group", report["abi_ctypes"])[str(sizes[0])]
+    print(json.dumps({
+        "metric": "small allreduce operations per second, %d-way fp32, back to back" % k,
+        "value": round(1e6 / best["sustained_us_per_op"], 1), "unit": "operations/s",
+        "n_gpus": 1, "steps": burst, "warmup": 1, "higher_is_better": True,
+        "dtype": "f32", "data": "synthetic: zeros", "vs_baseline": None,
+        "config": {"workload": "smallops", "k": k, "elements": sizes}, "detail": report}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -546,6 +625,9 @@ def main():
     if args.blocks_per_cu:
         _capi.lib().frg_set_tuning(args.blocks_per_cu)
 
+    if args.workload == "smallops":
+        run_small_ops(args, torch, fa)
+        return
     if args.workload in ("c2", "copy"):
         value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,
                                                                        oracle, "f32")
