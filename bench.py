@@ -596,6 +596,32 @@ def run_small_ops(args, torch, fa):
             return lambda: pg.allreduce([own])
 
         report["process_group"] = measure(submit_pg, lambda w: w.wait())
+    # the one-launch entry point on the caller's stream: eager, and the same loop captured
+    # once into a HIP graph and replayed (it allocates nothing and records no event)
+    nb = 64
+    xs = [[torch.zeros(sizes[1], device="cuda:0") for _ in range(k)] for _ in range(nb)]
+    outs = [torch.empty(sizes[1], device="cuda:0") for _ in range(nb)]
+
+    def loop():
+        for o, c in zip(outs, xs):
+            fa.reduce_slice(o, c, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+
+    loop()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loop()
+    rounds = max(burst // nb, 1)
+    direct = {}
+    for name, fn in (("eager", loop), ("graph_replay", graph.replay)):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(rounds):
+            fn()
+        torch.cuda.synchronize()
+        direct[name + "_us_per_launch"] = round((time.perf_counter() - t0) / (rounds * nb) * 1e6, 2)
+    report["reduce_slice_%d_elements" % sizes[1]] = direct
     best = report.get("process_group", report["abi_ctypes"])[str(sizes[0])]
     print(json.dumps({
         "metric": "small allreduce operations per second, %d-way fp32, back to back" % k,

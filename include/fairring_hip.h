@@ -109,7 +109,12 @@ FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
  * integer types and MAX, but a bf16 / fp16 SUM then rounds once per launch.
  * frg_allreduce chains those through fp32 accumulators instead and rounds once
  * for any K. n == 0 is a no-op (device.cc:120-122). Asynchronous: returns
- * after enqueueing. */
+ * after enqueueing. The call allocates nothing, records no event and clears
+ * no memory, so it may be issued on a stream that is being captured into a
+ * HIP graph (the pointer table is copied into the launch, the graph replays
+ * on the captured addresses); the same holds for frg_reduce_slice_compressed.
+ * The pipeline entry points (frg_allreduce*) hand work to another thread and
+ * are not for capture. */
 FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);
