@@ -134,11 +134,85 @@ __device__ __forceinline__ void compressedOne(void* out, const float* raw, const
   }
 }
 
+// The hook's own shapes (a raw fp32 bucket, KW = 1, 3 or 7 peers, fp32 output,
+// no scale or the multiply by 1/K) with everything but the own term's place
+// fixed at compile time: all loads are issued first, the fold is straight-line
+// code with one uniform branch per position the own term can take, and the
+// body is a tenth of the general one's code (which matters when a launch
+// lasts 20 us and every CU starts it with a cold instruction cache). Same
+// arithmetic, in the same order, as compressedOne.
+template <typename W, int KW, int SC>
+__device__ __forceinline__ void compressedFixed(float* out, const float* raw, const Ptrs<KW>& wire,
+                                                int rawPos, float scale, int64_t elemBase,
+                                                unsigned int lane) {
+  using vec_t = typename W::vec_t;
+  using elem_t = typename W::elem_t;
+  using Side = Fp32Side<W::kLanes>;
+  const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
+  const typename Side::regs_t rawRegs = Side::load(raw + elemBase, lane);
+  vec_t v[KW];
+#pragma unroll
+  for (int k = 0; k < KW; ++k) {
+    const char* b = reinterpret_cast<const char*>(static_cast<const elem_t*>(wire.p[k]) + elemBase);
+    v[k] = ldStream(reinterpret_cast<const vec_t*>(b + laneBytes));
+  }
+  // buffer.to(wire) then div_(world) in the wire type: two roundings
+  float own[W::kLanes];
+  Side::unpack(rawRegs, own);
+#pragma unroll
+  for (int j = 0; j < W::kLanes; ++j) {
+    float c = W::roundStorage(own[j]);
+    if (SC == FRG_SCALE_MUL) c = W::roundStorage(c * scale);
+    own[j] = c;
+  }
+  float acc[W::kLanes];
+  float f[W::kLanes];
+  W::unpack(v[0], f);
+  if (rawPos == 0) {
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) acc[j] = own[j] + f[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) acc[j] = f[j];
+  }
+#pragma unroll
+  for (int k = 1; k < KW; ++k) {
+    if (k == rawPos) {
+#pragma unroll
+      for (int j = 0; j < W::kLanes; ++j) acc[j] = acc[j] + own[j];
+    }
+    W::unpack(v[k], f);
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) acc[j] = acc[j] + f[j];
+  }
+  if (rawPos == KW) {
+#pragma unroll
+    for (int j = 0; j < W::kLanes; ++j) acc[j] = acc[j] + own[j];
+  }
+  // one rounding to the wire type, stored widened
+#pragma unroll
+  for (int j = 0; j < W::kLanes; ++j) acc[j] = W::roundStorage(acc[j]);
+  Side::store(out + elemBase, lane, acc);
+}
+
+// KW > 0: the fixed shape above (OUT32, raw term present, scale mode SC);
+// KW == 0: the general body.
+template <typename W, bool OUT32, int KW, int SC>
+__device__ __forceinline__ void compressedLane(void* out, const float* raw, const Ptrs<KW>& wire,
+                                               int Kw, int rawPos, int scaleMode, float scale,
+                                               int64_t elemBase, unsigned int lane) {
+  if constexpr (KW > 0) {
+    compressedFixed<W, KW, SC>(static_cast<float*>(out), raw, wire, rawPos, scale, elemBase, lane);
+  } else {
+    compressedOne<W, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase, lane);
+  }
+}
+
 // Same dealing of tiles, remainder pieces and ragged edges as the plain
 // reduction kernel; a "vector" is a lane's group of 8 elements.
-template <typename WV, typename WS, bool OUT32>
+template <typename WV, typename WS, bool OUT32, int KW, int SC>
 __global__ void __launch_bounds__(kBlock)
-    compressedKernel(void* out, const float* raw, Ptrs<0> wire, int Kw, int rawPos, int scaleMode,
+    compressedKernel(void* out, const float* raw, Ptrs<KW> wire, int Kw, int rawPos, int scaleMode,
                      float scale, int64_t head, int64_t nvec, int64_t tail, int64_t roundTiles,
                      int64_t pieces) {
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
@@ -147,8 +221,8 @@ __global__ void __launch_bounds__(kBlock)
     const int64_t elemBase = head + t * kTile * WV::kLanes;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      compressedOne<WV, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
-                               threadIdx.x + u * kBlock);
+      compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
+                                        threadIdx.x + u * kBlock);
     }
   }
   const int64_t restBase = roundTiles * kTile;
@@ -160,8 +234,8 @@ __global__ void __launch_bounds__(kBlock)
     for (int u = 0; u < kPiece; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
       if (v0 + lane < nvec) {
-        compressedOne<WV, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale,
-                                 head + v0 * WV::kLanes, lane);
+        compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale,
+                                          head + v0 * WV::kLanes, lane);
       }
     }
   }
@@ -169,24 +243,27 @@ __global__ void __launch_bounds__(kBlock)
     const int64_t e = threadIdx.x < head
                           ? static_cast<int64_t>(threadIdx.x)
                           : head + nvec * WV::kLanes + (threadIdx.x - head);
-    compressedOne<WS, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, e, 0u);
+    compressedLane<WS, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, e, 0u);
   }
 }
 
-template <typename WV, typename WS, bool OUT32>
-hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptrs<0>& wire, int Kw,
+template <typename WV, typename WS, bool OUT32, int KW = 0, int SC = 0>
+hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptrs<0>& all, int Kw,
                             int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
                             hipStream_t stream) {
+  Ptrs<KW> wire;
+  for (int k = 0; k < (KW > 0 ? KW : kMaxContribsPerLaunch); ++k) wire.p[k] = all.p[k];
   const GridPlan plan = planGrid(nvec, a.K, numCus);
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
-    hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32>),
+    hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
                           dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream,
                           a.startEvent, a.stopEvent, 0, a.out, raw, wire, Kw, rawPos, a.scale_mode,
                           a.scale, head, nvec, tail, plan.roundTiles, plan.pieces);
   } else {
-    hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32>), dim3(static_cast<unsigned>(plan.grid)),
-                       dim3(kBlock), 0, stream, a.out, raw, wire, Kw, rawPos, a.scale_mode,
-                       a.scale, head, nvec, tail, plan.roundTiles, plan.pieces);
+    hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
+                       dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream, a.out, raw,
+                       wire, Kw, rawPos, a.scale_mode, a.scale, head, nvec, tail, plan.roundTiles,
+                       plan.pieces);
   }
   return hipGetLastError();
 }
@@ -196,6 +273,27 @@ hipError_t dispatchOut(const CompressedArgs& a, const float* raw, const Ptrs<0>&
                        int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
                        hipStream_t stream) {
   if (nvec > 0) {
+    // the hook's own shapes: a raw fp32 bucket and 1, 3 or 7 peers, fp32 output,
+    // no scale or the multiply by 1/K
+    if (a.out_dtype == FRG_F32 && raw != nullptr &&
+        (a.scale_mode == FRG_SCALE_NONE || a.scale_mode == FRG_SCALE_MUL)) {
+      const bool mul = a.scale_mode == FRG_SCALE_MUL;
+#define FRG_FIXED_CASE(KK)                                                                        \
+  case KK:                                                                                        \
+    return mul ? launchCompressed<WV, WS, true, KK, FRG_SCALE_MUL>(a, raw, wire, Kw, rawPos, head, \
+                                                                   nvec, tail, numCus, stream)     \
+               : launchCompressed<WV, WS, true, KK, FRG_SCALE_NONE>(a, raw, wire, Kw, rawPos,      \
+                                                                    head, nvec, tail, numCus,      \
+                                                                    stream);
+      switch (Kw) {
+        FRG_FIXED_CASE(1)
+        FRG_FIXED_CASE(3)
+        FRG_FIXED_CASE(7)
+        default:
+          break;
+      }
+#undef FRG_FIXED_CASE
+    }
     return a.out_dtype == FRG_F32
                ? launchCompressed<WV, WS, true>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus,
                                                 stream)

@@ -567,6 +567,8 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
   const int total = static_cast<int>(ptrs.size());
+  // (the compressed reduction keeps the 12.5 MiB of wire per contribution: sizing its
+  // launches by the bytes they move, 10.2 MiB for the 8-way hook, measured within noise)
   const int64_t launchBytes =
       launchBytesByContribs_ && !req.compressed ? defaultLaunchBytes(total) : maxLaunchBytes_;
   const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;

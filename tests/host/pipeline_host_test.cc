@@ -14,7 +14,15 @@
 #include <thread>
 #include <vector>
 
+#include "../../fairring_amd/csrc/layout.h"
 #include "../../include/fairring_hip.h"
+
+// The default launch sizes, pinned: 50 MiB up to 2 contributions, 12.5 MiB up to
+// 8, about 100 MiB / K above.
+static_assert(frg::defaultLaunchBytes(2) == 50ll << 20);
+static_assert(frg::defaultLaunchBytes(8) == 13107200);
+static_assert(frg::defaultLaunchBytes(16) == 6553600);
+static_assert(frg::defaultLaunchBytes(64) == 3276800);
 
 #define CHECK(cond)                                                                  \
   do {                                                                               \
