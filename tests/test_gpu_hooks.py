@@ -54,7 +54,7 @@ def bits_of(t):
 
 # ---- pre-scale -------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("k", [1, 2, 3, 6, 8, 17, 64])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 6, 8, 17, 64])
 @pytest.mark.parametrize("n", [5, 4099, 262147])
 def test_pre_scale_f32(k, n):
     _print_case("pre-scale f32", k, n)
@@ -73,7 +73,7 @@ def test_pre_scale_f32(k, n):
 
 
 @pytest.mark.parametrize("kind,tdt", WIRES + [("f64", torch.float64)])
-@pytest.mark.parametrize("k", [2, 7, 8, 33])
+@pytest.mark.parametrize("k", [2, 4, 7, 8, 33])
 def test_pre_scale_other_floating_types(kind, tdt, k):
     _print_case("pre-scale", kind, k)
     n = 70001
@@ -148,7 +148,7 @@ def _compressed_case(wire, tdt, k, n, raw, rng, shift=0, in_place=True, out_f32=
 
 
 @pytest.mark.parametrize("wire,tdt", WIRES)
-@pytest.mark.parametrize("k", [1, 2, 3, 8, 9, 17, 64])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 8, 9, 17, 64])
 @pytest.mark.parametrize("n", [1, 7, 8, 9, 2051, 262147])
 def test_compressed_sizes(wire, tdt, k, n):
     _print_case("compressed sizes", wire, k, n)
@@ -156,6 +156,25 @@ def test_compressed_sizes(wire, tdt, k, n):
     for raw in sorted({0, k // 2, k - 1}):
         got, want = _compressed_case(wire, tdt, k, n, raw, rng)
         assert_bits_equal(got, want, "%s k %d n %d raw %d" % (wire, k, n, raw))
+
+
+@pytest.mark.parametrize("wire,tdt", WIRES)
+@pytest.mark.parametrize("k", [2, 4, 8])
+def test_compressed_hook_shapes_with_the_own_term_at_every_rank(wire, tdt, k):
+    # the shapes with compile-time variants (raw fp32 bucket + 1, 3 or 7 peers, fp32 output):
+    # the own term joins the fold at its rank's place, whichever that is; a ragged length so
+    # that the element-wise edges run the same variant
+    _print_case("compressed hook shapes", wire, k)
+    rng = np.random.default_rng(8800 + k)
+    for raw in range(k):
+        for mode in ("mul", "none"):         # the two scale modes those variants are compiled for
+            for in_place in (True, False):
+                got, want = _compressed_case(wire, tdt, k, 70003, raw, rng, in_place=in_place,
+                                             mode=mode)
+                assert_bits_equal(got, want, "%s k %d raw %d %s in place %s" % (
+                    wire, k, raw, mode, in_place))
+    got, want = _compressed_case(wire, tdt, k, 70003, k - 1, rng, shift=3, mode="mul")
+    assert_bits_equal(got, want, "%s k %d off the 16-byte boundary" % (wire, k))
 
 
 @pytest.mark.parametrize("wire,tdt", WIRES)
