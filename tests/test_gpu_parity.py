@@ -563,3 +563,65 @@ def test_pipeline_other_types_unaligned(kind, tdt):
                       half=kind == "f16")
     assert int(torch.count_nonzero(out[:shift].view(torch.uint8) if tdt != torch.uint8 else out[:shift])) == 0
     dev.close()
+
+
+def test_pipeline_submitters_on_several_threads():
+    # the reference is called from whichever thread autograd runs a bucket's hook on
+    # (fairring/process_group.cc:131-155 takes no lock of the caller's): four threads share one
+    # context, each producing its inputs on a stream of its own and submitting 40 operations of
+    # mixed sizes, types and contribution counts; every result against torch's own chain on the
+    # GPU (fp32, int32) or the single-rounding rule (bf16)
+    import threading
+    _print_case("pipeline submitters on several threads")
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=256 * 1024, max_memory_allocated_in_bytes=MiB,
+                            num_reduce_streams=2)
+    failures = []
+
+    def worker(tid):
+        try:
+            torch.cuda.set_device(0)
+            gen = torch.Generator(device=DEV)
+            gen.manual_seed(500 + tid)
+            side = torch.cuda.Stream()
+            rng = np.random.default_rng(600 + tid)
+            pending = []
+            with torch.cuda.stream(side):
+                for i in range(40):
+                    k = int(rng.integers(1, 12))
+                    n = int(rng.integers(1, 400_000))
+                    kind = ("f32", "bf16", "i32")[int(rng.integers(0, 3))]
+                    if kind == "i32":
+                        xs = [torch.randint(-1000, 1000, (n,), dtype=torch.int32, device=DEV,
+                                            generator=gen) for _ in range(k)]
+                        want = xs[0].clone()
+                        for x in xs[1:]:
+                            want += x
+                    else:
+                        xs = [torch.randn(n, device=DEV, generator=gen) * 0.01 for _ in range(k)]
+                        if kind == "bf16":
+                            xs = [x.to(torch.bfloat16) for x in xs]
+                        want = xs[0].float()
+                        for x in xs[1:]:
+                            want = want + x.float()
+                        want = want.to(xs[0].dtype)
+                    out = torch.empty_like(xs[0])
+                    w = dev.allreduce(out, xs)          # ordered after this thread's side stream
+                    pending.append((i, kind, k, n, w, out, want, xs))
+                for i, kind, k, n, w, out, want, xs in pending:
+                    w.wait()
+                    side.synchronize()
+                    view = torch.int16 if kind == "bf16" else torch.int32
+                    if not bool(torch.equal(out.view(view), want.view(view))):
+                        failures.append("thread %d op %d: %s k %d n %d" % (tid, i, kind, k, n))
+        except Exception as e:  # noqa: BLE001  (reported by the main thread)
+            failures.append("thread %d: %r" % (tid, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a submitter thread did not finish"
+    assert not failures, failures[:5]
+    assert dev.progress()["submitted"] >= 160
+    dev.close()
