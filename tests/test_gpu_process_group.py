@@ -189,6 +189,51 @@ def test_data_moving_collectives_exist_for_a_group_of_one_only():
             call()
 
 
+def test_allreduce_from_two_threads_and_futures_with_callbacks():
+    # two threads share the group (its submit path is serialised inside); each reduces its
+    # own tensors 30 times and chains a Python callback on every future, which the command
+    # thread runs: no result may be lost, late or mixed up
+    import threading
+    print("[case] pg two threads", flush=True)
+    size, rank, n = 4, 1, 200_003
+    pg = make_pg(rank, size, slice_bytes=256 * 1024, total=MiB)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(91)
+    peers = [torch.randn(n, device=DEV, generator=gen) * 0.01 for _ in range(size - 1)]
+    pg._set_simulated_peer_contributions(peers)
+    torch.cuda.synchronize()
+    failures, seen = [], []
+
+    def worker(tid):
+        try:
+            g = torch.Generator(device=DEV)
+            g.manual_seed(92 + tid)
+            for i in range(30):
+                own = torch.randn(n, device=DEV, generator=g) * 0.01
+                chain = ordered(own.clone(), peers, rank)
+                want = chain[0].clone()
+                for c in chain[1:]:
+                    want += c
+                fut = pg.allreduce([own]).get_future().then(
+                    lambda f, tag=(tid, i): (seen.append(tag), f.value()[0])[1])
+                got = fut.wait()
+                torch.cuda.current_stream().synchronize()
+                if got.data_ptr() != own.data_ptr() or not bool(
+                        torch.equal(got.view(torch.int32), want.view(torch.int32))):
+                    failures.append("thread %d op %d" % (tid, i))
+        except Exception as e:  # noqa: BLE001
+            failures.append("thread %d: %r" % (tid, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not any(t.is_alive() for t in threads), "a thread did not finish"
+    assert not failures, failures[:5]
+    assert sorted(seen) == [(t, i) for t in range(2) for i in range(30)]
+
+
 def test_missing_peers_is_a_loud_error():
     print("[case] pg missing peers", flush=True)
     pg = make_pg(0, 2)
