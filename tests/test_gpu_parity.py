@@ -625,3 +625,27 @@ def test_pipeline_submitters_on_several_threads():
     assert not failures, failures[:5]
     assert dev.progress()["submitted"] >= 160
     dev.close()
+
+
+def test_against_the_reference_call_itself_where_its_order_is_sequential():
+    # doReduction calls at::sum_out over operand[K, n] (fairring/device.cc:125). On the GPU that
+    # kernel folds the rows in order for K = 2 and 4 (it regroups them from K = 8 on, which is why
+    # the contract is the at::add chain); there the library must equal the reference's own call
+    # bit for bit. For bf16 the single rounding hides the regrouping on this data: equal for K = 8.
+    _print_case("at::sum_out on the GPU")
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(2024)
+    n = 3_000_017
+    for k in (2, 4):
+        st = torch.empty(k, n, device=DEV).normal_(0, 0.01, generator=gen)
+        out = torch.empty(n, device=DEV)
+        fa.reduce_slice(out, [st[i] for i in range(k)])
+        ref = torch.sum(st, dim=0)
+        torch.cuda.synchronize()
+        assert bool(torch.equal(out.view(torch.int32), ref.view(torch.int32))), "fp32 K=%d" % k
+    st = torch.empty(8, n, device=DEV).normal_(0, 0.01, generator=gen).to(torch.bfloat16)
+    out = torch.empty(n, device=DEV, dtype=torch.bfloat16)
+    fa.reduce_slice(out, [st[i] for i in range(8)])
+    ref = torch.sum(st, dim=0)
+    torch.cuda.synchronize()
+    assert bool(torch.equal(out.view(torch.int16), ref.view(torch.int16))), "bf16 K=8"
