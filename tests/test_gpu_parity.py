@@ -649,3 +649,40 @@ def test_against_the_reference_call_itself_where_its_order_is_sequential():
     ref = torch.sum(st, dim=0)
     torch.cuda.synchronize()
     assert bool(torch.equal(out.view(torch.int16), ref.view(torch.int16))), "bf16 K=8"
+
+
+@pytest.mark.parametrize("tdt", [torch.float32, torch.bfloat16, torch.float16, torch.float64,
+                                 torch.int32, torch.int64, torch.uint8, torch.int8])
+def test_max_against_amax_on_the_gpu(tdt):
+    # the reference's MAX is at::amax_out over operand[K, n] (fairring/device.cc:127):
+    # order-independent, NaN wins; only the sign of a zero maximum is left open (+0 == -0)
+    _print_case("at::amax_out on the GPU", tdt)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(77)
+    n = 500_009
+    for k in (1, 2, 5, 8, 13, 64, 70):
+        if tdt.is_floating_point:
+            st = (torch.randn(k, n, device=DEV, generator=gen) * 3).to(tdt)
+            st[k // 2, 5::1001] = float("nan")
+            st[0, 7::1003] = float("inf")
+            st[k - 1, 9::1007] = -float("inf")
+        else:
+            info = torch.iinfo(tdt)
+            st = torch.randint(info.min, info.max, (k, n), device=DEV, generator=gen,
+                               dtype=torch.int64).to(tdt)
+        out = torch.empty(n, device=DEV, dtype=tdt)
+        dev = fa.DeviceFairring(0, slice_size_in_bytes=256 * 1024, max_memory_allocated_in_bytes=MiB)
+        dev.allreduce(out, [st[i] for i in range(k)], op=fa.MAX).wait()
+        dev.close()
+        ref = torch.amax(st, dim=0)
+        torch.cuda.synchronize()
+        if tdt.is_floating_point:
+            both_nan = out.isnan() & ref.isnan()
+            zero = (out == 0) & (ref == 0)
+            same = (out == ref) | both_nan
+            assert bool(same.all()), "%s K=%d" % (tdt, k)
+            bits = {2: torch.int16, 4: torch.int32, 8: torch.int64}[out.element_size()]
+            strict = (out.view(bits) == ref.view(bits)) | both_nan | zero
+            assert bool(strict.all()), "%s K=%d bits" % (tdt, k)
+        else:
+            assert bool(torch.equal(out, ref)), "%s K=%d" % (tdt, k)
