@@ -213,12 +213,16 @@ __device__ __forceinline__ void compressedLane(void* out, const float* raw, cons
 template <typename WV, typename WS, bool OUT32, int KW, int SC>
 __global__ void __launch_bounds__(kBlock)
     compressedKernel(void* out, const float* raw, Ptrs<KW> wire, int Kw, int rawPos, int scaleMode,
-                     float scale, int64_t head, int64_t nvec, int64_t tail, int64_t roundTiles,
-                     int64_t pieces) {
+                     float scale, int64_t head, int lead, int64_t nvec, int64_t tail,
+                     int64_t roundTiles, int64_t pieces) {
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
   const int64_t grid = gridDim.x;
+  // the first `lead` groups are a piece of their own, so that the tiles start
+  // on a 4 KiB boundary of the first wire contribution
+  const int64_t bodyBase = head + static_cast<int64_t>(lead) * WV::kLanes;
+  const int64_t bodyVecs = nvec - lead;
   for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
-    const int64_t elemBase = head + t * kTile * WV::kLanes;
+    const int64_t elemBase = bodyBase + t * kTile * WV::kLanes;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
@@ -233,10 +237,15 @@ __global__ void __launch_bounds__(kBlock)
 #pragma unroll
     for (int u = 0; u < kPiece; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
-      if (v0 + lane < nvec) {
+      if (v0 + lane < bodyVecs) {
         compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale,
-                                          head + v0 * WV::kLanes, lane);
+                                          bodyBase + v0 * WV::kLanes, lane);
       }
+    }
+  }
+  if (lead > 0 && blockIdx.x == gridDim.x - 1) {
+    for (unsigned int lane = threadIdx.x; lane < static_cast<unsigned int>(lead); lane += kBlock) {
+      compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, head, lane);
     }
   }
   if (blockIdx.x == 0 && threadIdx.x < head + tail) {
@@ -253,17 +262,28 @@ hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptr
                             hipStream_t stream) {
   Ptrs<KW> wire;
   for (int k = 0; k < (KW > 0 ? KW : kMaxContribsPerLaunch); ++k) wire.p[k] = all.p[k];
-  const GridPlan plan = planGrid(nvec, a.K, numCus);
+  // groups between the first one and the next 4 KiB boundary of the first wire
+  // contribution (of the fp32 bucket at twice the stride when it stands alone)
+  int lead = 0;
+  if (sizeof(typename WV::vec_t) == 16) {
+    const uintptr_t first =
+        Kw > 0 ? reinterpret_cast<uintptr_t>(all.p[0]) + static_cast<uintptr_t>(head) * 2
+               : (reinterpret_cast<uintptr_t>(raw) + static_cast<uintptr_t>(head) * 4) / 2;
+    const int64_t l = static_cast<int64_t>(
+        ((kLaunchAlignBytes - (first & (kLaunchAlignBytes - 1))) & (kLaunchAlignBytes - 1)) / 16);
+    lead = l < nvec ? static_cast<int>(l) : 0;
+  }
+  const GridPlan plan = planGrid(nvec - lead, a.K, numCus);
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
     hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
                           dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream,
                           a.startEvent, a.stopEvent, 0, a.out, raw, wire, Kw, rawPos, a.scale_mode,
-                          a.scale, head, nvec, tail, plan.roundTiles, plan.pieces);
+                          a.scale, head, lead, nvec, tail, plan.roundTiles, plan.pieces);
   } else {
     hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
                        dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream, a.out, raw,
-                       wire, Kw, rawPos, a.scale_mode, a.scale, head, nvec, tail, plan.roundTiles,
-                       plan.pieces);
+                       wire, Kw, rawPos, a.scale_mode, a.scale, head, lead, nvec, tail,
+                       plan.roundTiles, plan.pieces);
   }
   return hipGetLastError();
 }

@@ -43,6 +43,9 @@ namespace {
 
 constexpr int kBlock = FRG_BLOCK;
 constexpr int kUnroll = FRG_UNROLL;
+// Tiles start on a multiple of this many bytes of the first contribution (the
+// default tile: 128 lanes x 2 vectors x 16 bytes).
+constexpr uintptr_t kLaunchAlignBytes = 4096;
 constexpr int kChunk = 8;  // contributions loaded together in the runtime-K path
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
