@@ -375,6 +375,33 @@ void scenarioCallback() {
   CHECK(frg_synchronize(ctx) == FRG_OK);
   CHECK(st.calls.load() == 1);
   CHECK(frg_destroy(ctx) == FRG_OK);
+
+  // the same through the host-staged path as a process group drives it: the
+  // rank's own term already in `out`, 15 peers staged through 2 slots, several
+  // operations in flight, completion known through the callback alone
+  ctx = makeCtx(2 * 4096, 4096, 0, 0);
+  const int ops = 6;
+  std::vector<std::vector<Vec>> all, rests(ops);
+  std::vector<Vec> outs(ops);
+  std::vector<CallbackState> sts(ops);
+  for (int i = 0; i < ops; ++i) {
+    const int64_t n = 5000 + 11 * i;
+    all.push_back(randomContribs(16, n, 300 + i));
+    outs[i] = all[i][0];
+    rests[i].assign(all[i].begin() + 1, all[i].end());
+    auto tr = table(rests[i]);
+    CHECK(frg_allreduce_host(ctx, outs[i].data(), tr.data(), 15, n, FRG_F32, FRG_SUM,
+                             FRG_SCALE_NONE, 1.f, /*carry=*/1, nullptr, &onDone, &sts[i],
+                             nullptr) == FRG_OK);
+  }
+  for (int i = 0; i < ops; ++i) {
+    while (sts[i].calls.load() == 0) std::this_thread::yield();
+    CHECK(sts[i].status.load() == FRG_OK);
+    CHECK(hipStreamSynchronize(static_cast<hipStream_t>(sts[i].stream.load())) == hipSuccess);
+    CHECK(same(outs[i], fold(all[i], FRG_SCALE_NONE, 1.f)));
+  }
+  CHECK(frg_synchronize(ctx) == FRG_OK);
+  CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
 void scenarioErrors() {
