@@ -152,3 +152,24 @@ def test_c_client_builds_and_fails_cleanly_without_a_gpu(tmp_path):
         assert r.returncode == 0 and "abi client ok" in r.stdout, r.stderr
     else:
         assert r.returncode == 2 and "abi 0.1" in r.stdout     # the HIP runtime finds no device
+
+
+def test_a_missing_library_is_a_loud_error_not_a_fallback(tmp_path):
+    # the product path has no CPU implementation to fall back on: without the built library
+    # the first use raises and names the build command
+    import subprocess
+    import sys
+    code = ("import fairring_amd as fa\n"
+            "try:\n"
+            "    fa.compute_layout(50 << 20, 1 << 20, 16, 1, 1)\n"
+            "except ImportError as e:\n"
+            "    print('raised:', e)\n")
+    env = dict(os.environ, PYTHONPATH=ROOT, FAIRRING_HIP_LIBRARY=str(tmp_path / "absent.so"))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "raised:" in r.stdout and "no fallback" in r.stdout and "fairring_amd.build" in r.stdout
+    # and the package never imports the oracle
+    src = "".join(open(os.path.join(ROOT, "fairring_amd", f)).read()
+                  for f in os.listdir(os.path.join(ROOT, "fairring_amd")) if f.endswith(".py"))
+    assert "import oracle" not in src and "from oracle" not in src
