@@ -415,6 +415,19 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     }
   }
 
+  {
+    // The pipeline hands the launches to its own thread and streams: under HIP
+    // graph capture that cannot be recorded into the caller's graph.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(req.producerStream, &capture) != hipSuccess) {
+      (void)hipGetLastError();
+    } else if (capture != hipStreamCaptureStatusNone) {
+      *err = "the producer stream is being captured into a HIP graph: the pipeline cannot be "
+             "captured, issue frg_reduce_slice on the capturing stream instead";
+      return FRG_ERR_UNSUPPORTED;
+    }
+  }
+
   Work* work = new Work();
   work->device = device_;
   work->progress = progress_;

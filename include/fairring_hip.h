@@ -114,7 +114,8 @@ FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
  * HIP graph (the pointer table is copied into the launch, the graph replays
  * on the captured addresses); the same holds for frg_reduce_slice_compressed.
  * The pipeline entry points (frg_allreduce*) hand work to another thread and
- * are not for capture. */
+ * are not for capture: with a producer stream that is being captured they
+ * return FRG_ERR_UNSUPPORTED. */
 FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);

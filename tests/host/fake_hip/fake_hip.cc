@@ -1,4 +1,5 @@
 // See hip/hip_runtime.h in this directory. Test infrastructure only.
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include <chrono>
@@ -240,6 +241,16 @@ hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) {
 hipError_t hipStreamQuery(hipStream_t stream) {
   enter("hipStreamQuery");
   return resolve(stream)->idle() ? hipSuccess : ret(hipErrorNotReady);
+}
+
+static std::atomic<int> gCapturing{0};
+
+void fake_hip_set_capturing(int on) { gCapturing = on; }
+
+hipError_t hipStreamIsCapturing(hipStream_t /*stream*/, hipStreamCaptureStatus* status) {
+  enter("hipStreamIsCapturing");
+  *status = gCapturing.load() ? hipStreamCaptureStatusActive : hipStreamCaptureStatusNone;
+  return hipSuccess;
 }
 
 hipError_t hipEventQuery(hipEvent_t event) {

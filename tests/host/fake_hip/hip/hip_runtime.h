@@ -49,6 +49,12 @@ const char* hipGetErrorString(hipError_t e);
 hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags);
 hipError_t hipStreamSynchronize(hipStream_t stream);
 hipError_t hipStreamQuery(hipStream_t stream);
+typedef enum hipStreamCaptureStatus {
+  hipStreamCaptureStatusNone = 0,
+  hipStreamCaptureStatusActive = 1,
+  hipStreamCaptureStatusInvalidated = 2
+} hipStreamCaptureStatus;
+hipError_t hipStreamIsCapturing(hipStream_t stream, hipStreamCaptureStatus* status);
 hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int flags);
 
 hipError_t hipEventCreate(hipEvent_t* event);
@@ -67,6 +73,8 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKin
 // ---- hooks for tests ------------------------------------------------------
 // Occupies `stream` (nullptr = the default stream) for `ms` milliseconds.
 void fake_hip_occupy(hipStream_t stream, int ms);
+// Makes hipStreamIsCapturing report a capture in progress on every stream (1) or none (0).
+void fake_hip_set_capturing(int on);
 // Makes the `nth` next call (1 = the very next) of the named API fail once.
 void fake_hip_fail_call(const char* api, int nth);
 // Calls made so far to the named API.

@@ -180,6 +180,15 @@ void scenarioPreScaleAndCompressed() {
   CHECK(frg_work_wait(w) == FRG_OK);
   CHECK(same(raw, want));
   frg_work_release(w);
+  // under graph capture the pipeline refuses (the one-launch entry points are the ones to capture)
+  fake_hip_set_capturing(1);
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3001, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, nullptr, nullptr, nullptr) == FRG_ERR_UNSUPPORTED);
+  CHECK(std::strstr(frg_last_error(), "captured") != nullptr);
+  CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, rawIndex, n, FRG_BF16,
+                                 FRG_SCALE_MUL, 0.2f, nullptr, nullptr, nullptr,
+                                 nullptr) == FRG_ERR_UNSUPPORTED);
+  fake_hip_set_capturing(0);
   // contract violations of the compressed entry point
   CHECK(frg_allreduce_compressed(ctx, raw.data(), FRG_F32, tab.data(), K, 7, n, FRG_BF16, 0, 1.f,
                                  nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);

@@ -103,3 +103,28 @@ def test_captured_compressed_reduction_replays_bit_exactly():
         torch.cuda.synchronize()
         for i, (b, e) in enumerate(zip(own, eager)):
             assert same_bits(b, e), "replay %d bucket %d" % (replay, i)
+
+
+def test_the_pipeline_refuses_a_capturing_stream():
+    # the pipeline launches from its own thread on its own streams, which a capture of the
+    # caller's stream cannot record: it says so instead of splitting the work across the graph
+    print("[case] pipeline under capture", flush=True)
+    n = 100_000
+    xs = [torch.ones(n, device=DEV) for _ in range(K)]
+    out = torch.zeros(n, device=DEV)
+    dev = fa.DeviceFairring(0)
+    dev.allreduce(out, xs).wait()
+    assert bool((out == K).all())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        with pytest.raises(fa.FairringError, match="captured"):
+            dev.allreduce(out, xs)
+        fa.reduce_slice(out, xs, scale_mode=fa.SCALE_MUL, scale=0.5)   # this one may be captured
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert bool((out == K * 0.5).all())
+    dev.allreduce(out, xs).wait()        # and the context works as before afterwards
+    assert bool((out == K).all())
+    dev.close()
