@@ -556,10 +556,6 @@ void Context::chainThroughScratch(const Request& req, const std::vector<const vo
   }
 }
 
-// Device-resident contributions: every slice (the slicing of
-// fairring/device.cc:315-326) is reduced by one launch, or by several when it
-// is larger than the launch size; launches are dealt round-robin to the reduce
-// streams so that neighbouring launches overlap.
 void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired) {
   // Once the producer's event has fired no stream needs to wait for it: a
   // wait that is already satisfied still costs a barrier packet on the queue.
@@ -573,6 +569,10 @@ void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fir
   if (!*fired) FRG_HIP_CHECK(hipStreamWaitEvent(stream, initialEvent, 0));
 }
 
+// Device-resident contributions: the tensor is cut into launches of the launch
+// size (or one per slice of fairring/device.cc:315-326 when asked for), dealt
+// round-robin to the reduce streams so that neighbouring launches overlap.
+// Returns the streams the operation's work ended on.
 std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   const int64_t nSlices = numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
