@@ -152,8 +152,8 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
     c->streamElems_.assign(c->reduceStreams_.size(), 0);
   } catch (const std::exception& e) {
     *err = e.what();
-    // partially built: release what exists, without a command thread to join
-    if (c->stagingPool_) (void)hipFree(c->stagingPool_);
+    // partially built: the destructor releases what exists (there is no command
+    // thread to join yet)
     delete c;
     return FRG_ERR_HIP;
   }

@@ -465,6 +465,9 @@ void scenarioErrors() {
   o.max_memory_allocated_in_bytes = 8192;
   fake_hip_fail_call("hipMalloc", 1);
   CHECK(frg_create(0, &o, &bad) == FRG_ERR_HIP && bad == nullptr);
+  // a failure after the staging pool exists: released once, nothing else left behind
+  fake_hip_fail_call("hipEventCreate", 1);
+  CHECK(frg_create(0, &o, &bad) == FRG_ERR_HIP && bad == nullptr);
   CHECK(frg_create(7, &o, &bad) == FRG_ERR_INVALID);
 }
 
