@@ -17,6 +17,19 @@ int fail(int code, const std::string& msg) {
   return code;
 }
 
+// No C++ exception may cross the ABI: whatever escapes the C++ side (an
+// allocation failure, in practice) becomes a status and a message.
+template <typename F>
+int guarded(F&& body) {
+  try {
+    return body();
+  } catch (const std::exception& e) {
+    return fail(FRG_ERR_HIP, std::string("internal failure: ") + e.what());
+  } catch (...) {
+    return fail(FRG_ERR_HIP, "internal failure");
+  }
+}
+
 Context* asCtx(frg_ctx* c) { return reinterpret_cast<Context*>(c); }
 Work* asWork(frg_work* w) { return reinterpret_cast<Work*>(w); }
 
@@ -28,25 +41,27 @@ int submitCommon(frg_ctx* ctx, void* out, const void* const* contribs, int K, in
   if (K < 0 || (K > 0 && contribs == nullptr) || (K == 0 && !carry)) {
     return fail(FRG_ERR_INVALID, "at least one contribution is required");
   }
-  Context::Request r;
-  r.out = out;
-  if (K > 0) r.contribs.assign(contribs, contribs + K);
-  r.carry = carry;
-  r.numel = numel;
-  r.dtype = dtype;
-  r.op = op;
-  r.scaleMode = scale_mode;
-  r.scale = scale;
-  r.fromHost = fromHost;
-  r.producerStream = static_cast<hipStream_t>(producer_stream);
-  r.done = done;
-  r.user = user;
-  std::string err;
-  Work* w = nullptr;
-  const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  if (work) *work = reinterpret_cast<frg_work*>(w);
-  return FRG_OK;
+  return guarded([&] {
+    Context::Request r;
+    r.out = out;
+    if (K > 0) r.contribs.assign(contribs, contribs + K);
+    r.carry = carry;
+    r.numel = numel;
+    r.dtype = dtype;
+    r.op = op;
+    r.scaleMode = scale_mode;
+    r.scale = scale;
+    r.fromHost = fromHost;
+    r.producerStream = static_cast<hipStream_t>(producer_stream);
+    r.done = done;
+    r.user = user;
+    std::string err;
+    Work* w = nullptr;
+    const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    if (work) *work = reinterpret_cast<frg_work*>(w);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 }  // namespace
@@ -142,12 +157,14 @@ int frg_create(int device, const frg_options* opts, frg_ctx** out) {
     return fail(FRG_ERR_HIP, "no HIP device available");
   }
   if (device < 0 || device >= count) return fail(FRG_ERR_INVALID, "device index out of range");
-  Context* c = nullptr;
-  std::string err;
-  const int rc = Context::create(device, o, &c, &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  *out = reinterpret_cast<frg_ctx*>(c);
-  return FRG_OK;
+  return guarded([&] {
+    Context* c = nullptr;
+    std::string err;
+    const int rc = Context::create(device, o, &c, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    *out = reinterpret_cast<frg_ctx*>(c);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_destroy(frg_ctx* ctx) {
@@ -168,10 +185,12 @@ int frg_get_layout(frg_ctx* ctx, frg_layout* out) {
 
 int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count) {
   if (ctx == nullptr || count == nullptr) return fail(FRG_ERR_INVALID, "null argument");
-  const std::vector<hipStream_t> v = asCtx(ctx)->streams();
-  *count = static_cast<int>(v.size());
-  for (int i = 0; i < *count && i < capacity && streams != nullptr; ++i) streams[i] = v[i];
-  return FRG_OK;
+  return guarded([&] {
+    const std::vector<hipStream_t> v = asCtx(ctx)->streams();
+    *count = static_cast<int>(v.size());
+    for (int i = 0; i < *count && i < capacity && streams != nullptr; ++i) streams[i] = v[i];
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
@@ -190,26 +209,28 @@ int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype, const void*
   if (K < 1 || contribs == nullptr) {
     return fail(FRG_ERR_INVALID, "at least one contribution is required");
   }
-  Context::Request r;
-  r.out = out;
-  r.contribs.assign(contribs, contribs + K);
-  r.numel = numel;
-  r.dtype = wire_dtype;
-  r.op = FRG_SUM;
-  r.scaleMode = scale_mode;
-  r.scale = scale;
-  r.compressed = true;
-  r.outDtype = out_dtype;
-  r.rawIndex = raw_index;
-  r.producerStream = static_cast<hipStream_t>(producer_stream);
-  r.done = done;
-  r.user = user;
-  std::string err;
-  Work* w = nullptr;
-  const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  if (work) *work = reinterpret_cast<frg_work*>(w);
-  return FRG_OK;
+  return guarded([&] {
+    Context::Request r;
+    r.out = out;
+    r.contribs.assign(contribs, contribs + K);
+    r.numel = numel;
+    r.dtype = wire_dtype;
+    r.op = FRG_SUM;
+    r.scaleMode = scale_mode;
+    r.scale = scale;
+    r.compressed = true;
+    r.outDtype = out_dtype;
+    r.rawIndex = raw_index;
+    r.producerStream = static_cast<hipStream_t>(producer_stream);
+    r.done = done;
+    r.user = user;
+    std::string err;
+    Work* w = nullptr;
+    const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    if (work) *work = reinterpret_cast<frg_work*>(w);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs, int K,
@@ -221,10 +242,12 @@ int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs
 
 int frg_work_wait(frg_work* work) {
   if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
-  std::string err;
-  const int rc = Context::waitWork(asWork(work), &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = Context::waitWork(asWork(work), &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_set_wait_timeout(double seconds) {
@@ -249,10 +272,12 @@ int frg_work_is_completed(frg_work* work) {
 
 int frg_work_block_stream(frg_work* work, void* stream) {
   if (work == nullptr) return fail(FRG_ERR_INVALID, "null work");
-  std::string err;
-  const int rc = Context::blockStream(asWork(work), static_cast<hipStream_t>(stream), &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = Context::blockStream(asWork(work), static_cast<hipStream_t>(stream), &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_work_release(frg_work* work) {
@@ -263,18 +288,22 @@ int frg_work_release(frg_work* work) {
 
 int frg_synchronize(frg_ctx* ctx) {
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  std::string err;
-  const int rc = asCtx(ctx)->synchronize(&err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = asCtx(ctx)->synchronize(&err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_profile_mark(frg_ctx* ctx) {
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  std::string err;
-  const int rc = asCtx(ctx)->profileMark(&err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = asCtx(ctx)->profileMark(&err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_set_profiling(frg_ctx* ctx, int per_launch) {
@@ -285,18 +314,22 @@ int frg_set_profiling(frg_ctx* ctx, int per_launch) {
 
 int frg_kernel_times(frg_ctx* ctx, float* ms, int capacity, int* count) {
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  std::string err;
-  const int rc = asCtx(ctx)->kernelTimes(ms, capacity, count, &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = asCtx(ctx)->kernelTimes(ms, capacity, count, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_launch_records(frg_ctx* ctx, frg_launch_record* records, int capacity, int* count) {
   if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
-  std::string err;
-  const int rc = asCtx(ctx)->launchRecords(records, capacity, count, &err);
-  if (rc != FRG_OK) return fail(rc, err);
-  return FRG_OK;
+  return guarded([&] {
+    std::string err;
+    const int rc = asCtx(ctx)->launchRecords(records, capacity, count, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_set_tuning(int blocks_per_cu) {
