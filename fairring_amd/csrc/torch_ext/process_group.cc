@@ -2,6 +2,7 @@
 
 #include "process_group.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstdlib>
 #include <thread>
@@ -30,6 +31,8 @@ namespace {
 at::Tensor viewAsFlat(const at::Tensor& t) {
   FRG_CHECK(t.layout() == at::kStrided);
   FRG_CHECK(t.is_non_overlapping_and_dense());
+  // already flat (what DDP hands over): the same view, without a dispatcher call
+  if (t.dim() == 1 && (t.numel() <= 1 || t.stride(0) == 1)) return t;
   return at::as_strided(t, {t.numel()}, {1}, t.storage_offset());
 }
 
@@ -209,6 +212,8 @@ frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
   o.min_parallelism = options_->minParallelism;
   o.slice_size_in_bytes = options_->sliceSizeInBytes;
   o.num_machines = getSize();  // every simulated peer counts as a machine with one device
+  o.num_reduce_streams = kNumReduceStreams;
+  o.num_copy_streams = kNumCopyStreams;
   frg_ctx* ctx = nullptr;
   const int rc = frg_create(device, &o, &ctx);
   if (rc == FRG_ERR_LAYOUT) {
@@ -225,8 +230,33 @@ frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
                  static_cast<int>(device), static_cast<long long>(l.num_staging_slots),
                  static_cast<long long>(l.slice_size_in_bytes));
   }
+  void* raw[16];
+  int nStreams = 0;
+  TORCH_CHECK(frg_get_streams(ctx, raw, 16, &nStreams) == FRG_OK, frg_last_error());
+  std::vector<c10::Stream>& streams = streams_[device];
+  for (int i = 0; i < nStreams && i < 16; ++i) {
+    streams.push_back(c10::hip::getStreamFromExternalMasqueradingAsCUDA(
+        static_cast<hipStream_t>(raw[i]), device));
+  }
   contexts_.emplace(device, ctx);
   return ctx;
+}
+
+// Tells the caching allocator which streams will touch these buffers
+// (fairring/device.cc:297-301): the reduce streams, and the copy streams as
+// well when contributions are staged from the host (they write `out`).
+void ProcessGroupFairring::recordOnPipelineStreams(
+    c10::DeviceIndex device, bool copyStreamsToo, std::initializer_list<const at::Tensor*> tensors,
+    const std::vector<at::Tensor>* more) {
+  const std::vector<c10::Stream>& streams = streams_[device];
+  const size_t n = copyStreamsToo ? streams.size()
+                                  : std::min(streams.size(), static_cast<size_t>(kNumReduceStreams));
+  for (size_t i = 0; i < n; ++i) {
+    for (const at::Tensor* t : tensors) t->record_stream(streams[i]);
+    if (more != nullptr) {
+      for (const at::Tensor& t : *more) t.record_stream(streams[i]);
+    }
+  }
 }
 
 void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor> peers) {
@@ -376,19 +406,10 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     if (r != rank) ++pi;
   }
 
-  // Tell the caching allocator which streams will touch these buffers
-  // (fairring/device.cc:297-301).
-  void* streams[16];
-  int nStreams = 0;
-  TORCH_CHECK(frg_get_streams(ctx, streams, 16, &nStreams) == FRG_OK, frg_last_error());
-  for (int i = 0; i < nStreams && i < 16; ++i) {
-    c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
-        static_cast<hipStream_t>(streams[i]), device);
-    out.record_stream(s);
-    own.record_stream(s);
-    if (!fromHost) {
-      for (at::Tensor& p : peers) p.record_stream(s);
-    }
+  if (own.data_ptr() == out.data_ptr()) {  // in place: one storage
+    recordOnPipelineStreams(device, fromHost, {&out}, fromHost ? nullptr : &peers);
+  } else {
+    recordOnPipelineStreams(device, fromHost, {&out, &own}, fromHost ? nullptr : &peers);
   }
 
   auto future = c10::make_intrusive<c10::ivalue::Future>(
@@ -549,15 +570,7 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
     table.push_back(r == rank ? t.data_ptr() : peers[pi].data_ptr());
     if (r != rank) ++pi;
   }
-  void* streams[16];
-  int nStreams = 0;
-  TORCH_CHECK(frg_get_streams(ctx, streams, 16, &nStreams) == FRG_OK, frg_last_error());
-  for (int i = 0; i < nStreams && i < 16; ++i) {
-    c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(
-        static_cast<hipStream_t>(streams[i]), device);
-    t.record_stream(s);
-    for (at::Tensor& p : peers) p.record_stream(s);
-  }
+  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&t}, &peers);
   auto future = c10::make_intrusive<c10::ivalue::Future>(
       c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();

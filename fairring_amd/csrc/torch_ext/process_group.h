@@ -160,6 +160,14 @@ class ProcessGroupFairring : public c10d::Backend {
   c10::intrusive_ptr<OptionsFairring> options_;
   std::mutex mutex_;
   std::map<c10::DeviceIndex, frg_ctx*> contexts_;  // built lazily (process_group.cc:140-152)
+  // The pipeline's streams per device as c10 streams, reduce streams first
+  // (numReduceStreams_ of them), then the copy streams.
+  std::map<c10::DeviceIndex, std::vector<c10::Stream>> streams_;
+  static constexpr int kNumReduceStreams = 2;
+  static constexpr int kNumCopyStreams = 2;
+  void recordOnPipelineStreams(c10::DeviceIndex device, bool copyStreamsToo,
+                               std::initializer_list<const at::Tensor*> tensors,
+                               const std::vector<at::Tensor>* more);
   std::vector<at::Tensor> peers_;
   bool fusedDivide_ = false;
 };
