@@ -22,9 +22,23 @@ constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init
 // K = 2: 4,530 / 5,990 / 6,290 / 6,340; K = 4: 5,370 / 6,565 / 6,460 / 6,280;
 // K = 8: 6,070 / 6,360 / 6,060 / - ; K = 16 (at 1.6 / 3.1 / 6.25 / 12.5 MiB): 4,930 /
 // 5,340 / 6,220 / 6,110; K = 64 (0.4 / 1.6 / 3.1 / 12.5 MiB): 3,180 / 6,100 / 6,125 / 6,055.
+// The 8-way fp32 sum (the variant that runs 3 blocks per CU) does better still
+// with launches of three whole rounds of its 768-block grid, 9 MiB: 6,552 GB/s
+// against 6,464 at 12.5 MiB (8 / 8.5 / 9.5 / 10 MiB: 6,505 / 6,461 / 6,527 / 6,468)
+// on an operation large enough to be cut into many; operations of a bucket's
+// size are best cut into launches that divide them (25 MiB: 2 x 12.5 MiB
+// 6,259, 9 + 9 + 7 MiB 6,210), so the 9 MiB apply from 100 MiB per contribution
+// (100 / 200 / 400 MiB operations: 6,462 / 6,458 / 6,445 against 6,359 / 6,380 /
+// 6,370). bf16 and K = 4 do not share this (12.5 MiB is their best).
 constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;
-inline constexpr int64_t defaultLaunchBytes(int numContribs) {
+constexpr int64_t kEightWayFp32LaunchBytes = 9ll * 1024 * 1024;
+constexpr int64_t kEightWayFp32LaunchFrom = 100ll * 1024 * 1024;
+inline constexpr int64_t defaultLaunchBytes(int numContribs, bool fp32Sum = false,
+                                            int64_t bytesPerContrib = 0) {
   if (numContribs <= 2) return 50ll * 1024 * 1024;
+  if (numContribs == 8 && fp32Sum && bytesPerContrib >= kEightWayFp32LaunchFrom) {
+    return kEightWayFp32LaunchBytes;
+  }
   if (numContribs <= 8) return kDefaultMaxLaunchBytes;
   const int64_t perContrib = 100ll * 1024 * 1024 / numContribs;
   const int64_t floor = 25ll * 1024 * 1024 / 8;  // 3.125 MiB

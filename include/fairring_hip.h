@@ -158,8 +158,10 @@ typedef struct frg_options {
                                              launches of this size on 4 KiB boundaries (the last
                                              one up to 1.5 times as long), dealt round-robin to the
                                              reduce streams. 0 = default (12.5 MiB for 3 to 8
-                                             contributions, 50 MiB for fewer, about 100 MiB / K
-                                             for more), < 0 = one launch per slice */
+                                             contributions, 9 MiB for 8-way fp32 sums of at
+                                             least 100 MiB, 50 MiB for fewer contributions,
+                                             about 100 MiB / K for more), < 0 = one launch per
+                                             slice */
 } frg_options;
 
 /* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,

@@ -21,6 +21,10 @@
 // 8, about 100 MiB / K above.
 static_assert(frg::defaultLaunchBytes(2) == 50ll << 20);
 static_assert(frg::defaultLaunchBytes(8) == 13107200);
+static_assert(frg::defaultLaunchBytes(8, true, 25ll << 20) == 13107200);   // a bucket: 2 x 12.5 MiB
+static_assert(frg::defaultLaunchBytes(8, true, 100ll << 20) == 9437184);   // a whole gradient: 9 MiB
+static_assert(frg::defaultLaunchBytes(8, false, 100ll << 20) == 13107200); // bf16, MAX, ...
+static_assert(frg::defaultLaunchBytes(4, true, 100ll << 20) == 13107200);
 static_assert(frg::defaultLaunchBytes(16) == 6553600);
 static_assert(frg::defaultLaunchBytes(64) == 3276800);
 
