@@ -44,6 +44,12 @@ inline constexpr int64_t defaultLaunchBytes(int numContribs, bool fp32Sum = fals
   const int64_t floor = 25ll * 1024 * 1024 / 8;  // 3.125 MiB
   return (perContrib > floor ? perContrib : floor) / 4096 * 4096;
 }
+// The 8-way reduction with compression folded in (2 blocks per CU, rounds of
+// 2 MiB of wire per contribution) wants whole rounds, and more of them: 12.5 /
+// 12 / 16 / 20 / 24 / 32 MiB of wire per contribution and launch ran at 6,222 /
+// 6,304 / 6,345 / 6,340 / 6,209 / 6,109 GB/s (8 / 9 / 10 / 11 / 14 MiB: 6,307 /
+// 6,262 / 6,293 / 6,272 / 6,285). A bucket of up to 24 MiB of wire is one launch.
+constexpr int64_t kEightWayCompressedLaunchBytes = 16ll * 1024 * 1024;
 constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {

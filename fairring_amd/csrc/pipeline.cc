@@ -580,12 +580,13 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
   const int total = static_cast<int>(ptrs.size());
-  // (the compressed reduction keeps the 12.5 MiB of wire per contribution: sizing its
-  // launches by the bytes they move, 10.2 MiB for the 8-way hook, measured within noise)
   const int64_t launchBytes =
-      launchBytesByContribs_ && !req.compressed
-          ? defaultLaunchBytes(total, req.dtype == FRG_F32 && req.op == FRG_SUM, req.numel * elsize)
-          : maxLaunchBytes_;
+      !launchBytesByContribs_
+          ? maxLaunchBytes_
+          : (req.compressed
+                 ? (total == 8 ? kEightWayCompressedLaunchBytes : kDefaultMaxLaunchBytes)
+                 : defaultLaunchBytes(total, req.dtype == FRG_F32 && req.op == FRG_SUM,
+                                      req.numel * elsize));
   const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;
   size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
   bool initialFired = false;
