@@ -186,16 +186,18 @@ DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch target per 
 LAUNCH_QUANTUM_BYTES = 4096
 
 
-def default_launch_bytes(k, fp32_sum=False, bytes_per_contrib=0):
-    """The library's default launch size by number of contributions (and, for
-    the 8-way fp32 sum, by the size of the operation)."""
+def default_launch_bytes(k, bytes_per_contrib=0):
+    """The library's default launch size by number of contributions and size of
+    the operation (layout.h::defaultLaunchShape)."""
     if k <= 2:
-        return 50 * MiB
-    if k == 8 and fp32_sum and bytes_per_contrib >= 100 * MiB:
-        return 9 * MiB
-    if k <= 8:
+        return 48 * MiB
+    large = bytes_per_contrib >= 100 * MiB
+    if k == 3:
+        return 15 * MiB if large else DEFAULT_LAUNCH_BYTES
+    if k <= 8 and not large:
         return DEFAULT_LAUNCH_BYTES
-    return max(100 * MiB // k, 25 * MiB // 8) // 4096 * 4096
+    rounds = max(1, (80 * MiB // (k + 1) + 2 * MiB) // (4 * MiB))
+    return rounds * 4 * MiB
 
 
 def launch_elems(args, op_elems, slice_elems, elsize, k=8):
@@ -204,7 +206,7 @@ def launch_elems(args, op_elems, slice_elems, elsize, k=8):
     boundaries from its start and whatever the slice size; the last launch takes
     up to one and a half times that. A negative target means one launch per
     slice."""
-    lb = args.launch_bytes or default_launch_bytes(k, elsize == 4, op_elems * elsize)
+    lb = args.launch_bytes or default_launch_bytes(k, op_elems * elsize)
     if lb < 0:
         return min(slice_elems, op_elems)
     max_elems = (lb - lb % 16) // elsize

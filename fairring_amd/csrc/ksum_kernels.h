@@ -30,6 +30,9 @@ struct ReduceArgs {
   // chain of launches rounds once, at its end.
   bool carry_acc = false;
   bool out_acc = false;
+  // Blocks of the persistent grid per CU; 0 = the kernel's own rule. The
+  // pipeline sets it together with the launch size (whole rounds of the grid).
+  int blocks_per_cu = 0;
   // Optional timing events (created with timing enabled) that receive the
   // begin and end timestamps of this launch.
   hipEvent_t startEvent = nullptr;

@@ -285,9 +285,14 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   // does (bf16, 8-way: 6,340 vs 6,050 GB/s; fp16: 6,330 vs 6,270).
   constexpr bool kPreScaledHalf =
       (SC == kPreMul || SC == kPreDiv) && sizeof(typename TRV::elem_t) == 2 && TRV::kFloating;
+  // More than 8 contributions are loaded 8 at a time: several dependent load
+  // phases per tile, which more resident waves hide (K = 16: 6,604 GB/s with 4
+  // blocks per CU against 6,229 with 2, launches of one round either way).
+  const int manyWay = KT == 0 && a.K > kChunk ? 4 : 0;
   const int lead = leadVectors<TRV>(a.contribs[0], head, nvec);
-  const GridPlan plan =
-      planGrid(nvec - lead, a.K, numCus, kEightWayFp32 || kPreScaledHalf ? 3 : 0);
+  const int hint = a.blocks_per_cu > 0 ? a.blocks_per_cu
+                                       : (kEightWayFp32 || kPreScaledHalf ? 3 : manyWay);
+  const GridPlan plan = planGrid(nvec - lead, a.K, numCus, hint);
   const int64_t grid = plan.grid, roundTiles = plan.roundTiles, pieces = plan.pieces;
   using elem_t = typename TRV::elem_t;
   const elem_t* carrySrc =

@@ -17,33 +17,61 @@ constexpr int64_t kAlignment = 8;
 constexpr int64_t kDefaultTotalMemory = 50ll * 1024 * 1024;   // fairring/__init__.py:26
 constexpr int64_t kDefaultPaddingMemory = 1024ll * 1024;      // fairring/__init__.py:30
 constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init__.py:34
-// Default bytes of one contribution per launch, by number of contributions.
-// Measured on MI355X (fp32, two reduce streams, GB/s at 6.25 / 12.5 / 25 / 50 MiB):
-// K = 2: 4,530 / 5,990 / 6,290 / 6,340; K = 4: 5,370 / 6,565 / 6,460 / 6,280;
-// K = 8: 6,070 / 6,360 / 6,060 / - ; K = 16 (at 1.6 / 3.1 / 6.25 / 12.5 MiB): 4,930 /
-// 5,340 / 6,220 / 6,110; K = 64 (0.4 / 1.6 / 3.1 / 12.5 MiB): 3,180 / 6,100 / 6,125 / 6,055.
-// The 8-way fp32 sum (the variant that runs 3 blocks per CU) does better still
-// with launches of three whole rounds of its 768-block grid, 9 MiB: 6,552 GB/s
-// against 6,464 at 12.5 MiB (8 / 8.5 / 9.5 / 10 MiB: 6,505 / 6,461 / 6,527 / 6,468)
-// on an operation large enough to be cut into many; operations of a bucket's
-// size are best cut into launches that divide them (25 MiB: 2 x 12.5 MiB
-// 6,259, 9 + 9 + 7 MiB 6,210), so the 9 MiB apply from 100 MiB per contribution
-// (100 / 200 / 400 MiB operations: 6,462 / 6,458 / 6,445 against 6,359 / 6,380 /
-// 6,370). bf16 and K = 4 do not share this (12.5 MiB is their best).
+// Default shape of a launch of the plain reduction: bytes of one contribution
+// per launch and blocks of the persistent grid per CU (0 = the kernel's own
+// rule), by number of contributions and size of the operation. All figures
+// measured on MI355X (256 CUs, 4 KiB of every contribution per block and step,
+// two reduce streams), GB/s of algorithmic bytes in one process unless noted.
+//
+// A launch should be a whole number of rounds of its grid, and the grid 4
+// blocks per CU (1024 blocks, rounds of 4 MiB), with about 80 MB moved per
+// launch:
+//   K = 4:  12.5 MiB 6,528 | 4 blocks, 12 / 16 MiB 6,570 / 6,565
+//   K = 5:  12.5 MiB (3 blocks) 6,558 | 4 blocks, 8 / 12 MiB 6,562 / 6,627
+//   K = 6:  12.5 MiB (2 blocks) 6,378 | 4 blocks, 8 / 12 MiB 6,596 / 6,569
+//   K = 7:  12.5 MiB (2 blocks) 6,023 | 4 blocks, 8 / 12 MiB 6,560 / 6,628
+//   K = 8 fp32: 3 blocks, 9 / 12.5 MiB 6,549 / 6,464 | 4 blocks, 4 / 8 / 12 / 16 MiB
+//           6,256 / 6,600 / 6,546 / 6,486; first process on a fresh box, whole job:
+//           6,457 (3 blocks, 12.5 MiB), 6,530 (3 blocks, 9 MiB), 6,580 (4 blocks, 8 MiB)
+//   K = 8 bf16, fresh box, whole job: 6,394 (2 blocks, 12.5 MiB), 6,593 (4 blocks, 8 MiB)
+//   K = 9:  2 blocks, 11 MiB 6,090 | 4 blocks, 4 / 8 / 12 MiB 5,643 / 6,640 / 6,557
+//   K = 10: 2 blocks, 10 MiB 6,308 | 4 blocks, 4 / 8 MiB 5,896 / 6,662
+//   K = 12: 2 blocks, 8.3 MiB 6,194 | 4 blocks, 4 / 8 / 12 MiB 6,418 / 6,574 / 6,445
+//   K = 14: 4 blocks, 4 / 8 / 12 MiB 6,405 / 6,375 / 6,281
+//   K = 16: 2 blocks, 6.25 MiB 6,302 | 4 blocks, 4 / 8 MiB 6,604 / 6,528
+//   K = 32: 2 blocks, 3.1 MiB 5,550 | 4 blocks, 4 / 8 / 12 MiB 6,428 / 6,348 / 6,265
+//   K = 64: 2 blocks, 3.1 MiB 5,968 | 4 blocks, 4 / 8 MiB 6,552 / 6,481
+// (more than 8 contributions are loaded 8 at a time, several dependent load
+// phases per tile, which the additional waves hide).
+// Operations of a DDP bucket's size are another matter: they want launches
+// that divide them. 25 MiB buckets, 8-way fp32, fresh boxes, whole job: 2 x
+// 12.5 MiB with 3 blocks per CU 6,345 to 6,367; with 4 blocks 6,216; 8 + 8 + 9 MiB
+// with 4 blocks 6,130, with 3 blocks 6,259; 12 + 13 MiB 6,286 to 6,313. So up
+// to 8 contributions the whole-round shape applies from 100 MiB per
+// contribution, and below that the launch is 12.5 MiB with the kernel's own
+// grid (3 blocks per CU for the 8-way fp32 sum, else 32 loads in flight per CU).
+// K = 3 (5 blocks per CU, rounds of 5 MiB): 12.5 MiB 6,395, 15 MiB 6,596.
+// K <= 2 (8 blocks per CU, rounds of 8 MiB): 48 / 50 / 56 MiB 6,450 / 6,407 / 6,433.
+struct LaunchShape {
+  int64_t bytes = 0;
+  int blocksPerCu = 0;
+};
 constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;
-constexpr int64_t kEightWayFp32LaunchBytes = 9ll * 1024 * 1024;
-constexpr int64_t kEightWayFp32LaunchFrom = 100ll * 1024 * 1024;
-inline constexpr int64_t defaultLaunchBytes(int numContribs, bool fp32Sum = false,
-                                            int64_t bytesPerContrib = 0) {
-  if (numContribs <= 2) return 50ll * 1024 * 1024;
-  if (numContribs == 8 && fp32Sum && bytesPerContrib >= kEightWayFp32LaunchFrom) {
-    return kEightWayFp32LaunchBytes;
-  }
-  if (numContribs <= 8) return kDefaultMaxLaunchBytes;
-  const int64_t perContrib = 100ll * 1024 * 1024 / numContribs;
-  const int64_t floor = 25ll * 1024 * 1024 / 8;  // 3.125 MiB
-  return (perContrib > floor ? perContrib : floor) / 4096 * 4096;
+constexpr int64_t kWholeRoundBytes = 4ll * 1024 * 1024;     // 256 CUs x 4 blocks x 4 KiB
+constexpr int64_t kWholeRoundsFrom = 100ll * 1024 * 1024;   // per contribution, up to 8 of them
+constexpr int64_t kBytesPerLaunchTarget = 80ll * 1024 * 1024;
+inline constexpr LaunchShape defaultLaunchShape(int numContribs, int64_t bytesPerContrib) {
+  if (numContribs <= 2) return LaunchShape{48ll * 1024 * 1024, 0};
+  const bool large = bytesPerContrib >= kWholeRoundsFrom;
+  if (numContribs == 3) return LaunchShape{large ? 15ll * 1024 * 1024 : kDefaultMaxLaunchBytes, 0};
+  if (numContribs <= 8 && !large) return LaunchShape{kDefaultMaxLaunchBytes, 0};
+  // whole rounds nearest to the target, at least one
+  const int64_t perContrib = kBytesPerLaunchTarget / (numContribs + 1);
+  int64_t rounds = (perContrib + kWholeRoundBytes / 2) / kWholeRoundBytes;
+  if (rounds < 1) rounds = 1;
+  return LaunchShape{rounds * kWholeRoundBytes, 4};
 }
+
 // The 8-way reduction with compression folded in (2 blocks per CU, rounds of
 // 2 MiB of wire per contribution) wants whole rounds, and more of them: 12.5 /
 // 12 / 16 / 20 / 24 / 32 MiB of wire per contribution and launch ran at 6,222 /

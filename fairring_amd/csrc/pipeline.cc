@@ -118,7 +118,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   // the second stream fills the ramp and drain of the first. Shorter launches
   // still (6 to 8 MiB) gain another 2 % in a bare launch loop but lose it again
   // to per-launch costs here.
-  c->launchBytesByContribs_ = o.max_launch_bytes == 0;  // the default: see defaultLaunchBytes
+  c->launchBytesByContribs_ = o.max_launch_bytes == 0;  // the default: see defaultLaunchShape
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
@@ -580,13 +580,15 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
   const int total = static_cast<int>(ptrs.size());
-  const int64_t launchBytes =
-      !launchBytesByContribs_
-          ? maxLaunchBytes_
-          : (req.compressed
-                 ? (total == 8 ? kEightWayCompressedLaunchBytes : kDefaultMaxLaunchBytes)
-                 : defaultLaunchBytes(total, req.dtype == FRG_F32 && req.op == FRG_SUM,
-                                      req.numel * elsize));
+  // Launch size and grid go together (whole rounds of the grid); a size asked
+  // for by the caller leaves the grid to the kernel's own rule.
+  LaunchShape shape{maxLaunchBytes_, 0};
+  if (launchBytesByContribs_) {
+    shape = req.compressed
+                ? LaunchShape{total == 8 ? kEightWayCompressedLaunchBytes : kDefaultMaxLaunchBytes, 0}
+                : defaultLaunchShape(total, req.numel * elsize);
+  }
+  const int64_t launchBytes = shape.bytes;
   const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;
   size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
   bool initialFired = false;
@@ -689,6 +691,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
                                                                         : FRG_SCALE_NONE;
       a.scale = req.scale;
       a.carry = k0 > 0;
+      a.blocks_per_cu = shape.blocksPerCu;
       launch(a, s);
     }
     lastIdx = si;

@@ -17,16 +17,26 @@
 #include "../../fairring_amd/csrc/layout.h"
 #include "../../include/fairring_hip.h"
 
-// The default launch sizes, pinned: 50 MiB up to 2 contributions, 12.5 MiB up to
-// 8, about 100 MiB / K above.
-static_assert(frg::defaultLaunchBytes(2) == 50ll << 20);
-static_assert(frg::defaultLaunchBytes(8) == 13107200);
-static_assert(frg::defaultLaunchBytes(8, true, 25ll << 20) == 13107200);   // a bucket: 2 x 12.5 MiB
-static_assert(frg::defaultLaunchBytes(8, true, 100ll << 20) == 9437184);   // a whole gradient: 9 MiB
-static_assert(frg::defaultLaunchBytes(8, false, 100ll << 20) == 13107200); // bf16, MAX, ...
-static_assert(frg::defaultLaunchBytes(4, true, 100ll << 20) == 13107200);
-static_assert(frg::defaultLaunchBytes(16) == 6553600);
-static_assert(frg::defaultLaunchBytes(64) == 3276800);
+// The default launch shapes, pinned: 48 MiB up to 2 contributions; up to 8
+// contributions 12.5 MiB with the kernel's own grid for operations of a bucket's
+// size and whole rounds of a 4-blocks-per-CU grid (4 MiB each, about 80 MB per
+// launch) from 100 MiB per contribution; whole rounds for more than 8 always.
+static_assert(frg::defaultLaunchShape(2, 1ll << 30).bytes == 48ll << 20);
+static_assert(frg::defaultLaunchShape(8, 25ll << 20).bytes == 13107200);
+static_assert(frg::defaultLaunchShape(8, 25ll << 20).blocksPerCu == 0);
+static_assert(frg::defaultLaunchShape(8, 100ll << 20).bytes == 8ll << 20);
+static_assert(frg::defaultLaunchShape(8, 100ll << 20).blocksPerCu == 4);
+static_assert(frg::defaultLaunchShape(4, 1ll << 30).bytes == 16ll << 20);
+static_assert(frg::defaultLaunchShape(5, 1ll << 30).bytes == 12ll << 20);
+static_assert(frg::defaultLaunchShape(7, 1ll << 30).bytes == 12ll << 20);
+static_assert(frg::defaultLaunchShape(3, 1ll << 30).bytes == 15ll << 20);
+static_assert(frg::defaultLaunchShape(3, 1ll << 20).bytes == 13107200);
+static_assert(frg::defaultLaunchShape(9, 1ll << 20).bytes == 8ll << 20);
+static_assert(frg::defaultLaunchShape(12, 1ll << 30).bytes == 8ll << 20);
+static_assert(frg::defaultLaunchShape(13, 1ll << 30).bytes == 4ll << 20);
+static_assert(frg::defaultLaunchShape(16, 1ll << 30).bytes == 4ll << 20);
+static_assert(frg::defaultLaunchShape(64, 1ll << 30).bytes == 4ll << 20);
+static_assert(frg::defaultLaunchShape(64, 1ll << 30).blocksPerCu == 4);
 
 #define CHECK(cond)                                                                  \
   do {                                                                               \

@@ -35,9 +35,9 @@ def test_defaults_are_the_headline_configuration():
 
 
 @pytest.mark.parametrize("op_elems,slice_elems,elsize,lb,want", [
-    (1_370_000_000, 6_553_600, 4, 0, 2_359_296),   # a whole fp32 gradient: 9 MiB launches, whatever the slice size
-    (1_300_000_000, 13_107_200, 2, 0, 6_553_600),  # bf16
-    (1_370_000_000, 819_196, 4, 0, 2_359_296),     # default layout (3,276,784 B slices): the same
+    (1_370_000_000, 6_553_600, 4, 0, 2_097_152),   # a whole fp32 gradient: 8 MiB launches, whatever the slice size
+    (1_300_000_000, 13_107_200, 2, 0, 4_194_304),  # bf16: the same 8 MiB
+    (1_370_000_000, 819_196, 4, 0, 2_097_152),     # default layout (3,276,784 B slices): the same
     (1_370_000_000, 6_553_600, 4, -1, 6_553_600),  # one launch per slice
     (6_553_600, 6_553_600, 4, 0, 3_276_800),       # one 25 MiB bucket: two launches
     (262_144, 6_553_600, 4, 0, 262_144),           # the 1 MiB bucket: one launch
