@@ -157,10 +157,12 @@ typedef struct frg_options {
                                              launch covers: device-resident tensors are cut into
                                              launches of this size on 4 KiB boundaries (the last
                                              one up to 1.5 times as long), dealt round-robin to the
-                                             reduce streams. 0 = default (12.5 MiB for 3 to 8
-                                             contributions, 9 MiB for 8-way fp32 sums of at
-                                             least 100 MiB, 50 MiB for fewer contributions,
-                                             about 100 MiB / K for more), < 0 = one launch per
+                                             reduce streams. 0 = default: size and grid chosen
+                                             together (whole rounds of a 4-blocks-per-CU grid,
+                                             about 80 MB per launch, for operations of at least
+                                             100 MiB per contribution and for more than 8
+                                             contributions; 12.5 MiB for smaller operations of
+                                             3 to 8; 48 MiB for fewer), < 0 = one launch per
                                              slice */
 } frg_options;
 
