@@ -193,7 +193,7 @@ def default_launch_bytes(k, bytes_per_contrib=0):
         return 48 * MiB
     large = bytes_per_contrib >= 100 * MiB
     if k == 3:
-        return 15 * MiB if large else DEFAULT_LAUNCH_BYTES
+        return 20 * MiB if large else DEFAULT_LAUNCH_BYTES
     if k <= 8 and not large:
         return DEFAULT_LAUNCH_BYTES
     rounds = max(1, (80 * MiB // (k + 1) + 2 * MiB) // (4 * MiB))

@@ -50,8 +50,11 @@ constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init
 // to 8 contributions the whole-round shape applies from 100 MiB per
 // contribution, and below that the launch is 12.5 MiB with the kernel's own
 // grid (3 blocks per CU for the 8-way fp32 sum, else 32 loads in flight per CU).
-// K = 3 (5 blocks per CU, rounds of 5 MiB): 12.5 MiB 6,395, 15 MiB 6,596.
-// K <= 2 (8 blocks per CU, rounds of 8 MiB): 48 / 50 / 56 MiB 6,450 / 6,407 / 6,433.
+// K = 3 (5 blocks per CU, rounds of 5 MiB): 12.5 MiB 6,395, 15 / 20 / 25 MiB 6,526-6,596 /
+// 6,571 / 6,552; 6 blocks, 12 / 18 / 24 MiB 6,113 / 6,365 / 6,343; 4 blocks, 16 MiB 6,235.
+// K <= 2 (8 blocks per CU, rounds of 8 MiB): 48 / 50 / 56 MiB 6,450 / 6,407 / 6,433; another
+// process: 8 blocks, 32 / 48 / 64 MiB 6,284 / 6,314 / 6,285; 6 blocks, 24 / 48 MiB 6,395 /
+// 6,436; 4 blocks, 16 / 32 / 48 MiB 5,753 / 6,394 / 6,208.
 struct LaunchShape {
   int64_t bytes = 0;
   int blocksPerCu = 0;
@@ -61,9 +64,9 @@ constexpr int64_t kWholeRoundBytes = 4ll * 1024 * 1024;     // 256 CUs x 4 block
 constexpr int64_t kWholeRoundsFrom = 100ll * 1024 * 1024;   // per contribution, up to 8 of them
 constexpr int64_t kBytesPerLaunchTarget = 80ll * 1024 * 1024;
 inline constexpr LaunchShape defaultLaunchShape(int numContribs, int64_t bytesPerContrib) {
-  if (numContribs <= 2) return LaunchShape{48ll * 1024 * 1024, 0};
   const bool large = bytesPerContrib >= kWholeRoundsFrom;
-  if (numContribs == 3) return LaunchShape{large ? 15ll * 1024 * 1024 : kDefaultMaxLaunchBytes, 0};
+  if (numContribs <= 2) return LaunchShape{48ll * 1024 * 1024, large ? 6 : 0};
+  if (numContribs == 3) return LaunchShape{large ? 20ll * 1024 * 1024 : kDefaultMaxLaunchBytes, 0};
   if (numContribs <= 8 && !large) return LaunchShape{kDefaultMaxLaunchBytes, 0};
   // whole rounds nearest to the target, at least one
   const int64_t perContrib = kBytesPerLaunchTarget / (numContribs + 1);

@@ -29,7 +29,9 @@ static_assert(frg::defaultLaunchShape(8, 100ll << 20).blocksPerCu == 4);
 static_assert(frg::defaultLaunchShape(4, 1ll << 30).bytes == 16ll << 20);
 static_assert(frg::defaultLaunchShape(5, 1ll << 30).bytes == 12ll << 20);
 static_assert(frg::defaultLaunchShape(7, 1ll << 30).bytes == 12ll << 20);
-static_assert(frg::defaultLaunchShape(3, 1ll << 30).bytes == 15ll << 20);
+static_assert(frg::defaultLaunchShape(3, 1ll << 30).bytes == 20ll << 20);
+static_assert(frg::defaultLaunchShape(2, 1ll << 30).blocksPerCu == 6);
+static_assert(frg::defaultLaunchShape(2, 1ll << 20).blocksPerCu == 0);
 static_assert(frg::defaultLaunchShape(3, 1ll << 20).bytes == 13107200);
 static_assert(frg::defaultLaunchShape(9, 1ll << 20).bytes == 8ll << 20);
 static_assert(frg::defaultLaunchShape(12, 1ll << 30).bytes == 8ll << 20);
