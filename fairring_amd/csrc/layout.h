@@ -76,11 +76,15 @@ inline constexpr LaunchShape defaultLaunchShape(int numContribs, int64_t bytesPe
 }
 
 // The 8-way reduction with compression folded in (2 blocks per CU, rounds of
-// 2 MiB of wire per contribution) wants whole rounds, and more of them: 12.5 /
-// 12 / 16 / 20 / 24 / 32 MiB of wire per contribution and launch ran at 6,222 /
-// 6,304 / 6,345 / 6,340 / 6,209 / 6,109 GB/s (8 / 9 / 10 / 11 / 14 MiB: 6,307 /
-// 6,262 / 6,293 / 6,272 / 6,285). A bucket of up to 24 MiB of wire is one launch.
-constexpr int64_t kEightWayCompressedLaunchBytes = 16ll * 1024 * 1024;
+// 2 MiB of wire per contribution; 3 and 4 blocks per CU are worse at every
+// size) wants whole rounds too. With the fp32 side staged through LDS, on a
+// whole gradient: 4 / 6 / 8 / 10 / 12 / 16 / 20 MiB of wire per contribution and
+// launch ran at 6,456 / 6,562 / 6,613 / 6,568 / 6,534 / 6,450 / 6,367 GB/s. A
+// bucket (25 MiB of fp32 = 12.5 MiB of wire) is best left as one launch:
+// 6,167-6,185 against 5,441 cut 8 + 4.5 and 5,660 cut 6.25 + 6.25. So 8 MiB from
+// 100 MiB of wire per contribution, and 16 MiB (one launch up to 24 MiB) below.
+constexpr int64_t kEightWayCompressedLaunchBytes = 8ll * 1024 * 1024;
+constexpr int64_t kEightWayCompressedBucketLaunchBytes = 16ll * 1024 * 1024;
 constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {

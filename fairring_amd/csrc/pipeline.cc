@@ -585,7 +585,11 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   LaunchShape shape{maxLaunchBytes_, 0};
   if (launchBytesByContribs_) {
     shape = req.compressed
-                ? LaunchShape{total == 8 ? kEightWayCompressedLaunchBytes : kDefaultMaxLaunchBytes, 0}
+                ? LaunchShape{total != 8 ? kDefaultMaxLaunchBytes
+                                         : (req.numel * elsize >= kWholeRoundsFrom
+                                                ? kEightWayCompressedLaunchBytes
+                                                : kEightWayCompressedBucketLaunchBytes),
+                              0}
                 : defaultLaunchShape(total, req.numel * elsize);
   }
   const int64_t launchBytes = shape.bytes;
