@@ -498,10 +498,13 @@ def run_hook(args, np, torch, fa, oracle):
     elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
     bytes_per_elem = 4 + 2 * (k - 1) + 4
     value = bytes_per_elem * numel * args.steps / elapsed / 1e9
-    # the library's default for the 8-way compressed reduction: 8 MiB of wire per contribution
-    # from 100 MiB on, 16 MiB below
-    largs = args if args.launch_bytes or k != 8 else argparse.Namespace(
-        launch_bytes=(8 if numel * 2 >= 100 * MiB else 16) * MiB)
+    # the library's default for the compressed reduction (layout.h::defaultCompressedLaunchBytes):
+    # whole rounds of 2 MiB of wire nearest to 80 MB per launch; a bucket is one launch
+    if k <= 8 and numel * 2 < 100 * MiB:
+        default_lb = 16 * MiB
+    else:
+        default_lb = max(1, -(-(2 * 80 * MiB // bytes_per_elem) // (2 * MiB))) * 2 * MiB
+    largs = args if args.launch_bytes else argparse.Namespace(launch_bytes=default_lb)
     roof = roofline_from_records(recs, bytes_per_elem, launch_elems(largs, numel, slice_elems, 2),
                                  SPAN_HOW)
     roof["kernel"] = "compressedKernel<Bf16Vec, out fp32>, K=%d" % k

@@ -27,6 +27,69 @@
 namespace frg {
 namespace {
 
+// The fp32 side of a group of 8 elements, moved coalesced and exchanged through LDS.
+//
+// A lane's 8 fp32 values are 32 consecutive bytes, two 16-byte accesses with a
+// stride of 32 bytes between lanes: every instruction of a wave then touches
+// sixteen 128-byte lines for eight lines' worth of data, which measured 4 %
+// on a kernel with one input and the output accessed that way. In whole tiles
+// (all 64 lanes of a wave take part) the fp32 side moves in the coalesced
+// pattern instead, lane l taking the 16-byte chunks l and l + 64 of the wave's
+// 2 KiB, and the two patterns are exchanged through a wave-private 2 KiB of
+// LDS (`stage`). A wave executes its LDS instructions in order, so the exchange
+// needs no barrier, only that the compiler keeps the order it is given.
+// The two halves of the load: the global loads are issued first, so that the
+// wire loads that follow them in program order are in flight before the
+// exchange waits for these two.
+struct StagedChunks {
+  f32x4 lo, hi;
+};
+
+__device__ __forceinline__ StagedChunks issueStaged(const float* base, int64_t elemBase,
+                                                    unsigned int lane) {
+  const unsigned int waveLane = lane & 63u;
+  const int64_t waveBase = elemBase + static_cast<int64_t>(lane - waveLane) * 8;
+  const f32x4* p = reinterpret_cast<const f32x4*>(base + waveBase) + waveLane;
+  StagedChunks c;
+  c.lo = ldStream(p);
+  c.hi = ldStream(p + 64);
+  return c;
+}
+
+__device__ __forceinline__ Fp32Side<8>::regs_t exchangeStaged(const StagedChunks& c,
+                                                             unsigned int lane, f32x4* stage) {
+  const unsigned int waveLane = lane & 63u;
+  stage[waveLane] = c.lo;
+  stage[waveLane + 64] = c.hi;
+  __builtin_amdgcn_wave_barrier();
+  Fp32Side<8>::regs_t r;
+  r.a = stage[2 * waveLane];
+  r.b = stage[2 * waveLane + 1];
+  __builtin_amdgcn_wave_barrier();
+  return r;
+}
+
+__device__ __forceinline__ void storeStaged(float* base, int64_t elemBase, unsigned int lane,
+                                            const float (&f)[8], f32x4* stage) {
+  const unsigned int waveLane = lane & 63u;
+  const int64_t waveBase = elemBase + static_cast<int64_t>(lane - waveLane) * 8;
+  f32x4 lo, hi;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    lo[j] = f[j];
+    hi[j] = f[4 + j];
+  }
+  stage[2 * waveLane] = lo;
+  stage[2 * waveLane + 1] = hi;
+  __builtin_amdgcn_wave_barrier();
+  const f32x4 outLo = stage[waveLane];
+  const f32x4 outHi = stage[waveLane + 64];
+  __builtin_amdgcn_wave_barrier();
+  f32x4* p = reinterpret_cast<f32x4*>(base + waveBase) + waveLane;
+  stStream(outLo, p);
+  stStream(outHi, p + 64);
+}
+
 // State of one lane's fold: the accumulator, whether it holds a term yet, and
 // this rank's own term (compressed once the loads that follow it are issued).
 template <typename W>
@@ -35,6 +98,11 @@ struct Fold {
   float own[W::kLanes];
   bool first = true;
   bool ownReady = false;
+  // where the own term comes from when the fp32 side is staged through LDS
+  // (issued by compressedOne, exchanged once the wire loads are in flight)
+  StagedChunks chunks;
+  f32x4* stage = nullptr;
+  unsigned int lane = 0;
 
   __device__ __forceinline__ void add(const float (&t)[W::kLanes]) {
     if (first) {
@@ -51,7 +119,14 @@ struct Fold {
   __device__ __forceinline__ void compress(const typename Fp32Side<W::kLanes>::regs_t& raw,
                                            int scaleMode, float scale) {
     if (ownReady) return;
-    Fp32Side<W::kLanes>::unpack(raw, own);
+    bool unpacked = false;
+    if constexpr (W::kLanes == 8) {
+      if (stage != nullptr) {
+        Fp32Side<8>::unpack(exchangeStaged(chunks, lane, stage), own);
+        unpacked = true;
+      }
+    }
+    if (!unpacked) Fp32Side<W::kLanes>::unpack(raw, own);
 #pragma unroll
     for (int j = 0; j < W::kLanes; ++j) {
       float c = W::roundStorage(own[j]);
@@ -93,16 +168,27 @@ __device__ __forceinline__ void foldWire(Fold<W>& st, const Ptrs<0>& in, int k0,
 
 // One lane's group of elements. `wire` holds the Kw peers' pointers in order,
 // `raw` this rank's fp32 buffer (rawPos = its place in the chain, -1: absent).
-template <typename W, bool OUT32>
+// STAGED (whole tiles of the 8-element variant only): the fp32 side goes
+// through loadStaged / storeStaged.
+template <typename W, bool OUT32, bool STAGED = false>
 __device__ __forceinline__ void compressedOne(void* out, const float* raw, const Ptrs<0>& wire,
                                               int Kw, int rawPos, int scaleMode, float scale,
-                                              int64_t elemBase, unsigned int lane) {
+                                              int64_t elemBase, unsigned int lane,
+                                              f32x4* stage = nullptr) {
   using vec_t = typename W::vec_t;
   using Side = Fp32Side<W::kLanes>;
   const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
   typename Side::regs_t rawRegs = {};
-  if (rawPos >= 0) rawRegs = Side::load(raw + elemBase, lane);
   Fold<W> st;
+  if (rawPos >= 0) {
+    if constexpr (STAGED) {
+      st.chunks = issueStaged(raw, elemBase, lane);
+      st.stage = stage;
+      st.lane = lane;
+    } else {
+      rawRegs = Side::load(raw + elemBase, lane);
+    }
+  }
   int k = 0;
   for (; k + kChunk <= Kw; k += kChunk) {
     foldWire<W, kChunk>(st, wire, k, elemBase, laneBytes, rawPos, rawRegs, scaleMode, scale);
@@ -126,7 +212,11 @@ __device__ __forceinline__ void compressedOne(void* out, const float* raw, const
     float r[W::kLanes];
 #pragma unroll
     for (int j = 0; j < W::kLanes; ++j) r[j] = W::roundStorage(st.acc[j]);
-    Side::store(static_cast<float*>(out) + elemBase, lane, r);
+    if constexpr (STAGED) {
+      storeStaged(static_cast<float*>(out), elemBase, lane, r, stage);
+    } else {
+      Side::store(static_cast<float*>(out) + elemBase, lane, r);
+    }
   } else {
     vec_t* o = reinterpret_cast<vec_t*>(
         reinterpret_cast<char*>(static_cast<typename W::elem_t*>(out) + elemBase) + laneBytes);
@@ -141,16 +231,7 @@ __device__ __forceinline__ void compressedOne(void* out, const float* raw, const
 // body is a tenth of the general one's code (which matters when a launch
 // lasts 20 us and every CU starts it with a cold instruction cache). Same
 // arithmetic, in the same order, as compressedOne.
-//
-// A lane's 8 fp32 values are 32 consecutive bytes, two 16-byte accesses with a
-// stride of 32 bytes between lanes: every instruction of a wave then touches
-// sixteen 128-byte lines for eight lines' worth of data, which measured 4 %
-// on a kernel with one input and the output accessed that way. With `stage`
-// (whole tiles only: all 64 lanes of the wave take part) the fp32 side moves in
-// the coalesced pattern instead, lane l taking the 16-byte chunks l and l + 64
-// of the wave's 2 KiB, and the two patterns are exchanged through a wave-private
-// 2 KiB of LDS. A wave executes its LDS instructions in order, so the exchange
-// needs no barrier, only that the compiler keeps the order it is given.
+// STAGED (whole tiles): the fp32 side goes through loadStaged / storeStaged.
 template <typename W, int KW, int SC, bool STAGED = false>
 __device__ __forceinline__ void compressedFixed(float* out, const float* raw, const Ptrs<KW>& wire,
                                                 int rawPos, float scale, int64_t elemBase,
@@ -160,14 +241,9 @@ __device__ __forceinline__ void compressedFixed(float* out, const float* raw, co
   using Side = Fp32Side<W::kLanes>;
   const unsigned int laneBytes = lane * static_cast<unsigned int>(sizeof(vec_t));
   typename Side::regs_t rawRegs;
-  // the wave's first group in the tile, and this lane's place in the wave
-  const unsigned int waveLane = lane & 63u;
-  const int64_t waveBase = elemBase + static_cast<int64_t>(lane - waveLane) * W::kLanes;
-  f32x4 chunkLo, chunkHi;
+  StagedChunks chunks;
   if constexpr (STAGED) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(raw + waveBase) + waveLane;
-    chunkLo = ldStream(p);
-    chunkHi = ldStream(p + 64);
+    chunks = issueStaged(raw, elemBase, lane);
   } else {
     rawRegs = Side::load(raw + elemBase, lane);
   }
@@ -177,14 +253,7 @@ __device__ __forceinline__ void compressedFixed(float* out, const float* raw, co
     const char* b = reinterpret_cast<const char*>(static_cast<const elem_t*>(wire.p[k]) + elemBase);
     v[k] = ldStream(reinterpret_cast<const vec_t*>(b + laneBytes));
   }
-  if constexpr (STAGED) {
-    stage[waveLane] = chunkLo;
-    stage[waveLane + 64] = chunkHi;
-    __builtin_amdgcn_wave_barrier();
-    rawRegs.a = stage[2 * waveLane];
-    rawRegs.b = stage[2 * waveLane + 1];
-    __builtin_amdgcn_wave_barrier();
-  }
+  if constexpr (STAGED) rawRegs = exchangeStaged(chunks, lane, stage);
   // buffer.to(wire) then div_(world) in the wire type: two roundings
   float own[W::kLanes];
   Side::unpack(rawRegs, own);
@@ -222,21 +291,7 @@ __device__ __forceinline__ void compressedFixed(float* out, const float* raw, co
 #pragma unroll
   for (int j = 0; j < W::kLanes; ++j) acc[j] = W::roundStorage(acc[j]);
   if constexpr (STAGED) {
-    f32x4 lo, hi;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      lo[j] = acc[j];
-      hi[j] = acc[4 + j];
-    }
-    stage[2 * waveLane] = lo;
-    stage[2 * waveLane + 1] = hi;
-    __builtin_amdgcn_wave_barrier();
-    const f32x4 outLo = stage[waveLane];
-    const f32x4 outHi = stage[waveLane + 64];
-    __builtin_amdgcn_wave_barrier();
-    f32x4* p = reinterpret_cast<f32x4*>(out + waveBase) + waveLane;
-    stStream(outLo, p);
-    stStream(outHi, p + 64);
+    storeStaged(out, elemBase, lane, acc, stage);
   } else {
     Side::store(out + elemBase, lane, acc);
   }
@@ -268,19 +323,25 @@ __global__ void __launch_bounds__(kBlock)
   // on a 4 KiB boundary of the first wire contribution
   const int64_t bodyBase = head + static_cast<int64_t>(lead) * WV::kLanes;
   const int64_t bodyVecs = nvec - lead;
-  constexpr bool kStaged = KW > 0 && WV::kLanes == 8 && kBlock % 64 == 0;
+  // whole tiles: every lane of every wave takes part, so the fp32 side can go
+  // through the wave's staging area in LDS
+  constexpr bool kStaged = WV::kLanes == 8 && kBlock % 64 == 0;
   __shared__ f32x4 stageAll[kStaged ? (kBlock / 64) * 128 : 1];
+  f32x4* stage = stageAll + (kStaged ? (threadIdx.x >> 6) * 128 : 0);
   for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
     const int64_t elemBase = bodyBase + t * kTile * WV::kLanes;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
-      if constexpr (kStaged) {
+      const unsigned int lane = threadIdx.x + u * kBlock;
+      if constexpr (kStaged && KW > 0) {
         compressedFixed<WV, KW, SC, true>(static_cast<float*>(out), raw, wire, rawPos, scale,
-                                          elemBase, threadIdx.x + u * kBlock,
-                                          stageAll + (threadIdx.x >> 6) * 128);
+                                          elemBase, lane, stage);
+      } else if constexpr (kStaged) {
+        compressedOne<WV, OUT32, true>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
+                                       lane, stage);
       } else {
         compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
-                                          threadIdx.x + u * kBlock);
+                                          lane);
       }
     }
   }

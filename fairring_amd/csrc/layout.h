@@ -75,16 +75,31 @@ inline constexpr LaunchShape defaultLaunchShape(int numContribs, int64_t bytesPe
   return LaunchShape{rounds * kWholeRoundBytes, 4};
 }
 
-// The 8-way reduction with compression folded in (2 blocks per CU, rounds of
-// 2 MiB of wire per contribution; 3 and 4 blocks per CU are worse at every
-// size) wants whole rounds too. With the fp32 side staged through LDS, on a
-// whole gradient: 4 / 6 / 8 / 10 / 12 / 16 / 20 MiB of wire per contribution and
-// launch ran at 6,456 / 6,562 / 6,613 / 6,568 / 6,534 / 6,450 / 6,367 GB/s. A
-// bucket (25 MiB of fp32 = 12.5 MiB of wire) is best left as one launch:
-// 6,167-6,185 against 5,441 cut 8 + 4.5 and 5,660 cut 6.25 + 6.25. So 8 MiB from
-// 100 MiB of wire per contribution, and 16 MiB (one launch up to 24 MiB) below.
-constexpr int64_t kEightWayCompressedLaunchBytes = 8ll * 1024 * 1024;
-constexpr int64_t kEightWayCompressedBucketLaunchBytes = 16ll * 1024 * 1024;
+// The reduction with compression folded in (2 blocks per CU, rounds of 2 MiB
+// of wire per contribution; 3 and 4 blocks per CU are worse at every size)
+// wants whole rounds too, and again about 80 MB per launch. 8-way hook (22
+// bytes per element) on a whole gradient: 4 / 6 / 8 / 10 / 12 / 16 / 20 MiB of
+// wire per contribution and launch ran at 6,456 / 6,562 / 6,613 / 6,568 / 6,534
+// / 6,450 / 6,367 GB/s; 16-way (38 bytes): 2 / 4 / 8 / 12.5 MiB 5,217 / 6,100 /
+// 6,104 / 5,902; 64-way (134 bytes): 2 / 4 / 8 / 12.5 MiB 6,292 / 6,087 / 5,966 /
+// 5,798. A bucket of up to 8 contributions (25 MiB of fp32 = 12.5 MiB of wire)
+// is best left as one launch: 6,167-6,185 against 5,441 cut 8 + 4.5 and 5,660 cut
+// 6.25 + 6.25; so below 100 MiB of wire per contribution those take 16 MiB (one
+// launch up to 24 MiB).
+constexpr int64_t kCompressedRoundBytes = 2ll * 1024 * 1024;  // 256 CUs x 2 blocks x 4 KiB
+constexpr int64_t kCompressedBucketLaunchBytes = 16ll * 1024 * 1024;
+inline constexpr int64_t defaultCompressedLaunchBytes(int numContribs, bool rawTerm,
+                                                      bool fp32Output, int64_t wireBytesPerContrib) {
+  if (numContribs <= 8 && wireBytesPerContrib < kWholeRoundsFrom) {
+    return kCompressedBucketLaunchBytes;
+  }
+  const int64_t bytesPerElem = 2 * static_cast<int64_t>(numContribs) + (rawTerm ? 2 : 0) +
+                               (fp32Output ? 4 : 2);
+  const int64_t perContrib = 2 * kBytesPerLaunchTarget / bytesPerElem;
+  // rounded up: 32-way (70 bytes per element, 2.3 MiB) 2 / 4 / 6 MiB 5,852 / 6,176 / 6,066
+  const int64_t rounds = (perContrib + kCompressedRoundBytes - 1) / kCompressedRoundBytes;
+  return (rounds < 1 ? 1 : rounds) * kCompressedRoundBytes;
+}
 constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {

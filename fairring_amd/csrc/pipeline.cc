@@ -585,10 +585,9 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   LaunchShape shape{maxLaunchBytes_, 0};
   if (launchBytesByContribs_) {
     shape = req.compressed
-                ? LaunchShape{total != 8 ? kDefaultMaxLaunchBytes
-                                         : (req.numel * elsize >= kWholeRoundsFrom
-                                                ? kEightWayCompressedLaunchBytes
-                                                : kEightWayCompressedBucketLaunchBytes),
+                ? LaunchShape{defaultCompressedLaunchBytes(total, req.rawIndex >= 0,
+                                                           req.outDtype == FRG_F32,
+                                                           req.numel * elsize),
                               0}
                 : defaultLaunchShape(total, req.numel * elsize);
   }

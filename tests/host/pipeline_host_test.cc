@@ -39,6 +39,13 @@ static_assert(frg::defaultLaunchShape(13, 1ll << 30).bytes == 4ll << 20);
 static_assert(frg::defaultLaunchShape(16, 1ll << 30).bytes == 4ll << 20);
 static_assert(frg::defaultLaunchShape(64, 1ll << 30).bytes == 4ll << 20);
 static_assert(frg::defaultLaunchShape(64, 1ll << 30).blocksPerCu == 4);
+// the compressed reduction: whole rounds of 2 MiB of wire, about 80 MB per launch; a bucket is one launch
+static_assert(frg::defaultCompressedLaunchBytes(8, true, true, 1ll << 30) == 8ll << 20);
+static_assert(frg::defaultCompressedLaunchBytes(8, true, true, 12ll << 20) == 16ll << 20);
+static_assert(frg::defaultCompressedLaunchBytes(16, true, true, 1ll << 30) == 6ll << 20);
+static_assert(frg::defaultCompressedLaunchBytes(32, true, true, 1ll << 30) == 4ll << 20);
+static_assert(frg::defaultCompressedLaunchBytes(64, true, true, 1ll << 20) == 2ll << 20);
+static_assert(frg::defaultCompressedLaunchBytes(2, true, true, 1ll << 30) == 16ll << 20);
 
 #define CHECK(cond)                                                                  \
   do {                                                                               \
