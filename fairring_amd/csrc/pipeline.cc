@@ -122,6 +122,10 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
+  if (const char* v = std::getenv("FAIRRING_CHAIN_SCRATCH_BYTES")) {
+    const long long b = std::atoll(v);
+    if (b >= 4096) c->carryScratchBytes_ = b / 4096 * 4096;
+  }
   try {
     DeviceGuard g(device);
     int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams : 2;
@@ -506,9 +510,9 @@ void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
 char* Context::scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize) {
   if (carryScratch_ == nullptr) {
     FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&carryScratch_),
-                            reduceStreams_.size() * static_cast<size_t>(kCarryScratchBytes + 16)));
+                            reduceStreams_.size() * static_cast<size_t>(carryScratchBytes_ + 16)));
   }
-  char* base = carryScratch_ + streamIdx * static_cast<size_t>(kCarryScratchBytes + 16);
+  char* base = carryScratch_ + streamIdx * static_cast<size_t>(carryScratchBytes_ + 16);
   const uintptr_t pos = reinterpret_cast<uintptr_t>(like) & 15;
   if (!acc) return base + pos;
   const uintptr_t headElems = ((16 - pos) & 15) / static_cast<uintptr_t>(elsize);
@@ -527,7 +531,7 @@ void Context::chainThroughScratch(const Request& req, const std::vector<const vo
   hipStream_t s = reduceStreams_[streamIdx];
   char* outBase = static_cast<char*>(req.out) + off * elsize;
   char* scratch = scratchFor(streamIdx, acc ? ptrs[0] : outBase, acc, elsize);
-  const int64_t pieceLen = kCarryScratchBytes / (acc ? 4 : elsize);
+  const int64_t pieceLen = carryScratchBytes_ / (acc ? 4 : elsize);
   std::vector<const void*> shifted(ptrs.size());
   for (int64_t q = 0; q < len; q += pieceLen) {
     const int64_t qlen = len - q < pieceLen ? len - q : pieceLen;
@@ -738,8 +742,8 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
   // are then as short as the scratch buffer that holds those partial sums.
   const bool accChain = req.op == FRG_SUM && (req.dtype == FRG_BF16 || req.dtype == FRG_F16) &&
                         K - (req.carry ? 0 : 1) > batch;
-  if (accChain && sliceBytes > kCarryScratchBytes / 4 * elsize) {
-    sliceBytes = kCarryScratchBytes / 4 * elsize;
+  if (accChain && sliceBytes > carryScratchBytes_ / 4 * elsize) {
+    sliceBytes = carryScratchBytes_ / 4 * elsize;
   }
   const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
 

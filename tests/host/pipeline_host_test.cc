@@ -113,7 +113,15 @@ void scenarioResident() {
   std::puts("resident: slicing, launch splitting, stream rotation");
   for (int streams : {1, 2, 3}) {
     for (int64_t launch : {int64_t(-1), int64_t(1024), int64_t(4096)}) {
+      // a chain scratch of one tile (two for three streams, the default for one):
+      // the chains below then walk it in several pieces
+      if (streams == 1) {
+        unsetenv("FAIRRING_CHAIN_SCRATCH_BYTES");
+      } else {
+        setenv("FAIRRING_CHAIN_SCRATCH_BYTES", streams == 2 ? "4096" : "8192", 1);
+      }
       frg_ctx* ctx = makeCtx(16384, 4096, streams, launch);
+      unsetenv("FAIRRING_CHAIN_SCRATCH_BYTES");
       auto c = randomContribs(8, 10007, 1);
       Vec out(10007);
       frg_work* w = nullptr;

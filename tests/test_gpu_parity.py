@@ -277,13 +277,24 @@ def test_pipeline_more_than_64_contributions():
     dev.close()
 
 
+@pytest.fixture(params=[None, 1 << 20, 40960], ids=["scratch-default", "scratch-1MiB", "scratch-40KiB"])
+def chain_scratch(request, monkeypatch):
+    # the scratch buffer that carries a chain's partial result (8 MiB per stream by default);
+    # small ones make the tensors of these tests span several pieces of it
+    if request.param is None:
+        monkeypatch.delenv("FAIRRING_CHAIN_SCRATCH_BYTES", raising=False)
+    else:
+        monkeypatch.setenv("FAIRRING_CHAIN_SCRATCH_BYTES", str(request.param))
+    return request.param
+
+
 @pytest.mark.parametrize("alias", [3, 64, 69])
 @pytest.mark.parametrize("shift", [0, 3])
-def test_pipeline_in_place_with_more_than_64_contributions(alias, shift):
+def test_pipeline_in_place_with_more_than_64_contributions(alias, shift, chain_scratch):
     # reduced in place into contribution `alias`; from index 64 on, that contribution is only
     # read by the second launch of the chain, so the partial result of the first must not
-    # land in it (it travels through a scratch buffer, 1 MiB at a time)
-    _print_case("pipeline in place, K=70", alias, shift)
+    # land in it (it travels through a scratch buffer, a piece at a time)
+    _print_case("pipeline in place, K=70", alias, shift, chain_scratch)
     k, n = 70, 700_001
     rng = np.random.default_rng(33 + alias)
     x = (rng.standard_normal((k, n + shift)) * 0.01).astype(np.float32)
@@ -300,7 +311,7 @@ def test_pipeline_in_place_with_more_than_64_contributions(alias, shift):
 
 @pytest.mark.parametrize("kind,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
 @pytest.mark.parametrize("shift", [0, 5])
-def test_pipeline_half_types_round_once_over_a_chain(kind, tdt, shift):
+def test_pipeline_half_types_round_once_over_a_chain(kind, tdt, shift, chain_scratch):
     # more contributions than one launch takes: the partial sums travel in fp32 between the
     # launches, so the result is the single fp32 fold with one rounding (at::sum_out over
     # [K, n]), not a fold that rounds to the storage type after every 64 terms
@@ -332,7 +343,7 @@ def test_pipeline_half_types_round_once_over_a_chain(kind, tdt, shift):
 
 @pytest.mark.parametrize("kind,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
 @pytest.mark.parametrize("slots,carry", [(1, False), (2, True), (4, False), (6, True)])
-def test_pipeline_host_staged_half_types_round_once(kind, tdt, slots, carry):
+def test_pipeline_host_staged_half_types_round_once(kind, tdt, slots, carry, chain_scratch):
     # few slots: the pinned contributions are folded batch after batch; the partial sums stay
     # in fp32 between the batches
     _print_case("half-type host staged", kind, slots, carry)
