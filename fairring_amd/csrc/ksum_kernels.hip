@@ -278,7 +278,9 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   // fp32 variant gains 1.3 % from 3 blocks per CU over 2 (6,342 vs 6,263 GB/s,
   // medians of 4 alternating runs); for every other count of contributions and
   // for the 2-byte types the rule of planGrid is at least as good.
-  constexpr bool kEightWayFp32 = sizeof(typename TRV::elem_t) == 4 && TRV::kFloating && KT == 8;
+  // (bf16, 25 MiB buckets, 12.5 MiB launches: 5,896 GB/s with 2 blocks per CU,
+  // 6,078 with 3, 6,068 with 4.)
+  constexpr bool kEightWayGradient = sizeof(typename TRV::elem_t) <= 4 && TRV::kFloating && KT == 8;
   // The pre-scaled sums of the 2-byte types round every term to the storage
   // type before the fold: four times the arithmetic of the plain sum, and with
   // one wave per SIMD nothing overlaps it with the loads. A third block per CU
@@ -291,7 +293,7 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   const int manyWay = KT == 0 && a.K > kChunk ? 4 : 0;
   const int lead = leadVectors<TRV>(a.contribs[0], head, nvec);
   const int hint = a.blocks_per_cu > 0 ? a.blocks_per_cu
-                                       : (kEightWayFp32 || kPreScaledHalf ? 3 : manyWay);
+                                       : (kEightWayGradient || kPreScaledHalf ? 3 : manyWay);
   const GridPlan plan = planGrid(nvec - lead, a.K, numCus, hint);
   const int64_t grid = plan.grid, roundTiles = plan.roundTiles, pieces = plan.pieces;
   using elem_t = typename TRV::elem_t;
