@@ -17,6 +17,10 @@ Other workloads (the remaining configurations of the benchmark definition, for t
         memory with hipMemcpyAsync, overlapped with the accumulate kernel
   c5    DDP backward stream: the 1.37 G gradient as 25 MiB buckets (first one
         1 MiB) released in reverse order, one allreduce call per bucket
+  c5pg  the same bucket stream through the drop-in surface: one
+        _fairring.ProcessGroup.allreduce per bucket (group of 8, 7 simulated
+        peers resident on the GPU, in place, completion through the future,
+        every work waited for at the end of the step)
   copy  K = 1 (a plain copy of known size), the calibration for HBM counters
   hook  torch's bf16 compression hook folded into the reduction: own fp32
         gradient compressed in registers + 7 peers' bf16 tensors, result
@@ -24,7 +28,9 @@ Other workloads (the remaining configurations of the benchmark definition, for t
 
 Prints one JSON line with the whole-job GB/s, the roofline of the reduction
 kernel (algorithmic bytes per launch / average launch duration from HIP events
-on the kernel's own stream) and a CPU baseline timed on this host's cores.
+on the kernel's own stream) and a CPU baseline timed on this host's cores. The
+default run (c2) then measures the other workloads as well, briefly, and adds
+them to the same line under "configs" (--no-extra-configs leaves them out).
 """
 import argparse
 import json
@@ -45,7 +51,10 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5", "copy", "hook", "smallops"])
+    ap.add_argument("--workload", default="c2",
+                    choices=["c2", "c3", "c4", "c5", "c5pg", "copy", "hook", "smallops"])
+    ap.add_argument("--no-extra-configs", action="store_true",
+                    help="default workload only: do not measure the other workloads afterwards")
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
     ap.add_argument("--k", type=int, default=0, help="override the number of contributions")
     ap.add_argument("--slice-bytes", type=int, default=25 * MiB)
@@ -293,7 +302,7 @@ def per_launch_pass(fa, args, run_steps):
     return recs
 
 
-def run_resident(args, np, torch, fa, oracle, dtype):
+def run_resident(args, np, torch, fa, oracle, dtype, keep=None):
     """c2 / c4 / copy: device-resident contributions, one allreduce per step."""
     elsize = 4 if dtype == "f32" else 2
     if args.workload == "copy":
@@ -355,6 +364,8 @@ def run_resident(args, np, torch, fa, oracle, dtype):
     if not args.no_cpu_baseline and args.workload != "copy":
         base = cpu_baseline(oracle, np, torch, xs, slice_elems, k,
                             min(args.cpu_slices, max(1, n_slices - 1)), dtype)
+    if keep is not None:
+        keep.extend([xs, out])
     return value, elapsed, cfg, roof, checked, base, dtype
 
 
@@ -362,12 +373,14 @@ def run_c3(args, np, torch, fa, oracle):
     """Server-side accumulation: K = 64 contributions of one 25 MiB fp32 slice in
     pinned host memory, staged through the pool and folded in order."""
     k, numel = args.k or 64, args.numel or 6_553_600
-    rng = np.random.default_rng(33)
+    g = torch.Generator(device="cuda:0")
     hs = []
     for r in range(k):
+        g.manual_seed(3300 + r)
         t = torch.empty(numel, dtype=torch.float32).pin_memory()
-        t.copy_(torch.from_numpy((rng.standard_normal(numel) * 0.01).astype(np.float32)))
+        t.copy_(torch.empty(numel, device="cuda:0").normal_(0.0, 0.01, generator=g))
         hs.append(t)
+    torch.cuda.synchronize()
     out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
     dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
                             slice_size_in_bytes=args.slice_bytes,
@@ -421,7 +434,7 @@ def ddp_buckets(numel, bucket_elems, first_elems):
     return spans
 
 
-def run_c5(args, np, torch, fa, oracle):
+def run_c5(args, np, torch, fa, oracle, shared=None):
     k, numel = args.k or 8, args.numel or 1_370_000_000
     slice_elems = args.slice_bytes // 4
     spans = ddp_buckets(numel, slice_elems, MiB // 4)
@@ -429,8 +442,11 @@ def run_c5(args, np, torch, fa, oracle):
                             slice_size_in_bytes=args.slice_bytes,
                             num_reduce_streams=args.streams,
                             max_launch_bytes=args.launch_bytes)
-    xs = synth(torch, numel, k, "f32", 20240)
-    out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    if shared is not None:   # the inputs of the c2 run (same seeds), still resident
+        xs, out = shared
+    else:
+        xs = synth(torch, numel, k, "f32", 20240)
+        out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
     views = [(out[lo:hi], [x[lo:hi] for x in xs]) for lo, hi in spans]
     torch.cuda.synchronize()
     prepared = {}
@@ -467,6 +483,102 @@ def run_c5(args, np, torch, fa, oracle):
                         numel, len(spans), MiB, args.slice_bytes, k, k),
         "k": k, "numel": numel, "buckets": len(spans), "staging_total_bytes": args.total_memory,
         "layout": layout, "reduce_streams": args.streams or "default",
+    }
+    return value, elapsed, cfg, roof, checked, None, "f32"
+
+
+def run_c5pg(args, np, torch, fa, oracle, shared=None):
+    """The DDP bucket stream of c5 through the surface the reference exposes: one
+    `_fairring.ProcessGroup.allreduce` per bucket on a group of 8 whose 7 other
+    ranks' buckets are resident on the GPU, reduced in place into this rank's
+    gradient with the divide fused, completion through the work's future; every
+    work is waited for at the end of the step, as DDP's reducer does."""
+    import datetime
+
+    import torch.distributed as dist
+
+    import fairring  # noqa: F401  (registers the backend, loads the extension)
+    from fairring_amd import _fairring
+
+    k, numel = args.k or 8, args.numel or 1_370_000_000
+    slice_elems = args.slice_bytes // 4
+    spans = ddp_buckets(numel, slice_elems, MiB // 4)
+    if shared is not None:
+        xs, own = shared       # `own` is overwritten: the group reduces in place
+    else:
+        xs = synth(torch, numel, k, "f32", 20240)
+        own = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    own.copy_(xs[0])
+    torch.cuda.synchronize()
+    o = _fairring.ProcessGroup.Options(
+        max_memory_allocated_in_bytes=args.total_memory, max_padding_allocated_in_bytes=MiB,
+        min_parallelism=2, is_high_priority_stream=True,
+        timeout=datetime.timedelta(seconds=60), slice_size_in_bytes=args.slice_bytes)
+    pg = _fairring.ProcessGroup(dist.HashStore(), 0, k, o)
+    pg._set_fused_divide(True)
+    own_views = [[own[lo:hi]] for lo, hi in spans]
+    peer_views = [[x[lo:hi] for x in xs[1:]] for lo, hi in spans]
+
+    def step():
+        works = []
+        for ov, pv in zip(own_views, peer_views):
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg.allreduce(ov))
+        return works
+
+    def finish(works):
+        for w in works:
+            w.wait()
+
+    for _ in range(max(args.warmup, 1)):
+        finish(step())
+    pg._synchronize()
+    torch.cuda.synchronize()
+    pg._launch_records()        # drop what the warm-up left
+    t0 = time.perf_counter()
+    pg._profile_mark()
+    pending = []
+    for _ in range(args.steps):
+        pending.append(step())
+    pg._profile_mark()
+    for works in pending:
+        finish(works)
+    pg._synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    recs = pg._launch_records()
+    step_bytes = (k + 1) * numel * 4
+    value = step_bytes * args.steps / elapsed / 1e9
+    roof = roofline_from_records(recs, (k + 1) * 4,
+                                 launch_elems(args, slice_elems, slice_elems, 4, k), SPAN_HOW)
+    roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
+    # parity on a fresh copy of this rank's gradient (the timed steps reduced in place)
+    own.copy_(xs[0])
+    finish(step())
+    pg._synchronize()
+    torch.cuda.synchronize()
+    checked = check_parity(oracle, np, torch, xs, own, numel, slice_elems, k, "f32", True)
+    chain = xs[0].clone()
+    for x in xs[1:]:
+        chain.add_(x)
+    chain.mul_(1.0 / k)
+    same = torch.equal(own.view(torch.int32), chain.view(torch.int32))
+    del chain
+    if not same:
+        raise SystemExit("parity FAILED against the at::add chain on the GPU (c5pg)")
+    checked = "%s; every element equal to torch's at::add chain on the GPU" % checked
+    layout = pg._layout()
+    del pg
+    cfg = {
+        "workload": "DDP backward stream through _fairring.ProcessGroup.allreduce: %d fp32 "
+                    "elements as %d buckets (first %d B, then %d B) released from the end of the "
+                    "gradient to its start, group of %d (7 simulated peers resident on the GPU), "
+                    "in place, fused x1/%d, every work waited for at the end of the step "
+                    "(configs[4] through the drop-in surface)" % (
+                        numel, len(spans), MiB, args.slice_bytes, k, k),
+        "k": k, "numel": numel, "buckets": len(spans), "staging_total_bytes": args.total_memory,
+        "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
+                   "staging_slots": layout[3]},
     }
     return value, elapsed, cfg, roof, checked, None, "f32"
 
@@ -666,24 +778,65 @@ def main():
     if args.workload == "smallops":
         run_small_ops(args, torch, fa)
         return
-    if args.workload in ("c2", "copy"):
-        value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,
-                                                                       oracle, "f32")
-    elif args.workload == "c4":
+
+    keep = []
+    result = measure(args, args.workload, np, torch, fa, oracle, keep=keep)
+    failed = []
+    if args.workload == "c2" and not args.no_extra_configs and not (
+            args.k or args.numel or args.launch_bytes or args.streams or args.blocks_per_cu):
+        # The other workloads, briefly, for the record: same code paths as when
+        # they are run on their own, fewer steps, no CPU baseline.
+        shared = tuple(keep) if keep else None
+        extra = {}
+        for name in ("c5", "c5pg", "c4", "hook", "c3"):
+            sub = argparse.Namespace(**vars(args))
+            sub.workload, sub.no_cpu_baseline = name, True
+            sub.steps, sub.warmup = min(args.steps, 3 if name == "c3" else 10), 2
+            if name == "c4":
+                shared = None
+                keep.clear()       # the fp32 inputs go before the bf16 ones are made
+            try:
+                r = measure(sub, name, np, torch, fa, oracle,
+                            shared=shared if name in ("c5", "c5pg") else None)
+                extra[name] = {key: r[key] for key in ("metric", "value", "unit", "steps",
+                                                       "ms_per_step", "dtype", "pct_of_hbm_peak",
+                                                       "parity", "roofline")}
+                extra[name]["workload"] = r["config"]["workload"]
+                if "host_link_GBps" in r["config"]:
+                    extra[name]["host_link_GBps"] = r["config"]["host_link_GBps"]
+            except (SystemExit, Exception) as e:  # noqa: BLE001  (reported, and the run fails)
+                extra[name] = {"error": "%s: %s" % (type(e).__name__, e)}
+                failed.append(name)
+        result["configs"] = extra
+    print(json.dumps(result))
+    if failed:
+        sys.exit("workloads that failed: %s" % ", ".join(failed))
+
+
+def measure(args, workload, np, torch, fa, oracle, keep=None, shared=None):
+    """Runs one workload and returns its result line as a dict."""
+    if workload in ("c2", "copy"):
+        value, elapsed, cfg, roof, checked, base, dtype = run_resident(
+            args, np, torch, fa, oracle, "f32", keep=keep if workload == "c2" else None)
+    elif workload == "c4":
         value, elapsed, cfg, roof, checked, base, dtype = run_resident(args, np, torch, fa,
                                                                        oracle, "bf16")
-    elif args.workload == "c3":
+    elif workload == "c3":
         value, elapsed, cfg, roof, checked, base, dtype = run_c3(args, np, torch, fa, oracle)
-    elif args.workload == "hook":
+    elif workload == "hook":
         value, elapsed, cfg, roof, checked, base, dtype = run_hook(args, np, torch, fa, oracle)
+    elif workload == "c5pg":
+        value, elapsed, cfg, roof, checked, base, dtype = run_c5pg(args, np, torch, fa, oracle,
+                                                                   shared=shared)
     else:
-        value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle)
+        value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle,
+                                                                 shared=shared)
 
     # HBM bytes per launch as measured with rocprofv3 --pmc (two counter runs,
-    # scaled by a copy of known size); the summary that holds the figure names
-    # the commands that produced it.
+    # scaled by a copy of known size) in an earlier run of the same command: a
+    # constant read from the summary named in traffic_source, not measured now.
     traffic_file = {"c2": "ksum_f32_k8_c2_hbm_traffic.md",
-                    "hook": "compressed_bf16_k8_hook_hbm_traffic.md"}.get(args.workload)
+                    "hook": "compressed_bf16_k8_hook_hbm_traffic.md"}.get(workload)
     if (traffic_file and args.slice_bytes == 25 * MiB and not args.k and not args.numel
             and not args.launch_bytes):
         tpath = os.path.join(ROOT, "profiles", traffic_file)
@@ -692,15 +845,20 @@ def main():
             m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", open(tpath).read())
             if m:
                 roof["traffic"] = int(m.group(1).replace(",", ""))
+                roof["traffic_source"] = ("profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                          "of an earlier run of this command; not measured in "
+                                          "this run)" % traffic_file)
 
     metric = {
         "c2": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",
         "c4": "reduce GB/s (bytes read+written), 8-way bf16, 25 MiB slices",
         "c3": "reduce GB/s (bytes read+written at HBM level), 64-way fp32 host-staged, one slice",
         "c5": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream",
+        "c5pg": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream through "
+                "ProcessGroup.allreduce",
         "copy": "copy GB/s (bytes read+written), 25 MiB slices",
         "hook": "reduce GB/s (bytes read+written), 8-way with the bf16 compression hook folded in",
-    }[args.workload]
+    }[workload]
     result = {
         "metric": metric,
         "value": round(value, 1),
@@ -722,7 +880,7 @@ def main():
     }
     if base is not None:
         result["cpu_baseline"] = base
-    print(json.dumps(result))
+    return result
 
 
 if __name__ == "__main__":

@@ -19,7 +19,7 @@ SCALE_PRE_MUL, SCALE_PRE_DIV = 3, 4
 EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_reduce_slice",
     "frg_reduce_slice_compressed", "frg_allreduce_compressed",
-    "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_allreduce", "frg_allreduce_host",
+    "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
     "frg_set_tuning",
@@ -88,6 +88,7 @@ def lib():
     L.frg_destroy.argtypes = [vp]
     L.frg_get_layout.argtypes = [vp, ctypes.POINTER(Layout)]
     L.frg_get_streams.argtypes = [vp, pvp, i32, ctypes.POINTER(i32)]
+    L.frg_get_copy_streams.argtypes = [vp, pvp, i32, ctypes.POINTER(i32)]
     L.frg_allreduce.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
     L.frg_reduce_slice_compressed.argtypes = [vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp]
     L.frg_allreduce_compressed.argtypes = [vp, vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp,

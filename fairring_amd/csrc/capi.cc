@@ -193,6 +193,16 @@ int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count) {
   });
 }
 
+int frg_get_copy_streams(frg_ctx* ctx, void** streams, int capacity, int* count) {
+  if (ctx == nullptr || count == nullptr) return fail(FRG_ERR_INVALID, "null argument");
+  return guarded([&] {
+    const std::vector<hipStream_t> v = asCtx(ctx)->copyStreams();
+    *count = static_cast<int>(v.size());
+    for (int i = 0; i < *count && i < capacity && streams != nullptr; ++i) streams[i] = v[i];
+    return static_cast<int>(FRG_OK);
+  });
+}
+
 int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, int64_t numel,
                   int dtype, int op, int scale_mode, float scale, void* producer_stream,
                   frg_done_fn done, void* user, frg_work** work) {

@@ -24,7 +24,7 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
-#include <mutex>
+#include <atomic>
 
 #include "../../include/fairring_hip.h"
 #include "device_traits.h"
@@ -389,10 +389,11 @@ hipError_t dispatchType(const ReduceArgs& a, int64_t head, int64_t nvec, int64_t
 }  // namespace
 
 int computeUnits(int device) {
-  static std::mutex mu;
-  static int cusOf[64];
-  std::lock_guard<std::mutex> g(mu);
-  int& cus = cusOf[device & 63];
+  // asked on every launch: a relaxed load once the device is known (two threads
+  // that ask first at the same time both ask the runtime and store the same answer)
+  static std::atomic<int> cusOf[64];
+  std::atomic<int>& slot = cusOf[device & 63];
+  int cus = slot.load(std::memory_order_relaxed);
   if (cus == 0) {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) !=
             hipSuccess ||
@@ -400,6 +401,7 @@ int computeUnits(int device) {
       (void)hipGetLastError();
       cus = 256;
     }
+    slot.store(cus, std::memory_order_relaxed);
   }
   return cus;
 }

@@ -100,6 +100,11 @@ inline constexpr int64_t defaultCompressedLaunchBytes(int numContribs, bool rawT
   const int64_t rounds = (perContrib + kCompressedRoundBytes - 1) / kCompressedRoundBytes;
   return (rounds < 1 ? 1 : rounds) * kCompressedRoundBytes;
 }
+// An operation of at most this many launches runs on one reduce stream, and
+// the next operation on the next stream; a longer one deals its launches over
+// all of them. With the default shapes that is every operation below 100 MiB
+// per contribution (8 launches of 12.5 MiB), where the whole-round shape begins.
+constexpr int kOneStreamLaunches = 8;
 constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {

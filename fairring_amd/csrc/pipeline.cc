@@ -56,17 +56,52 @@ class DeviceGuard {
 void setLastError(const std::string& msg) { tlsError = msg; }
 const char* lastError() { return tlsError.c_str(); }
 
+namespace {
+
+// How long a thread polls for something it expects within microseconds before
+// it goes to sleep on a condition variable.
+constexpr std::chrono::microseconds kSpinBeforeSleep{60};
+
+inline void cpuRelax() {
+#if defined(__x86_64__) || defined(__i386__)
+  __builtin_ia32_pause();
+#else
+  std::this_thread::yield();
+#endif
+}
+
+// Polls `ready` for at most kSpinBeforeSleep; true as soon as it holds.
+template <typename F>
+bool spinFor(F&& ready) {
+  if (ready()) return true;
+  const auto until = std::chrono::steady_clock::now() + kSpinBeforeSleep;
+  for (;;) {
+    for (int i = 0; i < 32; ++i) {
+      if (ready()) return true;
+      cpuRelax();
+    }
+    if (std::chrono::steady_clock::now() > until) return false;
+  }
+}
+
+}  // namespace
+
 void CommandQueue::enqueue(std::function<void()> fn) {
-  std::unique_lock<std::mutex> lock(mutex_);
-  fns_.push_back(std::move(fn));
+  {
+    std::unique_lock<std::mutex> lock(mutex_);
+    fns_.push_back(std::move(fn));
+    pending_.fetch_add(1, std::memory_order_release);
+  }
   cv_.notify_one();
 }
 
 std::function<void()> CommandQueue::dequeue() {
+  spinFor([&] { return pending_.load(std::memory_order_acquire) > 0; });
   std::unique_lock<std::mutex> lock(mutex_);
   cv_.wait(lock, [&] { return !fns_.empty(); });
   std::function<void()> fn = std::move(fns_.front());
   fns_.pop_front();
+  pending_.fetch_sub(1, std::memory_order_relaxed);
   return fn;
 }
 
@@ -136,14 +171,19 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
       FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
       c->reduceStreams_.push_back(s);
     }
-    const int nCopy = o.num_copy_streams > 0 ? o.num_copy_streams : 2;
-    for (int i = 0; i < nCopy && i < 4; ++i) {
-      hipStream_t s;
-      FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-      c->copyStreams_.push_back(s);
-    }
+    // The copy streams of the host-staged path are created when that path is
+    // first used (copyStreams()): until then the context holds its reduce
+    // streams only.
+    c->numCopyStreams_ = o.num_copy_streams > 0 ? (o.num_copy_streams < 4 ? o.num_copy_streams : 4)
+                                                : 2;
     FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->stagingPool_),
                             static_cast<size_t>(c->numSlots_ * c->slotBytes_)));
+    // The scratch of the launch chains, here rather than on first use: an
+    // allocation that fails in the middle of training would only surface as an
+    // asynchronous failure of some operation.
+    FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->carryScratch_),
+                            c->reduceStreams_.size() *
+                                static_cast<size_t>(c->carryScratchBytes_ + 16)));
     for (int64_t i = 0; i < c->numSlots_; ++i) {
       hipEvent_t a, b;
       FRG_HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
@@ -154,11 +194,17 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
     c->slotUsed_.assign(static_cast<size_t>(c->numSlots_), 0);
     c->streamLaunches_.assign(c->reduceStreams_.size(), 0);
     c->streamElems_.assign(c->reduceStreams_.size(), 0);
+    c->history_.resize(c->reduceStreams_.size());
+    c->orderedAfter_.assign(c->reduceStreams_.size(),
+                            std::vector<int64_t>(c->reduceStreams_.size(), 0));
   } catch (const std::exception& e) {
     *err = e.what();
     // partially built: the destructor releases what exists (there is no command
-    // thread to join yet)
+    // thread to join yet). Nothing has run on the streams and nobody else has
+    // seen them, so unlike those of a context that worked they can go.
+    std::vector<hipStream_t> made = c->reduceStreams_;
     delete c;
+    for (hipStream_t s : made) (void)hipStreamDestroy(s);
     return FRG_ERR_HIP;
   }
 
@@ -200,6 +246,34 @@ Context::~Context() {
   // The streams are not destroyed: a consumer may still hold an event that
   // orders its own stream after one of them (fairring/machine.cc:162-175).
   (void)hipSetDevice(prev);
+}
+
+std::vector<hipStream_t> Context::copyStreams() {
+  std::lock_guard<std::mutex> g(copyMu_);
+  if (copyStreams_.empty()) {
+    DeviceGuard dg(device_);
+    std::vector<hipStream_t> made;
+    try {
+      for (int i = 0; i < numCopyStreams_; ++i) {
+        hipStream_t s;
+        // default priority, like the reduce streams
+        FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+        made.push_back(s);
+      }
+    } catch (...) {
+      for (hipStream_t s : made) (void)hipStreamDestroy(s);
+      throw;
+    }
+    copyStreams_ = std::move(made);
+  }
+  return copyStreams_;
+}
+
+std::vector<hipStream_t> Context::streams() {
+  std::vector<hipStream_t> v = reduceStreams_;
+  std::lock_guard<std::mutex> g(copyMu_);
+  v.insert(v.end(), copyStreams_.begin(), copyStreams_.end());
+  return v;
 }
 
 hipEvent_t Context::takeEvent() {
@@ -263,6 +337,8 @@ int Context::waitWork(Work* w, std::string* err) {
   const auto deadline = std::chrono::steady_clock::now() +
                         std::chrono::duration_cast<std::chrono::steady_clock::duration>(
                             std::chrono::duration<double>(limit));
+  // a small operation is enqueued within microseconds: poll before sleeping
+  spinFor([&] { return w->enqueuedFlag.load(std::memory_order_acquire); });
   {
     std::unique_lock<std::mutex> lock(w->mu);
     if (limit > 0.0) {
@@ -318,9 +394,23 @@ int Context::waitWork(Work* w, std::string* err) {
 }
 
 int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
+  const double limit = waitTimeoutSeconds();
   {
     std::unique_lock<std::mutex> lock(w->mu);
-    w->cv.wait(lock, [&] { return w->enqueued; });
+    if (limit > 0.0) {
+      // the host's share of this call is the enqueue; it gives up like frg_work_wait
+      const auto wallDeadline =
+          std::chrono::system_clock::now() +
+          std::chrono::duration_cast<std::chrono::system_clock::duration>(
+              std::chrono::duration<double>(limit));
+      if (!w->cv.wait_until(lock, wallDeadline, [&] { return w->enqueued; })) {
+        *err = "gave up after " + std::to_string(limit) +
+               " s waiting for the command thread to enqueue " + progressReport(w);
+        return FRG_ERR_NOT_READY;
+      }
+    } else {
+      w->cv.wait(lock, [&] { return w->enqueued; });
+    }
     if (w->status != FRG_OK) {
       *err = w->error;
       return w->status;
@@ -502,16 +592,11 @@ void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
   launchAndCount<CompressedArgs>(args, stream, &launchCompressedReduce);
 }
 
-// The scratch region of a reduce stream (allocated on first use; reused in
-// stream order), placed so that the vector variant of the kernel still runs:
+// The scratch region of a reduce stream (reused in stream order), placed so that the vector variant of the kernel still runs:
 // at the same position within 16 bytes as `like` for a buffer of the storage
 // type, or, for fp32 accumulators of a 2-byte type, such that it reaches a
 // 16-byte boundary after as many elements as `like` does.
 char* Context::scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize) {
-  if (carryScratch_ == nullptr) {
-    FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&carryScratch_),
-                            reduceStreams_.size() * static_cast<size_t>(carryScratchBytes_ + 16)));
-  }
   char* base = carryScratch_ + streamIdx * static_cast<size_t>(carryScratchBytes_ + 16);
   const uintptr_t pos = reinterpret_cast<uintptr_t>(like) & 15;
   if (!acc) return base + pos;
@@ -556,6 +641,95 @@ void Context::chainThroughScratch(const Request& req, const std::vector<const vo
       a.carry_src = scratch;
       a.carry_acc = acc;
       launch(a, s);
+    }
+  }
+}
+
+// ---- order between operations ----------------------------------------------
+
+Context::OpSpans Context::spansOf(const Request& req) {
+  OpSpans op;
+  const uintptr_t wireSize = static_cast<uintptr_t>(elementSize(req.dtype));
+  const uintptr_t outSize =
+      req.compressed ? static_cast<uintptr_t>(elementSize(req.outDtype)) : wireSize;
+  const uintptr_t n = static_cast<uintptr_t>(req.numel);
+  const uintptr_t o = reinterpret_cast<uintptr_t>(req.out);
+  op.write = Span{o, o + n * outSize};
+  if (!req.fromHost) {  // host memory is not written by any operation of the pipeline
+    op.reads.reserve(req.contribs.size());
+    for (size_t k = 0; k < req.contribs.size(); ++k) {
+      const uintptr_t p = reinterpret_cast<uintptr_t>(req.contribs[k]);
+      if (p == o) continue;  // in place: covered by the write
+      const uintptr_t es = (req.compressed && static_cast<int>(k) == req.rawIndex) ? 4 : wireSize;
+      op.reads.push_back(Span{p, p + n * es});
+    }
+  }
+  return op;
+}
+
+// Two operations conflict when one writes what the other reads or writes.
+bool Context::conflict(const OpSpans& a, const OpSpans& b) {
+  auto overlap = [](const Span& x, const Span& y) { return x.lo < y.hi && y.lo < x.hi; };
+  if (overlap(a.write, b.write)) return true;
+  for (const Span& r : b.reads) {
+    if (overlap(a.write, r)) return true;
+  }
+  for (const Span& r : a.reads) {
+    if (overlap(r, b.write)) return true;
+  }
+  return false;
+}
+
+void Context::joinTail(size_t src, size_t target) {
+  hipEvent_t e = takeEvent();
+  hipError_t r = hipEventRecord(e, reduceStreams_[src]);
+  if (r == hipSuccess) r = hipStreamWaitEvent(reduceStreams_[target], e, 0);
+  giveEvent(e);  // the wait holds what it needs of the record
+  FRG_HIP_CHECK(r);
+  if (!history_[src].empty()) orderedAfter_[target][src] = history_[src].back().seq;
+}
+
+void Context::orderAfterConflicts(const OpSpans& op, const std::vector<size_t>& targets) {
+  const size_t n = reduceStreams_.size();
+  if (n < 2) return;
+  for (size_t s = 0; s < n; ++s) {
+    if (history_[s].empty()) continue;
+    for (size_t t : targets) {
+      if (t == s) continue;
+      const int64_t seen = orderedAfter_[t][s];
+      bool hit = false;
+      // newest first: what conflicts is most often what was submitted last
+      for (auto it = history_[s].rbegin(); it != history_[s].rend() && it->seq > seen; ++it) {
+        if (conflict(op, *it)) {
+          hit = true;
+          break;
+        }
+      }
+      if (hit) joinTail(s, t);
+    }
+  }
+}
+
+void Context::remember(OpSpans op, const std::vector<size_t>& targets) {
+  const size_t n = reduceStreams_.size();
+  if (n < 2 || op.write.lo == op.write.hi) return;
+  op.seq = ++spanSeq_;
+  for (size_t t : targets) {
+    std::deque<OpSpans>& h = history_[t];
+    h.push_back(op);
+    // what every other stream already follows need not be kept
+    int64_t followed = h.back().seq;
+    for (size_t u = 0; u < n; ++u) {
+      if (u != t && orderedAfter_[u][t] < followed) followed = orderedAfter_[u][t];
+    }
+    while (!h.empty() && h.front().seq <= followed) h.pop_front();
+    if (h.size() > kMaxHistory) {
+      // bounded memory and search: order every other stream after this one
+      // (one event record, one wait per stream, once in kMaxHistory operations)
+      for (size_t u = 0; u < n; ++u) {
+        if (u != t) joinTail(t, u);
+      }
+      h.clear();
     }
   }
 }
@@ -646,10 +820,29 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     if (req.numel > off) ranges.emplace_back(off, req.numel - off);
   }
 
+  // An operation of a few launches (a DDP bucket) stays on one stream and the
+  // next operation takes the next stream: neighbouring operations overlap, each
+  // ends on a single stream (nothing to join for its completion), and nothing is
+  // recorded between two launches. A large operation deals its own launches
+  // round-robin over the streams.
+  const bool oneStream = ranges.size() <= static_cast<size_t>(kOneStreamLaunches);
+  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
+  if (oneStream && !ranges.empty()) ++nextLaunch_;
+  const OpSpans spans = spansOf(req);
+  std::vector<size_t> targets;
+  if (!ranges.empty()) {
+    if (oneStream) {
+      targets.push_back(opStream);
+    } else {
+      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
+    }
+    orderAfterConflicts(spans, targets);
+  }
+
   for (const auto& range : ranges) {
     const int64_t off = range.first;
     const int64_t len = range.second;
-    const size_t si = static_cast<size_t>(nextLaunch_++) % nStreams;
+    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
     hipStream_t s = reduceStreams_[si];
     if (!waited[si]) {
       // Only the first launch on a stream needs the producer's event; later
@@ -703,6 +896,13 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     }
     lastIdx = si;
   }
+  if (!ranges.empty()) {
+    std::vector<size_t> ran;
+    for (size_t si = 0; si < nStreams; ++si) {
+      if (waited[si]) ran.push_back(si);
+    }
+    remember(spans, ran);
+  }
   // The streams that took part, the one of the last launch at the back.
   if (!waited[lastIdx]) {
     waitInitial(reduceStreams_[lastIdx], initialEvent, &initialFired);
@@ -730,10 +930,26 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       layout_.sliceSizeInBytes < slotBytes_ ? layout_.sliceSizeInBytes : slotBytes_;
   const int K = static_cast<int>(req.contribs.size());
   hipStream_t s = reduceStreams_[0];
+  const std::vector<hipStream_t> copies = copyStreams();  // created on first use
+  // The copy streams write `out` and the slots and know nothing of earlier
+  // operations: the whole operation is ordered after everything enqueued so far
+  // (it is bound by the host link; two event packets do not show).
+  for (size_t src = 1; src < reduceStreams_.size(); ++src) {
+    if (!history_[src].empty()) joinTail(src, 0);
+  }
+  {
+    hipEvent_t tail = takeEvent();
+    hipError_t r = hipEventRecord(tail, s);
+    for (hipStream_t cs : copies) {
+      if (r == hipSuccess) r = hipStreamWaitEvent(cs, tail, 0);
+    }
+    giveEvent(tail);
+    FRG_HIP_CHECK(r);
+  }
   bool initialFired = false;
   waitInitial(s, initialEvent, &initialFired);
-  for (hipStream_t cs : copyStreams_) waitInitial(cs, initialEvent, &initialFired);
-  const size_t nCopy = copyStreams_.size();
+  for (hipStream_t cs : copies) waitInitial(cs, initialEvent, &initialFired);
+  const size_t nCopy = copies.size();
   int64_t batch = numSlots_ / 2;
   if (batch < 1) batch = 1;
   if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
@@ -758,9 +974,9 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       // contribution 0 needs no staging: it lands in `out` directly
       FRG_HIP_CHECK(hipMemcpyAsync(outp,
                                    static_cast<const char*>(req.contribs[0]) + off * elsize,
-                                   bytes, hipMemcpyHostToDevice, copyStreams_[0]));
+                                   bytes, hipMemcpyHostToDevice, copies[0]));
       hipEvent_t first = takeEvent();
-      FRG_HIP_CHECK(hipEventRecord(first, copyStreams_[0]));
+      FRG_HIP_CHECK(hipEventRecord(first, copies[0]));
       FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
       giveEvent(first);
       firstStaged = 1;
@@ -790,7 +1006,7 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       slots.clear();
       for (; k < K && static_cast<int64_t>(staged.size()) < batch; ++k) {
         const int64_t slot = (nextStagingSlot_++) % numSlots_;
-        hipStream_t cs = copyStreams_[static_cast<size_t>(slot) % nCopy];
+        hipStream_t cs = copies[static_cast<size_t>(slot) % nCopy];
         if (slotUsed_[slot]) {
           FRG_HIP_CHECK(hipStreamWaitEvent(cs, slotFreeEvents_[slot], 0));
         }
@@ -835,6 +1051,8 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
     // The next slice's first copy overwrites nothing this slice still reads
     // (it targets another range of `out`), so no extra wait is needed here.
   }
+  // every copy of the operation has been joined into the reduce stream
+  if (req.numel > 0) remember(spansOf(req), {0});
   return {s};
 }
 
@@ -881,6 +1099,7 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
     work->error = error;
     work->lastStream = lastStream;
     work->enqueued = true;
+    work->enqueuedFlag.store(true, std::memory_order_release);
   }
   work->cv.notify_all();
   if (req.done) req.done(req.user, status, lastStream);

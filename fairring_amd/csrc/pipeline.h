@@ -26,12 +26,15 @@ namespace frg {
 class CommandQueue {
  public:
   void enqueue(std::function<void()> fn);
+  // Polls for a short while before it sleeps: a sleeping thread takes tens of
+  // microseconds to wake, which is most of what a small operation costs.
   std::function<void()> dequeue();
 
  private:
   std::mutex mutex_;
   std::condition_variable cv_;
   std::deque<std::function<void()>> fns_;
+  std::atomic<int64_t> pending_{0};  // closures enqueued and not yet taken
 };
 
 // Progress counters of a context, shared with the works it hands out so that a
@@ -50,6 +53,7 @@ struct Work {
   std::mutex mu;
   std::condition_variable cv;
   bool enqueued = false;  // the command thread is done with it
+  std::atomic<bool> enqueuedFlag{false};  // the same, for a waiter that polls first
   int status = FRG_OK;
   std::string error;
   // The streams the operation's work ended on. No event is recorded per
@@ -73,11 +77,12 @@ class Context {
   const Layout& layout() const { return layout_; }
   int device() const { return device_; }
   const Progress& progress() const { return *progress_; }
-  std::vector<hipStream_t> streams() const {
-    std::vector<hipStream_t> v = reduceStreams_;
-    v.insert(v.end(), copyStreams_.begin(), copyStreams_.end());
-    return v;
-  }
+  // The reduce streams, then the copy streams that exist so far.
+  std::vector<hipStream_t> streams();
+  // The copy streams of the host-staged path, created on first use: a context
+  // that only reduces resident tensors holds its reduce streams and no more.
+  // Throws on a HIP failure.
+  std::vector<hipStream_t> copyStreams();
 
   struct Request {
     void* out = nullptr;
@@ -137,6 +142,38 @@ class Context {
   hipEvent_t takeEvent();
   void giveEvent(hipEvent_t e);
 
+  // ---- order between operations ------------------------------------------
+  // Operations are dealt to the reduce streams so that neighbours overlap, but
+  // a caller sees one pipeline: an operation that touches memory an earlier one
+  // on another stream wrote (or writes what that one read) must run after it,
+  // as it would on the reference's single chain of streams
+  // (fairring/device.cc:291-353). The command thread keeps, per reduce stream,
+  // the address ranges of the operations enqueued there that some other stream
+  // is not yet ordered after; a new operation is checked against them and its
+  // streams wait on the tails of the streams it conflicts with: one event
+  // record and wait per conflict, nothing for independent buckets.
+  struct Span {
+    uintptr_t lo = 0;
+    uintptr_t hi = 0;
+  };
+  struct OpSpans {
+    int64_t seq = 0;
+    Span write;
+    std::vector<Span> reads;
+  };
+  static OpSpans spansOf(const Request& req);
+  static bool conflict(const OpSpans& a, const OpSpans& b);
+  // Makes every stream in `targets` wait for what `op` conflicts with on the
+  // other reduce streams.
+  void orderAfterConflicts(const OpSpans& op, const std::vector<size_t>& targets);
+  // Makes `target` wait for everything enqueued on reduce stream `src` so far.
+  void joinTail(size_t src, size_t target);
+  void remember(OpSpans op, const std::vector<size_t>& targets);
+  static constexpr size_t kMaxHistory = 32;  // operations remembered per stream
+  std::vector<std::deque<OpSpans>> history_;         // per reduce stream, oldest first
+  std::vector<std::vector<int64_t>> orderedAfter_;   // [t][s]: t follows s's history up to this seq
+  int64_t spanSeq_ = 0;
+
   int device_ = 0;
   Layout layout_;
   int64_t numSlots_ = 0;
@@ -149,6 +186,8 @@ class Context {
   // Slot s is filled on copy stream s % copyStreams_.size(): while one stream works through the
   // event packets around its copy, the other's copy keeps the host link busy.
   std::vector<hipStream_t> copyStreams_;
+  int numCopyStreams_ = 2;
+  std::mutex copyMu_;  // guards the creation of copyStreams_
 
   char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
   // Allocated on first use, one region per reduce stream: carries the partial

@@ -48,6 +48,10 @@ void bind(py::module& m) {
             py::arg("peers"), py::call_guard<py::gil_scoped_release>());
   group.def("_set_fused_divide", &PG::setFusedDivide, py::arg("on"));
   group.def("_layout", &PG::layout);
+  // measurement hooks of the pipeline behind the group (include/fairring_hip.h)
+  group.def("_profile_mark", &PG::profileMark, py::call_guard<py::gil_scoped_release>());
+  group.def("_launch_records", &PG::launchRecords, py::call_guard<py::gil_scoped_release>());
+  group.def("_synchronize", &PG::synchronizeAll, py::call_guard<py::gil_scoped_release>());
   // the allreduce with one of torch's DDP communication hooks folded in
   group.def("_allreduce_pre_divided", &PG::allreducePreDivided, py::arg("bucket"),
             py::call_guard<py::gil_scoped_release>());

@@ -84,6 +84,27 @@ void onDone(void* user, int status, void* lastStream) {
   }
 }
 
+// Lets go of Python's global lock for a scope if this thread holds it. The
+// command thread's completion callbacks may need that lock (a future's Python
+// callbacks; the last reference to a tensor that Python created), so nothing
+// here may wait for the command thread while holding it. Python's bindings of
+// Work.wait and Future.wait let go of it themselves; those of Work.result and
+// Work.synchronize, and the deallocation of a group, do not.
+class GilRelease {
+ public:
+  GilRelease() {
+    if (Py_IsInitialized() && PyGILState_Check()) saved_ = PyEval_SaveThread();
+  }
+  ~GilRelease() {
+    if (saved_ != nullptr) PyEval_RestoreThread(saved_);
+  }
+  GilRelease(const GilRelease&) = delete;
+  GilRelease& operator=(const GilRelease&) = delete;
+
+ private:
+  PyThreadState* saved_ = nullptr;
+};
+
 }  // namespace
 
 // ---- WorkFairring ---------------------------------------------------------
@@ -120,6 +141,22 @@ void ProcessGroupFairring::WorkFairring::awaitCompletion() {
     const double s = v ? std::atof(v) : 0.0;
     return s > 0.0 ? s : 0.0;
   }();
+  if (future_->completed()) {
+    future_->wait();  // orders the current stream after the result, no more
+    return;
+  }
+  GilRelease unlocked;
+  // A small operation completes within microseconds of the call: poll for a
+  // short while before sleeping on the future (a sleeping thread takes tens of
+  // microseconds to wake).
+  {
+    const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(60);
+    while (!future_->completed() && std::chrono::steady_clock::now() < until) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+    }
+  }
   if (limit > 0.0) {
     const auto deadline = std::chrono::steady_clock::now() +
                           std::chrono::duration_cast<std::chrono::steady_clock::duration>(
@@ -193,12 +230,9 @@ ProcessGroupFairring::~ProcessGroupFairring() {
   // Destroying a context drains its command thread, whose completion callbacks
   // may run Python code (future.then) or drop the last reference to a tensor
   // that Python created: both take the GIL. When this destructor runs from
-  // Python's deallocation of the group, the GIL is held here, so let go of it
-  // for the duration.
-  PyThreadState* saved = nullptr;
-  if (Py_IsInitialized() && PyGILState_Check()) saved = PyEval_SaveThread();
+  // Python's deallocation of the group, the GIL is held here.
+  GilRelease unlocked;
   for (auto& kv : contexts_) frg_destroy(kv.second);
-  if (saved != nullptr) PyEval_RestoreThread(saved);
 }
 
 const std::string ProcessGroupFairring::getBackendName() const { return kPgName; }
@@ -230,6 +264,7 @@ frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
                  static_cast<int>(device), static_cast<long long>(l.num_staging_slots),
                  static_cast<long long>(l.slice_size_in_bytes));
   }
+  // the reduce streams; the copy streams do not exist until something is staged
   void* raw[16];
   int nStreams = 0;
   TORCH_CHECK(frg_get_streams(ctx, raw, 16, &nStreams) == FRG_OK, frg_last_error());
@@ -242,21 +277,37 @@ frg_ctx* ProcessGroupFairring::contextFor(c10::DeviceIndex device) {
   return ctx;
 }
 
+const std::vector<c10::Stream>& ProcessGroupFairring::copyStreamsFor(c10::DeviceIndex device,
+                                                                     frg_ctx* ctx) {
+  std::vector<c10::Stream>& streams = copyStreams_[device];
+  if (streams.empty()) {
+    void* raw[8];
+    int n = 0;
+    TORCH_CHECK(frg_get_copy_streams(ctx, raw, 8, &n) == FRG_OK, frg_last_error());
+    for (int i = 0; i < n && i < 8; ++i) {
+      streams.push_back(c10::hip::getStreamFromExternalMasqueradingAsCUDA(
+          static_cast<hipStream_t>(raw[i]), device));
+    }
+  }
+  return streams;
+}
+
 // Tells the caching allocator which streams will touch these buffers
 // (fairring/device.cc:297-301): the reduce streams, and the copy streams as
 // well when contributions are staged from the host (they write `out`).
 void ProcessGroupFairring::recordOnPipelineStreams(
     c10::DeviceIndex device, bool copyStreamsToo, std::initializer_list<const at::Tensor*> tensors,
     const std::vector<at::Tensor>* more) {
-  const std::vector<c10::Stream>& streams = streams_[device];
-  const size_t n = copyStreamsToo ? streams.size()
-                                  : std::min(streams.size(), static_cast<size_t>(kNumReduceStreams));
-  for (size_t i = 0; i < n; ++i) {
-    for (const at::Tensor* t : tensors) t->record_stream(streams[i]);
-    if (more != nullptr) {
-      for (const at::Tensor& t : *more) t.record_stream(streams[i]);
+  auto record = [&](const std::vector<c10::Stream>& streams) {
+    for (const c10::Stream& s : streams) {
+      for (const at::Tensor* t : tensors) t->record_stream(s);
+      if (more != nullptr) {
+        for (const at::Tensor& t : *more) t.record_stream(s);
+      }
     }
-  }
+  };
+  record(streams_[device]);
+  if (copyStreamsToo) record(copyStreamsFor(device, contexts_.at(device)));
 }
 
 void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor> peers) {
@@ -276,6 +327,41 @@ std::vector<int64_t> ProcessGroupFairring::layout() {
   TORCH_CHECK(frg_get_layout(contexts_.begin()->second, &l) == FRG_OK, frg_last_error());
   return {l.slot_size_in_bytes, l.slice_size_in_bytes, l.num_padding_slots,
           l.num_staging_slots};
+}
+
+void ProcessGroupFairring::profileMark() {
+  std::lock_guard<std::mutex> g(mutex_);
+  TORCH_CHECK(!contexts_.empty(), "fairring: no device initialised yet");
+  TORCH_CHECK(frg_profile_mark(contexts_.begin()->second) == FRG_OK, frg_last_error());
+}
+
+std::vector<std::tuple<double, double, int64_t, int, int, int>>
+ProcessGroupFairring::launchRecords() {
+  frg_ctx* ctx = nullptr;
+  {
+    std::lock_guard<std::mutex> g(mutex_);
+    TORCH_CHECK(!contexts_.empty(), "fairring: no device initialised yet");
+    ctx = contexts_.begin()->second;
+  }
+  std::vector<frg_launch_record> recs(1 << 16);
+  int n = 0;
+  TORCH_CHECK(frg_launch_records(ctx, recs.data(), static_cast<int>(recs.size()), &n) == FRG_OK,
+              frg_last_error());
+  std::vector<std::tuple<double, double, int64_t, int, int, int>> out;
+  for (int i = 0; i < n && i < static_cast<int>(recs.size()); ++i) {
+    out.emplace_back(recs[i].begin_ms, recs[i].end_ms, recs[i].numel, recs[i].num_contributions,
+                     recs[i].stream_index, recs[i].launches);
+  }
+  return out;
+}
+
+void ProcessGroupFairring::synchronizeAll() {
+  std::vector<frg_ctx*> all;
+  {
+    std::lock_guard<std::mutex> g(mutex_);
+    for (auto& kv : contexts_) all.push_back(kv.second);
+  }
+  for (frg_ctx* ctx : all) TORCH_CHECK(frg_synchronize(ctx) == FRG_OK, frg_last_error());
 }
 
 c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduce(

@@ -144,6 +144,15 @@ class ProcessGroupFairring : public c10d::Backend {
   // {slot size, slice size, padding slots, staging slots} once initialised.
   std::vector<int64_t> layout();
 
+  // Not in the reference: the measurement hooks of the pipeline behind the
+  // group (frg_profile_mark / frg_launch_records / frg_synchronize of the first
+  // device's context), so that a benchmark can time the kernel through this
+  // surface. A record is (begin ms, end ms, elements, contributions, reduce
+  // stream, launches).
+  void profileMark();
+  std::vector<std::tuple<double, double, int64_t, int, int, int>> launchRecords();
+  void synchronizeAll();
+
  private:
   frg_ctx* contextFor(c10::DeviceIndex device);
   void requireGroupOfOne(const char* what) const;
@@ -160,9 +169,11 @@ class ProcessGroupFairring : public c10d::Backend {
   c10::intrusive_ptr<OptionsFairring> options_;
   std::mutex mutex_;
   std::map<c10::DeviceIndex, frg_ctx*> contexts_;  // built lazily (process_group.cc:140-152)
-  // The pipeline's streams per device as c10 streams, reduce streams first
-  // (numReduceStreams_ of them), then the copy streams.
+  // The pipeline's reduce streams per device as c10 streams, and its copy
+  // streams, which exist from the first host-staged operation on.
   std::map<c10::DeviceIndex, std::vector<c10::Stream>> streams_;
+  std::map<c10::DeviceIndex, std::vector<c10::Stream>> copyStreams_;
+  const std::vector<c10::Stream>& copyStreamsFor(c10::DeviceIndex device, frg_ctx* ctx);
   static constexpr int kNumReduceStreams = 2;
   static constexpr int kNumCopyStreams = 2;
   void recordOnPipelineStreams(c10::DeviceIndex device, bool copyStreamsToo,

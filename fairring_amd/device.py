@@ -199,6 +199,34 @@ class DeviceFairring:
         _capi.check(_capi.lib().frg_create(int(device), ctypes.byref(o), ctypes.byref(h)))
         self._h = h
         self.device = int(device)
+        self._reduce_streams = None
+        self._copy_streams = None
+
+    def _external_streams(self, getter):
+        import torch
+        raw = (ctypes.c_void_p * 16)()
+        n = ctypes.c_int()
+        _capi.check(getter(self._h, raw, 16, ctypes.byref(n)))
+        return [torch.cuda.ExternalStream(raw[i], device=self.device)
+                for i in range(min(n.value, 16))]
+
+    def _record_on_streams(self, tensors, host=False):
+        """Tells torch's caching allocator which of the pipeline's streams touch
+        these tensors (the reference does so on its five streams,
+        fairring/device.cc:297-301): memory freed while an operation is still
+        running is then not handed out again before that stream has passed it.
+        The copy streams write `out` when contributions are staged from the host."""
+        if self._reduce_streams is None:
+                self._reduce_streams = self._external_streams(_capi.lib().frg_get_streams)
+        streams = self._reduce_streams
+        if host:
+            if self._copy_streams is None:
+                self._copy_streams = self._external_streams(_capi.lib().frg_get_copy_streams)
+            streams = streams + self._copy_streams
+        for s in streams:
+            for t in tensors:
+                if t.is_cuda:
+                    t.record_stream(s)
 
     @property
     def layout(self):
@@ -221,6 +249,7 @@ class DeviceFairring:
         head = (self._h, out.data_ptr(), tab, len(contribs), out.numel(), _dtype_code(out), op,
                 scale_mode, scale)
         tail = (stream.cuda_stream, _capi.DONE_FN(), None, ctypes.byref(wh))
+        self._record_on_streams([out] if host else [out] + list(contribs), host=host)
         if host:
             _capi.check(L.frg_allreduce_host(*head, 1 if carry else 0, *tail))
         else:
@@ -248,6 +277,7 @@ class DeviceFairring:
         stream = torch.cuda.current_stream(out.device) if stream is None else stream
         tab = _capi.ptr_table([c.data_ptr() for c in contribs])
         wh = ctypes.c_void_p()
+        self._record_on_streams([out] + list(contribs))
         _capi.check(_capi.lib().frg_allreduce_compressed(
             self._h, out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index,
             out.numel(), wire, scale_mode, scale, stream.cuda_stream, _capi.DONE_FN(), None,
@@ -270,7 +300,8 @@ class DeviceFairring:
         """Validate and marshal an allreduce once; the returned callable submits
         it with a single foreign call (for callers that repeat the same
         operation, e.g. one per DDP bucket per step). The callable returns a
-        Work; the tensors stay referenced by it."""
+        Work; the tensors stay referenced by the callable and are recorded on
+        the pipeline's streams once, here."""
         import torch
         _check_dense(out, "output")
         for c in contribs:
@@ -285,6 +316,7 @@ class DeviceFairring:
                 ctypes.c_int64(out.numel()), _dtype_code(out), op, scale_mode,
                 ctypes.c_float(scale), ctypes.c_void_p(stream.cuda_stream), _capi.DONE_FN(), None)
         keep = (out, list(contribs), tab)
+        self._record_on_streams([out] + list(contribs))
 
         def submit():
             wh = ctypes.c_void_p()

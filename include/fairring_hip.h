@@ -152,7 +152,8 @@ typedef struct frg_options {
   int64_t slice_size_in_bytes;            /* FAIRRING_SLICE_SIZE; 0 = derive with computeLayout */
   int64_t num_machines;                   /* M used by computeLayout (simulated peers), >= 1 */
   int32_t num_reduce_streams;             /* 0 = default (2) */
-  int32_t num_copy_streams;               /* host-staged path; 0 = default (2), at most 4 */
+  int32_t num_copy_streams;               /* host-staged path; 0 = default (2), at most 4;
+                                             created on first use */
   int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
                                              launch covers: device-resident tensors are cut into
                                              launches of this size on 4 KiB boundaries (the last
@@ -180,9 +181,19 @@ FRG_API int frg_destroy(frg_ctx* ctx);
 FRG_API int frg_get_layout(frg_ctx* ctx, frg_layout* out);
 
 /* The streams the pipeline launches on (reduce streams first, then the copy
- * streams), for callers that must tell an allocator which streams touch a buffer
- * (the reference calls record_stream on its five streams, device.cc:297-301). */
+ * streams that exist so far), for callers that must tell an allocator which
+ * streams touch a buffer (the reference calls record_stream on its five
+ * streams, device.cc:297-301). */
 FRG_API int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* count);
+
+/* The copy streams of the host-staged path (the role of the reference's
+ * collectStream_, device.cc:239-243,547-566: where contributions arrive in the
+ * staging slots). They are created by the first call of this function or by the
+ * first frg_allreduce_host, whichever comes first, so that a context that only
+ * reduces device-resident tensors holds its reduce streams and nothing else. A
+ * caller that records buffers on the pipeline's streams calls this before it
+ * submits a host-staged operation (they write `out`). */
+FRG_API int frg_get_copy_streams(frg_ctx* ctx, void** streams, int capacity, int* count);
 
 /* Called on the command thread once the last slice of an operation has been
  * enqueued (status FRG_OK) or enqueueing failed; `last_stream` is the stream
@@ -196,8 +207,16 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
  * elements each. The slices of the layout only count here (they advance the
  * slot cursor): resident contributions need no slot, so the tensor is reduced
  * by launches of frg_options.max_launch_bytes per contribution, cut on 4 KiB
- * boundaries from its start and rotating over the reduce streams, whatever
- * the slice size (max_launch_bytes < 0: one launch per slice). More than 64 contributions are folded by a chain of
+ * boundaries from its start, whatever the slice size (max_launch_bytes < 0:
+ * one launch per slice). An operation of up to 8 launches (a DDP bucket) runs
+ * on one reduce stream and the next operation on the next one; a longer one
+ * deals its launches over all reduce streams. Operations are ordered as on one
+ * stream wherever that can be observed: one that writes memory an earlier
+ * operation of this context reads or writes, or reads what that one writes,
+ * runs after it (the streams involved are joined with an event); operations on
+ * disjoint buffers, such as the buckets of a gradient, overlap. Waiting for an
+ * operation therefore covers every earlier one it shares memory with, not the
+ * others. More than 64 contributions are folded by a chain of
  * launches per range; the result is that of one fold over all of them, with
  * one rounding (bf16 / fp16 partial sums travel as fp32), also when `out` is
  * one of the contributions. `producer_stream` is the stream the caller's

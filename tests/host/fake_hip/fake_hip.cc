@@ -13,6 +13,8 @@
 #include <mutex>
 #include <string>
 #include <thread>
+#include <utility>
+#include <vector>
 
 namespace {
 
@@ -51,37 +53,19 @@ hipError_t ret(hipError_t e) {
 
 }  // namespace
 
-struct FakeStream {
+// A hardware queue: packets of every stream mapped onto it run strictly in the
+// order they were written, one at a time, so a wait packet holds up everything
+// behind it whatever stream that belongs to (the barrier bit of an in-order AQL
+// queue). With fake_hip_set_hw_queues(0) every stream has a queue of its own.
+struct HwQueue {
   std::mutex mu;
   std::condition_variable cv;
-  std::deque<std::function<void()>> tasks;
-  long submitted = 0;
-  long finished = 0;
+  std::deque<std::pair<FakeStream*, std::function<void()>>> packets;
   bool stop = false;
   std::thread worker;
 
-  FakeStream() {
-    worker = std::thread([this] {
-      while (true) {
-        std::function<void()> fn;
-        {
-          std::unique_lock<std::mutex> lock(mu);
-          cv.wait(lock, [&] { return stop || !tasks.empty(); });
-          if (tasks.empty()) return;
-          fn = std::move(tasks.front());
-          tasks.pop_front();
-        }
-        fn();
-        {
-          std::lock_guard<std::mutex> g(mu);
-          ++finished;
-        }
-        cv.notify_all();
-      }
-    });
-  }
-
-  ~FakeStream() {
+  HwQueue();
+  ~HwQueue() {
     {
       std::lock_guard<std::mutex> g(mu);
       stop = true;
@@ -89,14 +73,41 @@ struct FakeStream {
     cv.notify_all();
     worker.join();
   }
+};
+
+struct FakeStream {
+  std::mutex mu;
+  std::condition_variable cv;
+  long submitted = 0;
+  long finished = 0;
+  bool blocking = false;  // takes part in the null stream's implicit synchronisation
+  HwQueue* queue = nullptr;
+  bool ownsQueue = false;
+
+  FakeStream(HwQueue* shared, bool blockingStream) : blocking(blockingStream) {
+    if (shared != nullptr) {
+      queue = shared;
+    } else {
+      queue = new HwQueue();
+      ownsQueue = true;
+    }
+  }
+
+  ~FakeStream() {
+    drain();
+    if (ownsQueue) delete queue;
+  }
 
   void push(std::function<void()> fn) {
     {
       std::lock_guard<std::mutex> g(mu);
-      tasks.push_back(std::move(fn));
       ++submitted;
     }
-    cv.notify_all();
+    {
+      std::lock_guard<std::mutex> g(queue->mu);
+      queue->packets.emplace_back(this, std::move(fn));
+    }
+    queue->cv.notify_all();
   }
 
   void drain() {
@@ -111,6 +122,27 @@ struct FakeStream {
   }
 };
 
+HwQueue::HwQueue() {
+  worker = std::thread([this] {
+    while (true) {
+      std::pair<FakeStream*, std::function<void()>> p;
+      {
+        std::unique_lock<std::mutex> lock(mu);
+        cv.wait(lock, [&] { return stop || !packets.empty(); });
+        if (packets.empty()) return;
+        p = std::move(packets.front());
+        packets.pop_front();
+      }
+      p.second();
+      {
+        std::lock_guard<std::mutex> g(p.first->mu);
+        ++p.first->finished;
+      }
+      p.first->cv.notify_all();
+    }
+  });
+}
+
 struct FakeEvent {
   std::mutex mu;
   std::shared_ptr<Record> current;  // the latest record, if any
@@ -118,17 +150,80 @@ struct FakeEvent {
 
 namespace {
 
+std::mutex gTopologyMu;
+std::vector<HwQueue*> gSharedQueues;  // empty: a queue per stream
+size_t gNextQueue = 0;
+FakeStream* gDefaultStream = nullptr;
+std::vector<FakeStream*> gBlockingStreams;  // live streams created without hipStreamNonBlocking
+
+HwQueue* pickQueueLocked() {
+  if (gSharedQueues.empty()) return nullptr;
+  return gSharedQueues[gNextQueue++ % gSharedQueues.size()];
+}
+
 FakeStream* defaultStream() {
-  static FakeStream* s = new FakeStream();  // lives for the process, like the null stream
-  return s;
+  std::lock_guard<std::mutex> g(gTopologyMu);
+  if (gDefaultStream == nullptr) {
+    // lives until the topology is changed, like the null stream
+    gDefaultStream = new FakeStream(pickQueueLocked(), /*blockingStream=*/true);
+  }
+  return gDefaultStream;
 }
 
 FakeStream* resolve(hipStream_t s) { return s ? s : defaultStream(); }
 
+std::shared_ptr<Record> recordOn(FakeStream* s) {
+  auto r = std::make_shared<Record>();
+  s->push([r] {
+    {
+      std::lock_guard<std::mutex> g(r->mu);
+      r->done = true;
+      r->when = Clock::now();
+    }
+    r->cv.notify_all();
+  });
+  return r;
+}
+
+void waitOn(FakeStream* s, std::shared_ptr<Record> r) {
+  s->push([r] {
+    std::unique_lock<std::mutex> lock(r->mu);
+    r->cv.wait(lock, [&] { return r->done; });
+  });
+}
+
+// The legacy null stream: work submitted to it starts after everything
+// submitted so far to the blocking streams, and work submitted to a blocking
+// stream starts after everything submitted so far to the null stream. Streams
+// created with hipStreamNonBlocking stay out of it.
+void implicitSync(FakeStream* target) {
+  std::vector<FakeStream*> others;
+  FakeStream* null = nullptr;
+  {
+    std::lock_guard<std::mutex> g(gTopologyMu);
+    null = gDefaultStream;
+    if (target == null) {
+      others = gBlockingStreams;
+    } else if (target->blocking && null != nullptr) {
+      others.push_back(null);
+    }
+  }
+  for (FakeStream* o : others) {
+    if (o != target && !o->idle()) waitOn(target, recordOn(o));
+  }
+}
+
+// Every submission of real work goes through here.
+void submit(hipStream_t stream, std::function<void()> fn) {
+  FakeStream* s = resolve(stream);
+  implicitSync(s);
+  s->push(std::move(fn));
+}
+
 }  // namespace
 
 void fake_hip_enqueue(hipStream_t stream, void (*fn)(void*), void* arg) {
-  resolve(stream)->push([fn, arg] { fn(arg); });
+  submit(stream, [fn, arg] { fn(arg); });
 }
 
 extern "C" {
@@ -179,9 +274,28 @@ const char* hipGetErrorString(hipError_t e) {
   }
 }
 
-hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int) {
+hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags) {
   if (enter("hipStreamCreateWithFlags")) return ret(hipErrorUnknown);
-  *stream = new FakeStream();
+  const bool blocking = (flags & hipStreamNonBlocking) == 0;
+  std::lock_guard<std::mutex> g(gTopologyMu);
+  *stream = new FakeStream(pickQueueLocked(), blocking);
+  if (blocking) gBlockingStreams.push_back(*stream);
+  return hipSuccess;
+}
+
+hipError_t hipStreamDestroy(hipStream_t stream) {
+  enter("hipStreamDestroy");
+  if (stream == nullptr) return ret(hipErrorInvalidValue);
+  {
+    std::lock_guard<std::mutex> g(gTopologyMu);
+    for (size_t i = 0; i < gBlockingStreams.size(); ++i) {
+      if (gBlockingStreams[i] == stream) {
+        gBlockingStreams.erase(gBlockingStreams.begin() + static_cast<long>(i));
+        break;
+      }
+    }
+  }
+  delete stream;  // drains it first
   return hipSuccess;
 }
 
@@ -199,10 +313,9 @@ hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int
     r = event->current;  // snapshot: later records of the event do not matter
   }
   if (!r) return hipSuccess;
-  resolve(stream)->push([r] {
-    std::unique_lock<std::mutex> lock(r->mu);
-    r->cv.wait(lock, [&] { return r->done; });
-  });
+  FakeStream* s = resolve(stream);
+  implicitSync(s);
+  waitOn(s, r);
   return hipSuccess;
 }
 
@@ -222,19 +335,12 @@ hipError_t hipEventDestroy(hipEvent_t event) {
 
 hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream) {
   if (enter("hipEventRecord")) return ret(hipErrorUnknown);
-  auto r = std::make_shared<Record>();
-  {
-    std::lock_guard<std::mutex> g(event->mu);
-    event->current = r;
-  }
-  resolve(stream)->push([r] {
-    {
-      std::lock_guard<std::mutex> g(r->mu);
-      r->done = true;
-      r->when = Clock::now();
-    }
-    r->cv.notify_all();
-  });
+  FakeStream* s = resolve(stream);
+  implicitSync(s);
+  // the packet is written and the event updated as one step, as the runtime
+  // does under the event's lock
+  std::lock_guard<std::mutex> g(event->mu);
+  event->current = recordOn(s);
   return hipSuccess;
 }
 
@@ -320,12 +426,27 @@ hipError_t hipFree(void* ptr) {
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind,
                           hipStream_t stream) {
   if (enter("hipMemcpyAsync")) return ret(hipErrorUnknown);
-  resolve(stream)->push([dst, src, bytes] { std::memcpy(dst, src, bytes); });
+  submit(stream, [dst, src, bytes] { std::memcpy(dst, src, bytes); });
   return hipSuccess;
 }
 
 void fake_hip_occupy(hipStream_t stream, int ms) {
-  resolve(stream)->push([ms] { std::this_thread::sleep_for(std::chrono::milliseconds(ms)); });
+  submit(stream, [ms] { std::this_thread::sleep_for(std::chrono::milliseconds(ms)); });
+}
+
+void fake_hip_set_hw_queues(int n) {
+  FakeStream* old = nullptr;
+  {
+    std::lock_guard<std::mutex> g(gTopologyMu);
+    old = gDefaultStream;
+    gDefaultStream = nullptr;
+  }
+  if (old != nullptr) old->drain();  // left alive: an event may still point into it
+  std::lock_guard<std::mutex> g(gTopologyMu);
+  // queues of an earlier topology stay: streams created then still run on them
+  gSharedQueues.clear();
+  gNextQueue = 0;
+  for (int i = 0; i < n; ++i) gSharedQueues.push_back(new HwQueue());
 }
 
 void fake_hip_fail_call(const char* api, int nth) {

@@ -3,9 +3,15 @@
 // paths) can run on a machine without a GPU and under ThreadSanitizer.
 // Test infrastructure only: the shipped library is never built against it.
 //
-// Semantics kept: a stream is an in-order queue drained by its own thread; an
-// event record is a point in its stream; a stream wait snapshots the event's
-// record at the time of the call; "device memory" is host memory.
+// Semantics kept: a stream is an in-order queue; an event record is a point in
+// its stream; a stream wait snapshots the event's record at the time of the
+// call; "device memory" is host memory. By default every stream is drained by a
+// thread of its own. fake_hip_set_hw_queues(n) instead maps the streams created
+// afterwards (the null stream included) round-robin onto n hardware queues, each
+// an in-order queue shared by its streams: a wait packet holds up every stream
+// behind it in that queue, as on a GPU whose process has fewer hardware queues
+// than streams. The null stream synchronises implicitly with streams created
+// without hipStreamNonBlocking, as the legacy default stream does.
 #pragma once
 
 #include <stddef.h>
@@ -47,6 +53,7 @@ hipError_t hipGetLastError(void);
 const char* hipGetErrorString(hipError_t e);
 
 hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags);
+hipError_t hipStreamDestroy(hipStream_t stream);
 hipError_t hipStreamSynchronize(hipStream_t stream);
 hipError_t hipStreamQuery(hipStream_t stream);
 typedef enum hipStreamCaptureStatus {
@@ -73,6 +80,9 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKin
 // ---- hooks for tests ------------------------------------------------------
 // Occupies `stream` (nullptr = the default stream) for `ms` milliseconds.
 void fake_hip_occupy(hipStream_t stream, int ms);
+// Streams created from now on share `n` in-order hardware queues (0: a queue
+// per stream, the default). Call it while no work is in flight.
+void fake_hip_set_hw_queues(int n);
 // Makes hipStreamIsCapturing report a capture in progress on every stream (1) or none (0).
 void fake_hip_set_capturing(int on);
 // Makes the `nth` next call (1 = the very next) of the named API fail once.

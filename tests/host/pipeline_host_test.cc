@@ -8,7 +8,9 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <chrono>
 #include <cstring>
+#include <mutex>
 #include <random>
 #include <string>
 #include <thread>
@@ -385,6 +387,234 @@ void scenarioHostStaged() {
   }
 }
 
+bool gSharedHwQueues = false;
+
+// Streams of a context as the ABI hands them out (reduce streams first).
+std::vector<hipStream_t> streamsOf(frg_ctx* ctx) {
+  void* raw[16];
+  int n = 0;
+  CHECK(frg_get_streams(ctx, raw, 16, &n) == FRG_OK);
+  std::vector<hipStream_t> v;
+  for (int i = 0; i < n && i < 16; ++i) v.push_back(static_cast<hipStream_t>(raw[i]));
+  return v;
+}
+
+void scenarioOrderBetweenOperations() {
+  std::puts("operations that share memory keep their order across the reduce streams");
+  // bucket-sized operations alternate between the two reduce streams; the first
+  // stream is held up, so whatever is not ordered after it runs too early
+  const int64_t n = 3000;
+  for (int round = 0; round < 3; ++round) {
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    CHECK(streamsOf(ctx).size() == 2);  // no copy streams until something is staged
+    hipStream_t s0 = streamsOf(ctx)[0];
+    auto c = randomContribs(4, n, 40 + round);
+    auto t = table(c);
+    Vec own = c[0];
+    std::vector<const void*> tab = t;
+    tab[0] = own.data();
+    frg_work* w[3] = {nullptr, nullptr, nullptr};
+    fake_hip_occupy(s0, 60);
+    if (round == 0) {
+      // three in-place reductions of the same tensor, none waited for (a scale
+      // of its own each, so that their order shows in the result)
+      Vec want = own;
+      const float scales[3] = {0.5f, 0.25f, 2.0f};
+      for (int i = 0; i < 3; ++i) {
+        std::vector<Vec> terms = {want, c[1], c[2], c[3]};
+        want = fold(terms, FRG_SCALE_MUL, scales[i]);
+        CHECK(frg_allreduce(ctx, own.data(), tab.data(), 4, n, FRG_F32, FRG_SUM, FRG_SCALE_MUL,
+                            scales[i], nullptr, nullptr, nullptr, &w[i]) == FRG_OK);
+      }
+      CHECK(frg_work_wait(w[2]) == FRG_OK);  // the last one covers the others
+      CHECK(same(own, want));
+    } else if (round == 1) {
+      // the output of one operation is a contribution of the next (a
+      // reduce-scatter's output fed to an allreduce)
+      Vec mid(n, -1.f), out(n, -1.f);
+      CHECK(frg_allreduce(ctx, mid.data(), t.data(), 4, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                          nullptr, nullptr, nullptr, &w[0]) == FRG_OK);
+      const void* second[2] = {mid.data(), c[1].data()};
+      CHECK(frg_allreduce(ctx, out.data(), second, 2, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                          nullptr, nullptr, nullptr, &w[1]) == FRG_OK);
+      CHECK(frg_work_wait(w[1]) == FRG_OK);
+      std::vector<Vec> terms = {fold(c, FRG_SCALE_NONE, 1.f), c[1]};
+      CHECK(same(out, fold(terms, FRG_SCALE_NONE, 1.f)));
+    } else {
+      // write after read: the second operation overwrites a contribution of the first
+      Vec out(n, -1.f);
+      const Vec want = fold(c, FRG_SCALE_NONE, 1.f);
+      CHECK(frg_allreduce(ctx, out.data(), t.data(), 4, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                          nullptr, nullptr, nullptr, &w[0]) == FRG_OK);
+      const void* second[2] = {c[1].data(), c[2].data()};
+      CHECK(frg_allreduce(ctx, c[3].data(), second, 2, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                          nullptr, nullptr, nullptr, &w[1]) == FRG_OK);
+      CHECK(frg_work_wait(w[0]) == FRG_OK);
+      CHECK(frg_work_wait(w[1]) == FRG_OK);
+      CHECK(same(out, want));
+    }
+    for (frg_work* x : w) {
+      if (x) frg_work_release(x);
+    }
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+  // independent buckets are not ordered against each other: with the first
+  // stream held up, the bucket on the second stream finishes first
+  {
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    hipStream_t s0 = streamsOf(ctx)[0];
+    auto a = randomContribs(3, n, 50), b = randomContribs(3, n, 51);
+    Vec outA(n), outB(n);
+    auto ta = table(a), tb = table(b);
+    frg_work *wa = nullptr, *wb = nullptr;
+    fake_hip_occupy(s0, 300);
+    CHECK(frg_allreduce(ctx, outA.data(), ta.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                        nullptr, nullptr, nullptr, &wa) == FRG_OK);
+    CHECK(frg_allreduce(ctx, outB.data(), tb.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                        nullptr, nullptr, nullptr, &wb) == FRG_OK);
+    CHECK(frg_work_wait(wb) == FRG_OK);
+    CHECK(same(outB, fold(b, FRG_SCALE_NONE, 1.f)));
+    // the first stream is still held up (streams that share a hardware queue
+    // cannot overtake each other, so this only holds with a queue per stream)
+    if (!gSharedHwQueues) CHECK(hipStreamQuery(s0) == hipErrorNotReady);
+    CHECK(frg_work_wait(wa) == FRG_OK);
+    CHECK(same(outA, fold(a, FRG_SCALE_NONE, 1.f)));
+    frg_work_release(wa);
+    frg_work_release(wb);
+    // many independent buckets: the bookkeeping stays bounded (a forced join now and then)
+    std::vector<Vec> outs(200, Vec(256));
+    auto small = randomContribs(2, 256, 52);
+    auto ts = table(small);
+    for (auto& o : outs) {
+      CHECK(frg_allreduce(ctx, o.data(), ts.data(), 2, 256, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                          nullptr, nullptr, nullptr, nullptr) == FRG_OK);
+    }
+    CHECK(frg_synchronize(ctx) == FRG_OK);
+    for (auto& o : outs) CHECK(same(o, fold(small, FRG_SCALE_NONE, 1.f)));
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+  // a resident operation followed by a host-staged one into the same tensor, and back
+  {
+    frg_ctx* ctx = makeCtx(2 * 4096, 4096, 2, 0);
+    auto c = randomContribs(3, n, 53);
+    auto t = table(c);
+    Vec out(n, -1.f);
+    hipStream_t s1 = streamsOf(ctx)[1];
+    CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 16, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                        nullptr, nullptr, nullptr, nullptr) == FRG_OK);  // takes stream 0
+    fake_hip_occupy(s1, 60);
+    CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                        nullptr, nullptr, nullptr, nullptr) == FRG_OK);  // stream 1, held up
+    // `out` now is the first term; the staged copies must not overtake the operation before
+    CHECK(frg_allreduce_host(ctx, out.data(), t.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                             1.f, /*carry=*/1, nullptr, nullptr, nullptr, nullptr) == FRG_OK);
+    frg_work* w = nullptr;
+    const void* again[2] = {out.data(), c[0].data()};
+    Vec out2(n, -1.f);
+    CHECK(frg_allreduce(ctx, out2.data(), again, 2, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                        nullptr, nullptr, nullptr, &w) == FRG_OK);
+    CHECK(frg_work_wait(w) == FRG_OK);
+    CHECK(streamsOf(ctx).size() == 4);  // the copy streams exist once something was staged
+    const Vec first = fold(c, FRG_SCALE_NONE, 1.f);
+    const Vec staged = fold(c, FRG_SCALE_NONE, 1.f, &first);
+    CHECK(same(out, staged));
+    std::vector<Vec> terms = {staged, c[0]};
+    CHECK(same(out2, fold(terms, FRG_SCALE_NONE, 1.f)));
+    frg_work_release(w);
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
+// What the c10d extension does around the ABI, with a mutex standing in for
+// Python's global lock: the caller holds it except inside the calls that let go
+// of it (submitting, waiting); the completion callback, on the command thread,
+// takes it briefly (it drops tensor references). 15 peers in host memory staged
+// through 2 slots, the rank's own term already in `out`, several operations,
+// each waited for through its callback alone.
+std::mutex gInterpreterLock;
+
+struct GroupPending {
+  std::atomic<int> done{0};
+  std::atomic<void*> stream{nullptr};
+};
+
+void onGroupDone(void* user, int status, void* lastStream) {
+  auto* p = static_cast<GroupPending*>(user);
+  CHECK(status == FRG_OK);
+  {
+    std::lock_guard<std::mutex> g(gInterpreterLock);  // "drop the tensor references"
+    p->stream = lastStream;
+  }
+  p->done = 1;
+}
+
+void scenarioProcessGroupShaped() {
+  std::puts("process-group-shaped: staged peers, callback that takes the interpreter lock");
+  frg_ctx* ctx = makeCtx(2 * 4096, 4096, 2, 0);
+  hipStream_t callerStream;
+  CHECK(hipStreamCreateWithFlags(&callerStream, hipStreamNonBlocking) == hipSuccess);
+  std::unique_lock<std::mutex> gil(gInterpreterLock);
+  const int ops = 8;
+  for (int i = 0; i < ops; ++i) {
+    const int64_t n = 2500 + 13 * i;
+    auto all = randomContribs(16, n, 400 + i);
+    Vec out = all[0];
+    std::vector<Vec> rest(all.begin() + 1, all.end());
+    auto tr = table(rest);
+    GroupPending pending;
+    fake_hip_occupy(i % 2 ? callerStream : nullptr, 2);  // the producer is still busy
+    gil.unlock();  // the binding lets go of the lock around the call
+    CHECK(frg_allreduce_host(ctx, out.data(), tr.data(), 15, n, FRG_F32, FRG_SUM, FRG_SCALE_MUL,
+                             1.f / 16, /*carry=*/1, i % 2 ? callerStream : nullptr, &onGroupDone,
+                             &pending, nullptr) == FRG_OK);
+    gil.lock();
+    gil.unlock();  // Work.wait lets go of it as well
+    while (pending.done.load() == 0) std::this_thread::yield();
+    gil.lock();
+    CHECK(hipStreamSynchronize(static_cast<hipStream_t>(pending.stream.load())) == hipSuccess);
+    CHECK(same(out, fold(all, FRG_SCALE_MUL, 1.f / 16)));
+  }
+  gil.unlock();
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
+void scenarioBlockStreamGivesUp() {
+  std::puts("blocking a stream on an operation gives up like a wait does");
+  frg_ctx* ctx = makeCtx(16384, 4096, 2, 1024);
+  auto c = randomContribs(4, 5000, 78);
+  Vec out(5000);
+  auto t = table(c);
+  // hold the command thread up: it queries and waits on the producer's event,
+  // then launches, only after a stalled operation ahead of it is through
+  hipStream_t consumer;
+  CHECK(hipStreamCreateWithFlags(&consumer, hipStreamNonBlocking) == hipSuccess);
+  CHECK(frg_set_wait_timeout(0.2) == FRG_OK);
+  std::atomic<int> release{0};
+  struct Held {
+    std::atomic<int>* release;
+  } held{&release};
+  // an operation whose completion callback blocks the command thread for a while
+  auto blocker = [](void* user, int, void*) {
+    auto* h = static_cast<Held*>(user);
+    while (h->release->load() == 0) std::this_thread::sleep_for(std::chrono::milliseconds(1));
+  };
+  Vec out0(5000);
+  CHECK(frg_allreduce(ctx, out0.data(), t.data(), 4, 5000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, blocker, &held, nullptr) == FRG_OK);
+  frg_work* w = nullptr;
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 4, 5000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_block_stream(w, consumer) == FRG_ERR_NOT_READY);
+  CHECK(std::strstr(frg_last_error(), "gave up after") != nullptr);
+  release = 1;
+  CHECK(frg_set_wait_timeout(0) == FRG_OK);
+  CHECK(frg_work_block_stream(w, consumer) == FRG_OK);
+  CHECK(hipStreamSynchronize(consumer) == hipSuccess);
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  frg_work_release(w);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
 struct CallbackState {
   std::atomic<int> calls{0};
   std::atomic<int> status{-1};
@@ -577,21 +807,73 @@ void scenarioConcurrentSubmitters() {
   CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
+// Ends the process when a scenario stops making progress, with its name, so
+// that a cycle of waits shows as a failure rather than as a run that never ends.
+std::atomic<long> gScenarioTicks{0};
+const char* volatile gScenarioName = "start-up";
+
+void watchdog() {
+  long seen = -1;
+  int stale = 0;
+  for (;;) {
+    std::this_thread::sleep_for(std::chrono::seconds(1));
+    const long now = gScenarioTicks.load();
+    stale = now == seen ? stale + 1 : 0;
+    seen = now;
+    if (stale > 150) {
+      std::fprintf(stderr, "no progress for 150 s in scenario: %s\n", gScenarioName);
+      std::abort();
+    }
+  }
+}
+
+void runAll() {
+  struct Scenario {
+    const char* name;
+    void (*fn)();
+  };
+  const Scenario all[] = {
+      {"resident", scenarioResident},
+      {"launch partition", scenarioLaunchPartition},
+      {"pre-scale and compressed", scenarioPreScaleAndCompressed},
+      {"busy producer", scenarioBusyProducer},
+      {"wait gives up", scenarioWaitGivesUp},
+      {"block stream gives up", scenarioBlockStreamGivesUp},
+      {"producer ordering", scenarioProducerOrdering},
+      {"order between operations", scenarioOrderBetweenOperations},
+      {"host staged", scenarioHostStaged},
+      {"callback", scenarioCallback},
+      {"process-group-shaped", scenarioProcessGroupShaped},
+      {"errors", scenarioErrors},
+      {"profiling", scenarioProfiling},
+      {"destroy with pending work", scenarioDestroyWithPendingWork},
+      {"concurrent submitters", scenarioConcurrentSubmitters},
+  };
+  for (const Scenario& sc : all) {
+    gScenarioName = sc.name;
+    gScenarioTicks++;
+    sc.fn();
+    gScenarioTicks++;
+  }
+}
+
 }  // namespace
 
 int main() {
-  scenarioResident();
-  scenarioLaunchPartition();
-  scenarioPreScaleAndCompressed();
-  scenarioBusyProducer();
-  scenarioWaitGivesUp();
-  scenarioProducerOrdering();
-  scenarioHostStaged();
-  scenarioCallback();
-  scenarioErrors();
-  scenarioProfiling();
-  scenarioDestroyWithPendingWork();
-  scenarioConcurrentSubmitters();
+  std::thread(watchdog).detach();
+  std::puts("== every stream on a queue of its own");
+  runAll();
+  // The shape of a GPU process with fewer hardware queues than streams: the
+  // null stream, the reduce and copy streams of every context and the callers'
+  // side streams multiplexed onto 4 in-order queues, where a wait packet holds
+  // up whatever sits behind it.
+  std::puts("== all streams on 4 shared in-order hardware queues");
+  fake_hip_set_hw_queues(4);
+  gSharedHwQueues = true;
+  runAll();
+  fake_hip_set_hw_queues(1);
+  std::puts("== all streams on 1 shared in-order hardware queue");
+  runAll();
   std::puts("ALL HOST SCENARIOS PASSED");
   return 0;
 }

@@ -470,6 +470,53 @@ def test_pipeline_many_small_operations_in_order():
     dev.close()
 
 
+def test_operations_sharing_a_tensor_keep_their_order_across_streams():
+    # Bucket-sized operations alternate between the reduce streams. Operations that share a
+    # tensor must still run in submission order: six in-place reductions of one 20 M-element
+    # tensor (80 MiB, several launches each, long enough to overlap if nothing orders them),
+    # each with a scale of its own so that the order shows in the bits; then the output of one
+    # operation as a contribution of the next, and an operation that overwrites a contribution
+    # of the one before. None is waited for until the end.
+    _print_case("order between operations")
+    k, n = 4, 20_000_003
+    g = torch.Generator(device=DEV)
+    g.manual_seed(61)
+    xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    own = xs[0].clone()
+    dev = fa.DeviceFairring(0)
+    torch.cuda.synchronize()
+    scales = [0.5, 0.25, 2.0, 1.0, 4.0, 0.125]
+    works = [dev.allreduce(own, [own] + xs[1:], scale_mode=fa.SCALE_MUL, scale=s) for s in scales]
+    works[-1].wait()            # covers the earlier ones: they share its tensor
+    want = xs[0].clone()
+    for s in scales:
+        for x in xs[1:]:
+            want.add_(x)
+        want.mul_(s)
+    assert bool(torch.equal(own.view(torch.int32), want.view(torch.int32)))
+    lo, hi = n - 70_001, n
+    acc = xs[0][lo:hi].cpu().numpy()
+    host = [x[lo:hi].cpu().numpy() for x in xs[1:]]
+    for s in scales:
+        acc = oracle.sum_f32([acc] + host, oracle.SCALE_MUL, s)
+    assert_bits_equal(own[lo:hi].cpu().numpy(), acc)
+    # read after write, then write after read
+    mid = torch.zeros(n, device=DEV)
+    out = torch.zeros(n, device=DEV)
+    spare = xs[3].clone()
+    w1 = dev.allreduce(mid, xs)                       # mid = x0 + x1 + x2 + x3
+    w2 = dev.allreduce(out, [mid, spare])             # reads mid
+    w3 = dev.allreduce(spare, [xs[1], xs[2]])         # overwrites what w2 reads
+    for w in (w1, w2, w3):
+        w.wait()
+    want_mid = xs[0] + xs[1]
+    want_mid.add_(xs[2]).add_(xs[3])
+    assert bool(torch.equal(mid.view(torch.int32), want_mid.view(torch.int32)))
+    assert bool(torch.equal(out.view(torch.int32), (want_mid + xs[3]).view(torch.int32)))
+    assert bool(torch.equal(spare.view(torch.int32), (xs[1] + xs[2]).view(torch.int32)))
+    dev.close()
+
+
 def test_pipeline_empty_tensor_and_layout_errors():
     _print_case("pipeline empty / layout errors")
     dev = fa.DeviceFairring(0)

@@ -194,6 +194,60 @@ def test_max_semantics():
     assert got[4] == 0.0
 
 
+@pytest.mark.parametrize("kind,tdt", [("f32", torch.float32), ("bf16", torch.bfloat16),
+                                      ("f16", torch.float16)])
+def test_max_of_every_floating_type_against_aten_amax(kind, tdt):
+    # the maximum of the 2-byte types, pinned directly against the installed ATen's amax on the
+    # CPU (what the reference calls, fairring/device.cc:127): NaN in any position wins, +-inf,
+    # +-0 (whose sign ATen leaves unspecified), subnormals, K = 1 ... 64
+    rng = np.random.default_rng(19)
+    for k in (1, 2, 3, 8, 17, 64):
+        n = 4000
+        x = (rng.standard_normal((k, n)) * np.exp(rng.uniform(-20, 20, (k, n)))).astype(np.float32)
+        x[:, 0] = np.inf
+        x[:, 1] = -np.inf
+        x[rng.integers(k), 2] = np.inf
+        x[rng.integers(k), 3] = -np.inf
+        x[rng.integers(k), 4] = np.nan                 # one NaN among finite values
+        x[:, 5] = np.nan
+        x[:, 6] = [(-0.0 if r % 2 else 0.0) for r in range(k)]
+        x[:, 7] = -0.0
+        x[:, 8] = np.float32(1e-41) * (np.arange(k) - k // 2)   # fp32 subnormals of both signs
+        x[:, 9] = np.float32(6e-8) * (np.arange(k) + 1)         # fp16 subnormals
+        x[rng.integers(k), 10] = np.nan
+        x[(rng.integers(k) + 1) % k, 10] = np.inf      # NaN beats +inf wherever either stands
+        t = torch.from_numpy(x).to(tdt)
+        want_t = torch.amax(t, dim=0)
+        if kind == "f32":
+            got, want = oracle.reduce(kind, list(x), "max"), want_t.numpy()
+            zero = want == 0
+        else:
+            bits = t.view(torch.int16).numpy().view(np.uint16)
+            got = oracle.reduce(kind, list(bits), "max")
+            want = want_t.view(torch.int16).numpy().view(np.uint16)
+            zero = (want & 0x7FFF) == 0
+        assert zero[6] and zero[7]
+        if kind == "f32":
+            assert (got[zero] == 0).all()
+        else:
+            assert ((got[zero] & 0x7FFF) == 0).all()
+        assert_bits_equal(got[~zero], want[~zero], "%s amax K=%d" % (kind, k), half=kind == "f16")
+    # exhaustively over pairs of special values and a few ordinary ones, both orders
+    specials = np.array([np.nan, np.inf, -np.inf, 0.0, -0.0, 1.0, -1.0, 65504.0, 6e-8, -6e-8,
+                         1e-41, 3.0e38], np.float32)
+    a, b = np.meshgrid(specials, specials)
+    pair = torch.from_numpy(np.stack([a.reshape(-1), b.reshape(-1)])).to(tdt)
+    want_t = torch.amax(pair, dim=0)
+    if kind == "f32":
+        got, want = oracle.reduce(kind, list(pair.numpy()), "max"), want_t.numpy()
+        zero = want == 0
+    else:
+        got = oracle.reduce(kind, list(pair.view(torch.int16).numpy().view(np.uint16)), "max")
+        want = want_t.view(torch.int16).numpy().view(np.uint16)
+        zero = (want & 0x7FFF) == 0
+    assert_bits_equal(got[~zero], want[~zero], kind + " amax of pairs", half=kind == "f16")
+
+
 # ---- the other element types ----------------------------------------------------------
 
 def test_f16_conversions_exhaustive_and_sum_vs_aten():
