@@ -109,15 +109,21 @@ TORCH_PASSES = 150   # timed passes of the CPU baseline (about ten seconds of CP
 ORACLE_PASSES = 30
 
 
-def cpu_baseline(oracle, np, torch, xs, slice_elems, k, n_sample, dtype):
+def cpu_baseline_sample(xs, slice_elems, n_sample):
+    """The first `n_sample` slices of every contribution, copied back from the GPU."""
+    return [[x[i * slice_elems:(i + 1) * slice_elems].cpu() for x in xs]
+            for i in range(n_sample)]
+
+
+def cpu_baseline(oracle, np, torch, host, slice_elems, k, dtype):
     """The contract's reduction on this host's cores: torch's at::add chain
     (acc = x0; acc += xk; acc /= K; bf16: fp32 accumulator, one final cast) over
-    `n_sample` distinct 25 MiB slices copied back from the GPU; 3 warm-up and
+    the distinct 25 MiB slices in `host` (cpu_baseline_sample); 3 warm-up and
     TORCH_PASSES timed passes, median. The repository's C restatement (OpenMP) is timed
     beside it. GB/s uses the same algorithmic-bytes formula as the GPU figure."""
-    host = [[x[i * slice_elems:(i + 1) * slice_elems].cpu() for x in xs]
-            for i in range(n_sample)]
+    n_sample = len(host)
     threads = torch.get_num_threads()
+    xs = host[0]
     acc = torch.empty(slice_elems, dtype=torch.float32)
     res = torch.empty(slice_elems, dtype=xs[0].dtype)
 
@@ -191,31 +197,24 @@ def union_length(intervals):
     return total
 
 
-DEFAULT_LAUNCH_BYTES = 25 * MiB // 2  # the library's default launch target per contribution
 LAUNCH_QUANTUM_BYTES = 4096
 
 
-def default_launch_bytes(k, bytes_per_contrib=0):
-    """The library's default launch size by number of contributions and size of
-    the operation (layout.h::defaultLaunchShape)."""
-    if k <= 2:
-        return 48 * MiB
-    large = bytes_per_contrib >= 100 * MiB
-    if k == 3:
-        return 20 * MiB if large else DEFAULT_LAUNCH_BYTES
-    if k <= 8 and not large:
-        return DEFAULT_LAUNCH_BYTES
-    rounds = max(1, (80 * MiB // (k + 1) + 2 * MiB) // (4 * MiB))
-    return rounds * 4 * MiB
+def launch_elems(args, op_elems, slice_elems, elsize, k=8, compressed_default=0):
+    """Elements of the commonest launch of an operation over `op_elems` elements.
+    With a launch size asked for (or the compressed reduction's default,
+    `compressed_default`), the pipeline cuts the tensor into launches of that size
+    on 4 KiB boundaries from its start, the last one up to one and a half times
+    as long; a negative size means one launch per slice. Otherwise the partition
+    is the library's own (frg_plan_launches: launches of whole rounds of their
+    grid from 4 contributions on)."""
+    lb = args.launch_bytes or compressed_default
+    if lb == 0:
+        import collections
 
-
-def launch_elems(args, op_elems, slice_elems, elsize, k=8):
-    """Elements of the commonest launch of an operation over `op_elems` elements:
-    the pipeline cuts the tensor into launches of the launch target, on 4 KiB
-    boundaries from its start and whatever the slice size; the last launch takes
-    up to one and a half times that. A negative target means one launch per
-    slice."""
-    lb = args.launch_bytes or default_launch_bytes(k, op_elems * elsize)
+        import fairring_amd as fa
+        sizes = collections.Counter(n for n, _ in fa.plan_launches(k, op_elems, elsize))
+        return sizes.most_common(1)[0][0] if sizes else 0
     if lb < 0:
         return min(slice_elems, op_elems)
     max_elems = (lb - lb % 16) // elsize
@@ -360,10 +359,12 @@ def run_resident(args, np, torch, fa, oracle, dtype, keep=None):
         "reduce_streams": args.streams or "default",
         "launch_bytes_per_contribution": args.launch_bytes or "default",
     }
+    # The CPU baseline is timed by the caller, after every GPU measurement of the
+    # run: the GPU idles while the host computes, and drops its clocks.
     base = None
     if not args.no_cpu_baseline and args.workload != "copy":
-        base = cpu_baseline(oracle, np, torch, xs, slice_elems, k,
-                            min(args.cpu_slices, max(1, n_slices - 1)), dtype)
+        sample = cpu_baseline_sample(xs, slice_elems, min(args.cpu_slices, max(1, n_slices - 1)))
+        base = lambda: cpu_baseline(oracle, np, torch, sample, slice_elems, k, dtype)  # noqa: E731
     if keep is not None:
         keep.extend([xs, out])
     return value, elapsed, cfg, roof, checked, base, dtype
@@ -616,9 +617,9 @@ def run_hook(args, np, torch, fa, oracle):
         default_lb = 16 * MiB
     else:
         default_lb = max(1, -(-(2 * 80 * MiB // bytes_per_elem) // (2 * MiB))) * 2 * MiB
-    largs = args if args.launch_bytes else argparse.Namespace(launch_bytes=default_lb)
-    roof = roofline_from_records(recs, bytes_per_elem, launch_elems(largs, numel, slice_elems, 2),
-                                 SPAN_HOW)
+    roof = roofline_from_records(recs, bytes_per_elem,
+                                 launch_elems(args, numel, slice_elems, 2,
+                                              compressed_default=default_lb), SPAN_HOW)
     roof["kernel"] = "compressedKernel<Bf16Vec, out fp32>, K=%d" % k
     # parity on a fresh bucket (the timed steps reduced in place)
     fresh = synth(torch, numel, 1, "f32", 777)[0]
@@ -791,7 +792,7 @@ def main():
         for name in ("c5", "c5pg", "c4", "hook", "c3"):
             sub = argparse.Namespace(**vars(args))
             sub.workload, sub.no_cpu_baseline = name, True
-            sub.steps, sub.warmup = min(args.steps, 3 if name == "c3" else 10), 2
+            sub.steps, sub.warmup = min(args.steps, 3 if name == "c3" else 10), 3
             if name == "c4":
                 shared = None
                 keep.clear()       # the fp32 inputs go before the bf16 ones are made
@@ -808,6 +809,9 @@ def main():
                 extra[name] = {"error": "%s: %s" % (type(e).__name__, e)}
                 failed.append(name)
         result["configs"] = extra
+    del keep[:]
+    if callable(result.get("cpu_baseline")):
+        result["cpu_baseline"] = result["cpu_baseline"]()
     print(json.dumps(result))
     if failed:
         sys.exit("workloads that failed: %s" % ", ".join(failed))

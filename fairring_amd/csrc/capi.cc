@@ -109,6 +109,31 @@ int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes, int64_t element
   return FRG_OK;
 }
 
+int frg_plan_launches(int K, int64_t numel, int64_t element_size,
+                      uint64_t first_contribution_address, uint64_t out_offset_in_allocation,
+                      int align_short_operations, int num_cus, int64_t* launch_elems,
+                      int32_t* blocks_per_cu, int capacity, int* count) {
+  if (K < 1 || numel < 0 || element_size < 1 || frg::kTileBytes % element_size != 0 ||
+      num_cus < 1 || count == nullptr) {
+    return fail(FRG_ERR_INVALID, "bad arguments to frg_plan_launches");
+  }
+  return guarded([&] {
+    const int64_t bytes = numel * element_size;
+    const std::vector<frg::LaunchPart> parts = frg::planDefaultLaunches(
+        K, bytes, out_offset_in_allocation, first_contribution_address, num_cus,
+        align_short_operations != 0);
+    int n = 0;
+    for (const frg::LaunchPart& p : parts) {
+      if (p.bytes <= 0) continue;
+      if (n < capacity && launch_elems != nullptr) launch_elems[n] = p.bytes / element_size;
+      if (n < capacity && blocks_per_cu != nullptr) blocks_per_cu[n] = p.blocksPerCu;
+      ++n;
+    }
+    *count = n;
+    return static_cast<int>(FRG_OK);
+  });
+}
+
 int frg_reduce_slice(void* out, const void* const* contribs, int K, int64_t n, int dtype,
                      int op, int scale_mode, float scale, int carry, void* stream) {
   frg::ReduceArgs a;

@@ -33,6 +33,11 @@ struct ReduceArgs {
   // Blocks of the persistent grid per CU; 0 = the kernel's own rule. The
   // pipeline sets it together with the launch size (whole rounds of the grid).
   int blocks_per_cu = 0;
+  // Bytes of the slice ahead of the first tile of the rounds; -1 = the kernel's
+  // own rule (up to the first 4 KiB boundary of the first contribution). The
+  // pipeline starts the rounds where the output reaches a 4 MiB boundary of its
+  // allocation.
+  int64_t lead_bytes = -1;
   // Optional timing events (created with timing enabled) that receive the
   // begin and end timestamps of this launch.
   hipEvent_t startEvent = nullptr;

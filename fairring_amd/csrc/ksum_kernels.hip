@@ -182,8 +182,9 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
 
 // Body kernel. The slice is [head scalars][nvec vectors][tail scalars], where
 // `head` brings every pointer to a 16-byte boundary. The first `lead` vectors
-// (fewer than a tile) are a piece of their own, so that the tiles start on a
-// 4 KiB boundary of the first contribution: a wave's load then covers eight
+// are dealt in pieces of their own, so that the tiles start on a 4 KiB
+// boundary of the first contribution (or where the caller wants its rounds to
+// start, ReduceArgs::lead_bytes): a wave's load then covers eight
 // whole 128-byte lines instead of straddling nine (measured on MI355X, 8-way
 // fp32: 6,465 GB/s from a 4 KiB boundary, 5,940 from 16 bytes past one). Full tiles of
 // kBlock*kUnroll vectors are dealt to the blocks round-robin for as many whole
@@ -238,10 +239,20 @@ __global__ void __launch_bounds__(kBlock)
       }
     }
   }
-  // the vectors ahead of the first tile, done by the last block (block 0 has the edges)
-  if (lead > 0 && blockIdx.x == gridDim.x - 1) {
-    for (unsigned int lane = threadIdx.x; lane < static_cast<unsigned int>(lead); lane += kBlock) {
-      reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags, head, lane);
+  // the vectors ahead of the first tile, in pieces like the remainder's, dealt
+  // from the last block downwards (the remainder's go from block 0 upwards, and
+  // block 0 has the edges). Fewer than a tile when they only bring the tiles to a
+  // 4 KiB boundary; up to a round when the caller starts the rounds further in.
+  const int64_t leadPieces = (static_cast<int64_t>(lead) + pieceVecs - 1) / pieceVecs;
+  for (int64_t p = grid - 1 - blockIdx.x; p < leadPieces; p += grid) {
+    const int64_t v0 = p * pieceVecs;
+#pragma unroll
+    for (int u = 0; u < kPiece; ++u) {
+      const unsigned int lane = threadIdx.x + u * kBlock;
+      if (v0 + lane < lead) {
+        reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags,
+                                   head + v0 * TRV::kLanes, lane);
+      }
     }
   }
   // ragged edges: at most kLanes-1 scalars on each side, done by block 0
@@ -257,8 +268,14 @@ __global__ void __launch_bounds__(kBlock)
 // its first contribution (0 for the element-wise variants and for slices that
 // end before the boundary).
 template <typename TRV>
-int leadVectors(const void* firstContrib, int64_t head, int64_t nvec) {
+int leadVectors(const void* firstContrib, int64_t head, int64_t nvec, int64_t leadBytesHint) {
   if (sizeof(typename TRV::vec_t) != 16) return 0;
+  if (leadBytesHint >= 0) {
+    // the caller's choice, counted from the first byte of the slice
+    const int64_t headBytes = head * static_cast<int64_t>(sizeof(typename TRV::elem_t));
+    const int64_t lead = leadBytesHint > headBytes ? (leadBytesHint - headBytes) / 16 : 0;
+    return lead < nvec && lead < (int64_t{1} << 30) ? static_cast<int>(lead) : 0;
+  }
   const uintptr_t first = reinterpret_cast<uintptr_t>(firstContrib) +
                           static_cast<uintptr_t>(head) * sizeof(typename TRV::elem_t);
   const int64_t lead = static_cast<int64_t>(((kLaunchAlignBytes - (first & (kLaunchAlignBytes - 1))) &
@@ -291,7 +308,7 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   // phases per tile, which more resident waves hide (K = 16: 6,604 GB/s with 4
   // blocks per CU against 6,229 with 2, launches of one round either way).
   const int manyWay = KT == 0 && a.K > kChunk ? 4 : 0;
-  const int lead = leadVectors<TRV>(a.contribs[0], head, nvec);
+  const int lead = leadVectors<TRV>(a.contribs[0], head, nvec, a.lead_bytes);
   const int hint = a.blocks_per_cu > 0 ? a.blocks_per_cu
                                        : (kEightWayGradient || kPreScaledHalf ? 3 : manyWay);
   const GridPlan plan = planGrid(nvec - lead, a.K, numCus, hint);

@@ -6,7 +6,11 @@
 
 #include <stdint.h>
 
+#include <stddef.h>
+
 #include <limits>
+#include <utility>
+#include <vector>
 
 namespace frg {
 
@@ -43,22 +47,23 @@ constexpr int64_t kDefaultParallelism = 16;                   // fairring/__init
 //   K = 64: 2 blocks, 3.1 MiB 5,968 | 4 blocks, 4 / 8 MiB 6,552 / 6,481
 // (more than 8 contributions are loaded 8 at a time, several dependent load
 // phases per tile, which the additional waves hide).
-// Operations of a DDP bucket's size are another matter: they want launches
-// that divide them. 25 MiB buckets, 8-way fp32, fresh boxes, whole job: 2 x
-// 12.5 MiB with 3 blocks per CU 6,345 to 6,367; with 4 blocks 6,216; 8 + 8 + 9 MiB
-// with 4 blocks 6,130, with 3 blocks 6,259; 12 + 13 MiB 6,286 to 6,313. So up
-// to 8 contributions the whole-round shape applies from 100 MiB per
-// contribution, and below that the launch is 12.5 MiB with the kernel's own
-// grid (3 blocks per CU for the 8-way fp32 sum, else 32 loads in flight per CU).
+// (Operations of a DDP bucket's size: see LaunchShape below.)
 // K = 3 (5 blocks per CU, rounds of 5 MiB): 12.5 MiB 6,395, 15 / 20 / 25 MiB 6,526-6,596 /
 // 6,571 / 6,552; 6 blocks, 12 / 18 / 24 MiB 6,113 / 6,365 / 6,343; 4 blocks, 16 MiB 6,235.
 // K <= 2 (8 blocks per CU, rounds of 8 MiB): 48 / 50 / 56 MiB 6,450 / 6,407 / 6,433; another
 // process: 8 blocks, 32 / 48 / 64 MiB 6,284 / 6,314 / 6,285; 6 blocks, 24 / 48 MiB 6,395 /
 // 6,436; 4 blocks, 16 / 32 / 48 MiB 5,753 / 6,394 / 6,208.
+//
+// From 4 contributions on, operations of every size are cut by planAlignedLaunches
+// (below): whole rounds of the 4-blocks-per-CU grid placed where the output's
+// allocation has its 4 MiB multiples.
 struct LaunchShape {
   int64_t bytes = 0;
   int blocksPerCu = 0;
+  // cut the operation with planAlignedLaunches, `bytes` being the size aimed at
+  bool wholeRounds = false;
 };
+constexpr int64_t kTileBytes = 4096;  // of every contribution, per block and step of the kernel
 constexpr int64_t kDefaultMaxLaunchBytes = 25ll * 1024 * 1024 / 2;
 constexpr int64_t kWholeRoundBytes = 4ll * 1024 * 1024;     // 256 CUs x 4 blocks x 4 KiB
 constexpr int64_t kWholeRoundsFrom = 100ll * 1024 * 1024;   // per contribution, up to 8 of them
@@ -67,12 +72,143 @@ inline constexpr LaunchShape defaultLaunchShape(int numContribs, int64_t bytesPe
   const bool large = bytesPerContrib >= kWholeRoundsFrom;
   if (numContribs <= 2) return LaunchShape{48ll * 1024 * 1024, large ? 6 : 0};
   if (numContribs == 3) return LaunchShape{large ? 20ll * 1024 * 1024 : kDefaultMaxLaunchBytes, 0};
-  if (numContribs <= 8 && !large) return LaunchShape{kDefaultMaxLaunchBytes, 0};
   // whole rounds nearest to the target, at least one
   const int64_t perContrib = kBytesPerLaunchTarget / (numContribs + 1);
   int64_t rounds = (perContrib + kWholeRoundBytes / 2) / kWholeRoundBytes;
   if (rounds < 1) rounds = 1;
-  return LaunchShape{rounds * kWholeRoundBytes, 4};
+  return LaunchShape{rounds * kWholeRoundBytes, 4, true};
+}
+
+// One launch of a partition: its share of every contribution, the grid it runs
+// on and the bytes it takes ahead of its first round.
+struct LaunchPart {
+  int64_t bytes = 0;
+  int blocksPerCu = 0;     // 0: the kernel's own rule
+  int64_t leadBytes = -1;  // -1: the kernel's own rule (up to the first 4 KiB boundary)
+};
+
+// A round of the 4-blocks-per-CU grid: 4 MiB of every contribution on MI355X.
+inline constexpr int64_t alignedRoundBytes(int numCus) {
+  return static_cast<int64_t>(numCus) * 4 * kTileBytes;
+}
+
+// Cuts `bytes` of every contribution into launches of whole rounds of the
+// 4-blocks-per-CU grid whose rounds all start `leadBytes` into the operation and
+// at multiples of a round from there. What matters is where the rounds lie in
+// memory: a round sweeps one window of 4 MiB per buffer, and on MI355X the rate
+// depends on where the OUTPUT's windows start relative to the start of its
+// allocation, with a period of 4 MiB (8-way fp32, one process, nine buffers
+// carved from one allocation at these offsets: all on a 4 MiB multiple 6,576
+// GB/s; all 1 MiB past one 6,280; all 2 MiB past one 6,205; the inputs on one
+// and the output 2 MiB past 6,322; the inputs 2 MiB past and the output on one
+// 6,508; half the inputs 2 MiB past 6,596). The caller therefore passes as
+// `leadBytes` the distance from the operation's start to where the output next
+// reaches such a multiple: those bytes go to the first launch as extra pieces
+// ahead of its rounds, the launches take `targetBytes` worth of rounds each
+// (what is left over one more on the last ones), and the bytes behind the last
+// whole round go to the last launch as remainder pieces. An operation of fewer
+// than two rounds is one launch on the kernel's own grid.
+inline std::vector<LaunchPart> planAlignedLaunches(int64_t bytes, int64_t leadBytes,
+                                                   int64_t targetBytes, int numCus) {
+  const int64_t round = alignedRoundBytes(numCus);
+  std::vector<LaunchPart> parts;
+  const int64_t body = bytes - leadBytes;
+  const int64_t rounds = body > 0 ? body / round : 0;
+  if (rounds < 2) {
+    parts.push_back(LaunchPart{bytes, 0, -1});
+    return parts;
+  }
+  int64_t perLaunch = (targetBytes + round / 2) / round;
+  if (perLaunch < 1) perLaunch = 1;
+  int64_t launches = rounds / perLaunch;
+  if (launches < 1) launches = 1;
+  int64_t extra = rounds - launches * perLaunch;  // rounds no launch has yet
+  for (int64_t i = 0; i < launches; ++i) {
+    // the extra rounds go one each to the last launches (all to the last one
+    // when there are more of them than launches)
+    int64_t mine = perLaunch;
+    if (launches - i <= extra) mine += 1;
+    parts.push_back(LaunchPart{mine * round, 4, -1});
+  }
+  int64_t given = 0;
+  for (const LaunchPart& p : parts) given += p.bytes;
+  parts.back().bytes += rounds * round - given;
+  parts.front().bytes += leadBytes;
+  parts.front().leadBytes = leadBytes;
+  parts.back().bytes += body - rounds * round;
+  return parts;
+}
+
+// Where the rounds of an operation start: `outOffset` is the output's distance
+// from the start of its allocation, `firstContrib` the address of the first
+// contribution (the kernel keeps its tiles on 4 KiB boundaries of that one).
+// The result is the number of bytes ahead of the first round: up to the next
+// multiple of a round in the output, moved back to the 4 KiB grid of the first
+// contribution where the two disagree.
+inline int64_t alignedLeadBytes(uint64_t outOffset, uint64_t firstContrib, int numCus) {
+  const uint64_t round = static_cast<uint64_t>(alignedRoundBytes(numCus));
+  const uint64_t toRound = (round - outOffset % round) % round;
+  const uint64_t toTile = (kTileBytes - firstContrib % kTileBytes) % kTileBytes;
+  return static_cast<int64_t>(toTile + (toRound + round - toTile) % round / kTileBytes * kTileBytes);
+}
+
+// Launches of `size` bytes cut on multiples of the kernel's 4 KiB tile from the
+// operation's start; the last one takes up to one and a half times that.
+inline std::vector<LaunchPart> planEqualLaunches(int64_t bytes, int64_t size, int blocksPerCu) {
+  std::vector<LaunchPart> parts;
+  int64_t part = size / kTileBytes * kTileBytes;
+  if (part < kTileBytes) part = (size + 15) / 16 * 16;  // below a tile: 16-byte boundaries
+  int64_t off = 0;
+  while (2 * (bytes - off) > 3 * part) {
+    parts.push_back(LaunchPart{part, blocksPerCu, -1});
+    off += part;
+  }
+  if (bytes > off || parts.empty()) parts.push_back(LaunchPart{bytes - off, blocksPerCu, -1});
+  return parts;
+}
+
+// Whether the rounds of an operation can be put on the output's multiples of
+// a round at little cost: at most a quarter of a round lies ahead of the first
+// such multiple.
+inline bool alignmentIsCheap(uint64_t outOffset, uint64_t firstContrib, int numCus) {
+  const int64_t toTile = static_cast<int64_t>((kTileBytes - firstContrib % kTileBytes) % kTileBytes);
+  return alignedLeadBytes(outOffset, firstContrib, numCus) - toTile <= alignedRoundBytes(numCus) / 4;
+}
+// An operation of this many rounds or more is aligned whatever lies ahead of its
+// first multiple: the two partial ends are spread over enough whole rounds.
+constexpr int64_t kAlwaysAlignFromRounds = 16;
+
+// The launches of an operation over `bytes` of each of `numContribs`
+// device-resident contributions when the caller asked for no launch size.
+// Up to 3 contributions: equal launches of the shape's size. From 4 on: whole
+// rounds (planAlignedLaunches) that start on the output's multiples of a round
+// for an operation of 16 rounds or more, and for a shorter one when
+// `alignShortOperations` says so and it is cheap (alignmentIsCheap). A shorter
+// operation that starts further from a multiple (a bucket cut from the middle
+// of a gradient) gains nothing from the alignment that the partial rounds at
+// its ends do not take back (25 MiB buckets at offsets of 0 to 3 MiB from a
+// multiple, one process: aligned 6,050 GB/s, equal halves on the kernel's own
+// grid 6,290), and a stream of buckets that changes shape from one to the next
+// loses more than the alignment gains (the same buckets, every fourth one
+// aligned: 5,900; 28 MiB buckets that all sit on a multiple: 6,386 aligned,
+// 6,236 in equal launches): the pipeline passes `alignShortOperations` only
+// while the short operations it sees keep being cheap to align. Otherwise, up
+// to 8 contributions, the operation is cut into equal launches of 12.5 MiB on
+// the kernel's own grid, beyond that into whole rounds from its start.
+inline std::vector<LaunchPart> planDefaultLaunches(int numContribs, int64_t bytes,
+                                                   uint64_t outOffset, uint64_t firstContrib,
+                                                   int numCus, bool alignShortOperations) {
+  const LaunchShape shape = defaultLaunchShape(numContribs, bytes);
+  if (!shape.wholeRounds) return planEqualLaunches(bytes, shape.bytes, shape.blocksPerCu);
+  const int64_t round = alignedRoundBytes(numCus);
+  const int64_t toTile = static_cast<int64_t>((kTileBytes - firstContrib % kTileBytes) % kTileBytes);
+  const int64_t lead = alignedLeadBytes(outOffset, firstContrib, numCus);
+  const bool large = (bytes - lead) / round >= kAlwaysAlignFromRounds;
+  if (large || (alignShortOperations && alignmentIsCheap(outOffset, firstContrib, numCus))) {
+    return planAlignedLaunches(bytes, lead, shape.bytes, numCus);
+  }
+  if (numContribs <= 8) return planEqualLaunches(bytes, kDefaultMaxLaunchBytes, 0);
+  return planAlignedLaunches(bytes, toTile, shape.bytes, numCus);
 }
 
 // The reduction with compression folded in (2 blocks per CU, rounds of 2 MiB
@@ -105,7 +241,7 @@ inline constexpr int64_t defaultCompressedLaunchBytes(int numContribs, bool rawT
 // all of them. With the default shapes that is every operation below 100 MiB
 // per contribution (8 launches of 12.5 MiB), where the whole-round shape begins.
 constexpr int kOneStreamLaunches = 8;
-constexpr int64_t kLaunchQuantumBytes = 4096;  // launch boundaries within a slice: the kernel's tile
+constexpr int64_t kLaunchQuantumBytes = kTileBytes;  // launch boundaries within a slice: the kernel's tile
 
 inline constexpr int64_t ceilOfRatio(int64_t num, int64_t den) {
   return num == 0 ? 0 : (num - 1) / den + 1;

@@ -105,6 +105,79 @@ std::function<void()> CommandQueue::dequeue() {
   return fn;
 }
 
+namespace {
+
+// The streams of every context of the process come from here and go back here
+// when the context goes. A stream is never destroyed (a consumer may still hold
+// an event that orders its own stream after it, fairring/machine.cc:162-175),
+// so without reuse every context created would leave its streams behind, and
+// the runtime maps streams onto a small number of hardware queues in the order
+// they are created: a process that creates contexts one after the other would
+// see its reduce streams land on other queues every time, now and then on the
+// one its default stream uses (measured: the same bucket stream on the same
+// buffers ran at 6.25 or 5.78 TB/s depending on nothing else). With reuse the
+// first context's streams are every later context's streams.
+class StreamPool {
+ public:
+  enum Kind { kReduce = 0, kCopy = 1 };
+
+  // `n` idle streams of the kind on `device`, the longest-lived first; creates
+  // what is missing (non-blocking, default priority). Throws HipFailure.
+  std::vector<hipStream_t> acquire(int device, Kind kind, int n) {
+    std::lock_guard<std::mutex> g(mu_);
+    std::vector<Entry>& all = streams_[kind];
+    std::vector<hipStream_t> out;
+    for (Entry& e : all) {
+      if (static_cast<int>(out.size()) == n) break;
+      if (e.device == device && !e.busy) {
+        e.busy = true;
+        out.push_back(e.stream);
+      }
+    }
+    while (static_cast<int>(out.size()) < n) {
+      hipStream_t s;
+      const hipError_t r = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+      if (r != hipSuccess) {
+        (void)hipGetLastError();
+        releaseLocked(kind, out);
+        throw HipFailure(std::string("hipStreamCreateWithFlags: ") + hipGetErrorString(r));
+      }
+      all.push_back(Entry{s, device, true});
+      out.push_back(s);
+    }
+    return out;
+  }
+
+  // The caller has drained them.
+  void release(Kind kind, const std::vector<hipStream_t>& streams) {
+    std::lock_guard<std::mutex> g(mu_);
+    releaseLocked(kind, streams);
+  }
+
+ private:
+  struct Entry {
+    hipStream_t stream;
+    int device;
+    bool busy;
+  };
+  void releaseLocked(Kind kind, const std::vector<hipStream_t>& streams) {
+    for (hipStream_t s : streams) {
+      for (Entry& e : streams_[kind]) {
+        if (e.stream == s) e.busy = false;
+      }
+    }
+  }
+  std::mutex mu_;
+  std::vector<Entry> streams_[2];
+};
+
+StreamPool& streamPool() {
+  static StreamPool* pool = new StreamPool();  // outlives every context and static destructor
+  return *pool;
+}
+
+}  // namespace
+
 int Context::create(int device, const frg_options& o, Context** out, std::string* err) {
   const int64_t total = o.max_memory_allocated_in_bytes > 0 ? o.max_memory_allocated_in_bytes
                                                              : kDefaultTotalMemory;
@@ -157,6 +230,13 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
+  if (const char* v = std::getenv("FAIRRING_IDLE_PRODUCER_CHECK")) {
+    c->idleProducerCheck_ = std::atoi(v) != 0;
+  }
+  if (const char* v = std::getenv("FAIRRING_ONE_STREAM_LAUNCHES")) {
+    const long long m = std::atoll(v);
+    if (m >= 0 && m <= 1 << 20) c->oneStreamLaunches_ = static_cast<int>(m);
+  }
   if (const char* v = std::getenv("FAIRRING_CHAIN_SCRATCH_BYTES")) {
     const long long b = std::atoll(v);
     if (b >= 4096) c->carryScratchBytes_ = b / 4096 * 4096;
@@ -166,11 +246,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
     int nStreams = o.num_reduce_streams > 0 ? o.num_reduce_streams : 2;
     if (nStreams > 8) nStreams = 8;
     // Default priority on purpose: all streams of the pipeline share one level.
-    for (int i = 0; i < nStreams; ++i) {
-      hipStream_t s;
-      FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-      c->reduceStreams_.push_back(s);
-    }
+    c->reduceStreams_ = streamPool().acquire(device, StreamPool::kReduce, nStreams);
     // The copy streams of the host-staged path are created when that path is
     // first used (copyStreams()): until then the context holds its reduce
     // streams only.
@@ -199,12 +275,9 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
                             std::vector<int64_t>(c->reduceStreams_.size(), 0));
   } catch (const std::exception& e) {
     *err = e.what();
-    // partially built: the destructor releases what exists (there is no command
-    // thread to join yet). Nothing has run on the streams and nobody else has
-    // seen them, so unlike those of a context that worked they can go.
-    std::vector<hipStream_t> made = c->reduceStreams_;
+    // partially built: the destructor releases what exists and hands the
+    // streams back (there is no command thread to join yet)
     delete c;
-    for (hipStream_t s : made) (void)hipStreamDestroy(s);
     return FRG_ERR_HIP;
   }
 
@@ -244,7 +317,10 @@ Context::~Context() {
     for (hipEvent_t e : m.events) (void)hipEventDestroy(e);
   }
   // The streams are not destroyed: a consumer may still hold an event that
-  // orders its own stream after one of them (fairring/machine.cc:162-175).
+  // orders its own stream after one of them (fairring/machine.cc:162-175). They
+  // are idle now and serve the next context of the process.
+  streamPool().release(StreamPool::kReduce, reduceStreams_);
+  streamPool().release(StreamPool::kCopy, copyStreams_);
   (void)hipSetDevice(prev);
 }
 
@@ -252,19 +328,7 @@ std::vector<hipStream_t> Context::copyStreams() {
   std::lock_guard<std::mutex> g(copyMu_);
   if (copyStreams_.empty()) {
     DeviceGuard dg(device_);
-    std::vector<hipStream_t> made;
-    try {
-      for (int i = 0; i < numCopyStreams_; ++i) {
-        hipStream_t s;
-        // default priority, like the reduce streams
-        FRG_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-        made.push_back(s);
-      }
-    } catch (...) {
-      for (hipStream_t s : made) (void)hipStreamDestroy(s);
-      throw;
-    }
-    copyStreams_ = std::move(made);
+    copyStreams_ = streamPool().acquire(device_, StreamPool::kCopy, numCopyStreams_);
   }
   return copyStreams_;
 }
@@ -530,9 +594,24 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   try {
     DeviceGuard g(device_);
     // Orders the pipeline after whatever produced the inputs
-    // (fairring/device.cc:294-295).
-    initial = takeEvent();
-    FRG_HIP_CHECK(hipEventRecord(initial, req.producerStream));
+    // (fairring/device.cc:294-295). A producer stream that has already drained
+    // has nothing to wait for, and no event is recorded on it: a record is a
+    // packet on the producer's hardware queue, and two hundred of them per step
+    // (one per bucket) are work for the command processor that the reduction's
+    // own queues then wait behind.
+    bool producerIdle = false;
+    if (idleProducerCheck_) {
+      const hipError_t q = hipStreamQuery(req.producerStream);
+      if (q == hipSuccess) {
+        producerIdle = true;
+      } else {
+        (void)hipGetLastError();  // "not ready" (or a failure the record below will report)
+      }
+    }
+    if (!producerIdle) {
+      initial = takeEvent();
+      FRG_HIP_CHECK(hipEventRecord(initial, req.producerStream));
+    }
   } catch (const std::exception& e) {
     *err = e.what();
     if (initial) giveEvent(initial);
@@ -645,6 +724,25 @@ void Context::chainThroughScratch(const Request& req, const std::vector<const vo
   }
 }
 
+// Start of the allocation that holds `p` (what hipMalloc returned for it), or 0
+// when the runtime does not know the pointer: physical memory is laid out from
+// there, so that is where the 4 MiB multiples that matter to the launch
+// partition are counted from. The last answer is kept: the buckets of a
+// gradient mostly share an allocation.
+uint64_t Context::allocationBase(const void* p) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  if (a >= allocBase_ && a - allocBase_ < allocSize_) return allocBase_;
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  if (hipMemGetAddressRange(&base, &size, const_cast<void*>(p)) != hipSuccess || size == 0) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  allocBase_ = reinterpret_cast<uint64_t>(base);
+  allocSize_ = size;
+  return allocBase_;
+}
+
 // ---- order between operations ----------------------------------------------
 
 Context::OpSpans Context::spansOf(const Request& req) {
@@ -735,6 +833,7 @@ void Context::remember(OpSpans op, const std::vector<size_t>& targets) {
 }
 
 void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired) {
+  if (initialEvent == nullptr) return;  // the producer stream was idle when the operation came in
   // Once the producer's event has fired no stream needs to wait for it: a
   // wait that is already satisfied still costs a barrier packet on the queue.
   if (!*fired) {
@@ -794,7 +893,16 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   // at slice boundaries ran at 5.0 TB/s, these run at 6.3. A launch size of
   // "whole slice" (max_launch_bytes < 0) keeps one launch per slice.
   nextStagingSlot_ += nSlices;
-  std::vector<std::pair<int64_t, int64_t>> ranges;  // (offset, length) in elements
+  struct Range {
+    int64_t first;   // offset in elements
+    int64_t second;  // length in elements
+    int blocksPerCu;
+    int64_t leadBytes;
+  };
+  std::vector<Range> ranges;
+  auto addRange = [&](int64_t off, int64_t len) {
+    ranges.push_back(Range{off, len, shape.blocksPerCu, -1});
+  };
   const bool identity = !req.compressed && total == 1 && req.contribs[0] == req.out &&
                         req.scaleMode == FRG_SCALE_NONE;
   if (identity) {
@@ -804,7 +912,36 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     for (int64_t i = 0; i < nSlices; ++i) {
       int64_t off, len;
       sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &off, &len);
-      ranges.emplace_back(off, len);
+      addRange(off, len);
+    }
+  } else if (launchBytesByContribs_ && !req.compressed) {
+    // no launch size asked for: the library's own partition (layout.h)
+    const int numCus = computeUnits(device_);
+    const uint64_t outOffset = (reinterpret_cast<uint64_t>(req.out) - allocationBase(req.out)) %
+                               static_cast<uint64_t>(alignedRoundBytes(numCus));
+    const uint64_t first = reinterpret_cast<uint64_t>(req.contribs[0]);
+    const int64_t bytes = req.numel * elsize;
+    // A stream of short operations keeps one launch shape: they are aligned
+    // only once several in a row were cheap to align, and not again after one
+    // that is not until as many have been.
+    const bool shortOp = bytes / alignedRoundBytes(numCus) < kAlwaysAlignFromRounds;
+    if (shortOp) {
+      cheapStreak_ = alignmentIsCheap(outOffset, first, numCus) ? cheapStreak_ + 1 : 0;
+    }
+    const bool alignShort = cheapStreak_ > kAlignAfterStreak;
+    if (bytes != planBytes_ || outOffset != planOutOffset_ || first % kTileBytes != planFirst_ ||
+        total != planContribs_ || alignShort != planAlignShort_) {
+      plan_ = planDefaultLaunches(total, bytes, outOffset, first, numCus, alignShort);
+      planAlignShort_ = alignShort;
+      planBytes_ = bytes;
+      planOutOffset_ = outOffset;
+      planFirst_ = first % kTileBytes;
+      planContribs_ = total;
+    }
+    int64_t off = 0;
+    for (const LaunchPart& p : plan_) {
+      if (p.bytes > 0) ranges.push_back(Range{off, p.bytes / elsize, p.blocksPerCu, p.leadBytes});
+      off += p.bytes / elsize;
     }
   } else {
     const int64_t quantum = kLaunchQuantumBytes / elsize;
@@ -814,10 +951,10 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     }
     int64_t off = 0;
     while (2 * (req.numel - off) > 3 * partLen) {
-      ranges.emplace_back(off, partLen);
+      addRange(off, partLen);
       off += partLen;
     }
-    if (req.numel > off) ranges.emplace_back(off, req.numel - off);
+    if (req.numel > off) addRange(off, req.numel - off);
   }
 
   // An operation of a few launches (a DDP bucket) stays on one stream and the
@@ -825,7 +962,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   // ends on a single stream (nothing to join for its completion), and nothing is
   // recorded between two launches. A large operation deals its own launches
   // round-robin over the streams.
-  const bool oneStream = ranges.size() <= static_cast<size_t>(kOneStreamLaunches);
+  const bool oneStream = ranges.size() <= static_cast<size_t>(oneStreamLaunches_);
   const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
   if (oneStream && !ranges.empty()) ++nextLaunch_;
   const OpSpans spans = spansOf(req);
@@ -891,7 +1028,8 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
                                                                         : FRG_SCALE_NONE;
       a.scale = req.scale;
       a.carry = k0 > 0;
-      a.blocks_per_cu = shape.blocksPerCu;
+      a.blocks_per_cu = range.blocksPerCu;
+      a.lead_bytes = range.leadBytes;
       launch(a, s);
     }
     lastIdx = si;
@@ -1091,7 +1229,7 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
     std::fprintf(stderr, "[fairring] operation #%lld failed: %s\n",
                  static_cast<long long>(seq), error.c_str());
   }
-  giveEvent(initialEvent);
+  if (initialEvent != nullptr) giveEvent(initialEvent);
   progress_->enqueued.fetch_add(1);
   {
     std::lock_guard<std::mutex> g(work->mu);

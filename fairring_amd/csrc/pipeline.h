@@ -180,7 +180,26 @@ class Context {
   int64_t slotBytes_ = 0;
   int64_t maxLaunchBytes_ = 0;   // per contribution and launch; 0 = whole slice
   bool launchBytesByContribs_ = false;  // no size was asked for: it follows the contribution count
-  int64_t nextLaunch_ = 0;       // deals launches to the reduce streams
+  uint64_t allocationBase(const void* p);
+  uint64_t allocBase_ = 0;  // the allocation looked up last
+  uint64_t allocSize_ = 0;
+  // The last partition computed (the buckets of a gradient repeat).
+  std::vector<LaunchPart> plan_;
+  int64_t planBytes_ = -1;
+  uint64_t planOutOffset_ = 0, planFirst_ = 0;
+  int planContribs_ = -1;
+  bool planAlignShort_ = false;
+  // Short operations in a row that were cheap to align (layout.h::planDefaultLaunches).
+  static constexpr int kAlignAfterStreak = 4;
+  int cheapStreak_ = 0;
+  int64_t nextLaunch_ = 0;       // deals launches (or whole operations) to the reduce streams
+  // An operation of at most this many launches stays on one reduce stream;
+  // FAIRRING_ONE_STREAM_LAUNCHES overrides it when the context is created (0:
+  // every operation deals its launches over all streams).
+  int oneStreamLaunches_ = kOneStreamLaunches;
+  // Ask the runtime whether the producer stream has drained before recording
+  // the initial event on it (FAIRRING_IDLE_PRODUCER_CHECK=0 records always).
+  bool idleProducerCheck_ = true;
 
   std::vector<hipStream_t> reduceStreams_;
   // Slot s is filled on copy stream s % copyStreams_.size(): while one stream works through the

@@ -52,6 +52,21 @@ def compute_layout(max_memory, max_padding, min_parallelism, num_machines, devic
                 padding_slots=out.num_padding_slots, staging_slots=out.num_staging_slots)
 
 
+def plan_launches(k, numel, element_size, first_contribution_address=0,
+                  out_offset_in_allocation=0, align_short_operations=False, num_cus=256):
+    """The launches the pipeline cuts an operation into by default:
+    [(elements, blocks per CU), ...] in order (frg_plan_launches)."""
+    cap = 1 << 16
+    elems = (ctypes.c_int64 * cap)()
+    bpc = (ctypes.c_int32 * cap)()
+    n = ctypes.c_int()
+    _capi.check(_capi.lib().frg_plan_launches(k, numel, element_size, first_contribution_address,
+                                              out_offset_in_allocation,
+                                              1 if align_short_operations else 0, num_cus, elems,
+                                              bpc, cap, ctypes.byref(n)))
+    return [(elems[i], bpc[i]) for i in range(min(n.value, cap))]
+
+
 def _dtype_code(t):
     import torch
     codes = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16, torch.float64: F64,

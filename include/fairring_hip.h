@@ -93,6 +93,34 @@ FRG_API int frg_slice_bounds(int64_t numel, int64_t slice_size_in_bytes,
                              int64_t element_size, int64_t idx,
                              int64_t* offset_in_elems, int64_t* size_in_elems);
 
+/* Not in the reference, which hands every slice to one library call: the
+ * launches into which frg_allreduce cuts an operation over `numel` elements of
+ * `element_size` bytes and K device-resident contributions when no launch size
+ * was asked for (frg_options.max_launch_bytes == 0), in order: elements per
+ * launch and blocks of the persistent grid per CU (0: the kernel's own rule).
+ * From 4 contributions on, an operation of 64 MiB or more per contribution is
+ * cut into whole rounds of a grid of 4 blocks per CU (a round: num_cus x 4
+ * blocks x 4 KiB of every contribution, 4 MiB on MI355X), and the rounds start
+ * where the output reaches a multiple of a round counted from the start of its
+ * allocation (`out_offset_in_allocation`: the output's address minus what
+ * hipMemGetAddressRange reports as the base; where the rounds lie in physical
+ * memory sets the rate) on the 4 KiB grid of the first contribution
+ * (`first_contribution_address`). The first launch also takes the bytes ahead
+ * of that point and the last one those behind the last whole round. A shorter
+ * operation is cut the same way when `align_short_operations` is set and at
+ * most a quarter of a round lies ahead of that point (the pipeline sets it once
+ * four short operations in a row met that condition, so that a stream of
+ * buckets keeps one shape); otherwise, up to 8 contributions, into equal
+ * launches of 12.5 MiB on the kernel's own grid. `num_cus`: compute units of
+ * the device (256 on MI355X). `*count` receives the number of launches, also
+ * when it exceeds `capacity`. */
+FRG_API int frg_plan_launches(int K, int64_t numel, int64_t element_size,
+                              uint64_t first_contribution_address,
+                              uint64_t out_offset_in_allocation,
+                              int align_short_operations, int num_cus,
+                              int64_t* launch_elems, int32_t* blocks_per_cu, int capacity,
+                              int* count);
+
 /* ---- one reduction launch (no pipeline) -------------------------------- */
 
 /* doReduction: fairring/device.cc:108-131 (at::sum_out / at::amax_out over

@@ -155,6 +155,7 @@ std::vector<HwQueue*> gSharedQueues;  // empty: a queue per stream
 size_t gNextQueue = 0;
 FakeStream* gDefaultStream = nullptr;
 std::vector<FakeStream*> gBlockingStreams;  // live streams created without hipStreamNonBlocking
+std::vector<FakeStream*> gAllStreams;       // every live stream but the null stream
 
 HwQueue* pickQueueLocked() {
   if (gSharedQueues.empty()) return nullptr;
@@ -280,6 +281,7 @@ hipError_t hipStreamCreateWithFlags(hipStream_t* stream, unsigned int flags) {
   std::lock_guard<std::mutex> g(gTopologyMu);
   *stream = new FakeStream(pickQueueLocked(), blocking);
   if (blocking) gBlockingStreams.push_back(*stream);
+  gAllStreams.push_back(*stream);
   return hipSuccess;
 }
 
@@ -288,10 +290,12 @@ hipError_t hipStreamDestroy(hipStream_t stream) {
   if (stream == nullptr) return ret(hipErrorInvalidValue);
   {
     std::lock_guard<std::mutex> g(gTopologyMu);
-    for (size_t i = 0; i < gBlockingStreams.size(); ++i) {
-      if (gBlockingStreams[i] == stream) {
-        gBlockingStreams.erase(gBlockingStreams.begin() + static_cast<long>(i));
-        break;
+    for (std::vector<FakeStream*>* list : {&gBlockingStreams, &gAllStreams}) {
+      for (size_t i = 0; i < list->size(); ++i) {
+        if ((*list)[i] == stream) {
+          list->erase(list->begin() + static_cast<long>(i));
+          break;
+        }
       }
     }
   }
@@ -411,15 +415,38 @@ hipError_t hipEventElapsedTime(float* ms, hipEvent_t start, hipEvent_t stop) {
   return hipSuccess;
 }
 
+static std::mutex gAllocMu;
+static std::map<uintptr_t, size_t> gAllocs;  // what hipMalloc handed out
+
 hipError_t hipMalloc(void** ptr, size_t size) {
   if (enter("hipMalloc")) return ret(hipErrorOutOfMemory);
   *ptr = std::malloc(size ? size : 1);
-  return *ptr ? hipSuccess : ret(hipErrorOutOfMemory);
+  if (*ptr == nullptr) return ret(hipErrorOutOfMemory);
+  std::lock_guard<std::mutex> g(gAllocMu);
+  gAllocs[reinterpret_cast<uintptr_t>(*ptr)] = size ? size : 1;
+  return hipSuccess;
 }
 
 hipError_t hipFree(void* ptr) {
   enter("hipFree");
+  {
+    std::lock_guard<std::mutex> g(gAllocMu);
+    gAllocs.erase(reinterpret_cast<uintptr_t>(ptr));
+  }
   std::free(ptr);
+  return hipSuccess;
+}
+
+hipError_t hipMemGetAddressRange(hipDeviceptr_t* base, size_t* size, hipDeviceptr_t ptr) {
+  enter("hipMemGetAddressRange");
+  const uintptr_t a = reinterpret_cast<uintptr_t>(ptr);
+  std::lock_guard<std::mutex> g(gAllocMu);
+  auto it = gAllocs.upper_bound(a);
+  if (it == gAllocs.begin()) return ret(hipErrorInvalidValue);
+  --it;
+  if (a - it->first >= it->second) return ret(hipErrorInvalidValue);
+  *base = reinterpret_cast<void*>(it->first);
+  *size = it->second;
   return hipSuccess;
 }
 
@@ -443,10 +470,18 @@ void fake_hip_set_hw_queues(int n) {
   }
   if (old != nullptr) old->drain();  // left alive: an event may still point into it
   std::lock_guard<std::mutex> g(gTopologyMu);
-  // queues of an earlier topology stay: streams created then still run on them
+  for (FakeStream* s : gAllStreams) s->drain();
+  for (HwQueue* q : gSharedQueues) delete q;  // idle: everything mapped onto them is drained
   gSharedQueues.clear();
   gNextQueue = 0;
   for (int i = 0; i < n; ++i) gSharedQueues.push_back(new HwQueue());
+  // the streams that exist move onto the new queues in the order they were created
+  for (FakeStream* s : gAllStreams) {
+    if (s->ownsQueue) delete s->queue;
+    HwQueue* shared = pickQueueLocked();
+    s->ownsQueue = shared == nullptr;
+    s->queue = shared != nullptr ? shared : new HwQueue();
+  }
 }
 
 void fake_hip_fail_call(const char* api, int nth) {

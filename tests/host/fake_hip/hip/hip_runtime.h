@@ -6,8 +6,9 @@
 // Semantics kept: a stream is an in-order queue; an event record is a point in
 // its stream; a stream wait snapshots the event's record at the time of the
 // call; "device memory" is host memory. By default every stream is drained by a
-// thread of its own. fake_hip_set_hw_queues(n) instead maps the streams created
-// afterwards (the null stream included) round-robin onto n hardware queues, each
+// thread of its own. fake_hip_set_hw_queues(n) instead maps the streams (those
+// that exist, in the order they were created, and those created afterwards; the
+// null stream included) round-robin onto n hardware queues, each
 // an in-order queue shared by its streams: a wait packet holds up every stream
 // behind it in that queue, as on a GPU whose process has fewer hardware queues
 // than streams. The null stream synchronises implicitly with streams created
@@ -72,7 +73,10 @@ hipError_t hipEventQuery(hipEvent_t event);
 hipError_t hipEventSynchronize(hipEvent_t event);
 hipError_t hipEventElapsedTime(float* ms, hipEvent_t start, hipEvent_t stop);
 
+typedef void* hipDeviceptr_t;
 hipError_t hipMalloc(void** ptr, size_t size);
+// Only memory that came from hipMalloc is known; everything else fails.
+hipError_t hipMemGetAddressRange(hipDeviceptr_t* base, size_t* size, hipDeviceptr_t ptr);
 hipError_t hipFree(void* ptr);
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind kind,
                           hipStream_t stream);
@@ -80,8 +84,8 @@ hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKin
 // ---- hooks for tests ------------------------------------------------------
 // Occupies `stream` (nullptr = the default stream) for `ms` milliseconds.
 void fake_hip_occupy(hipStream_t stream, int ms);
-// Streams created from now on share `n` in-order hardware queues (0: a queue
-// per stream, the default). Call it while no work is in flight.
+// Every stream, existing or yet to be created, shares `n` in-order hardware
+// queues (0: a queue per stream, the default). Call it while no work is in flight.
 void fake_hip_set_hw_queues(int n);
 // Makes hipStreamIsCapturing report a capture in progress on every stream (1) or none (0).
 void fake_hip_set_capturing(int on);

@@ -19,28 +19,29 @@
 #include "../../fairring_amd/csrc/layout.h"
 #include "../../include/fairring_hip.h"
 
-// The default launch shapes, pinned: 48 MiB up to 2 contributions; up to 8
-// contributions 12.5 MiB with the kernel's own grid for operations of a bucket's
-// size and whole rounds of a 4-blocks-per-CU grid (4 MiB each, about 80 MB per
-// launch) from 100 MiB per contribution; whole rounds for more than 8 always.
+// The default launch shapes, pinned: 48 MiB up to 2 contributions; 3 contributions
+// 12.5 MiB with the kernel's own grid, 20 MiB from 100 MiB per contribution; from 4
+// contributions on launches of whole rounds aimed at about 80 MB per launch.
 static_assert(frg::defaultLaunchShape(2, 1ll << 30).bytes == 48ll << 20);
-static_assert(frg::defaultLaunchShape(8, 25ll << 20).bytes == 13107200);
-static_assert(frg::defaultLaunchShape(8, 25ll << 20).blocksPerCu == 0);
+static_assert(frg::defaultLaunchShape(2, 1ll << 30).blocksPerCu == 6);
+static_assert(frg::defaultLaunchShape(2, 1ll << 20).blocksPerCu == 0);
+static_assert(!frg::defaultLaunchShape(2, 1ll << 30).wholeRounds);
+static_assert(frg::defaultLaunchShape(3, 1ll << 30).bytes == 20ll << 20);
+static_assert(frg::defaultLaunchShape(3, 1ll << 20).bytes == 13107200);
+static_assert(!frg::defaultLaunchShape(3, 1ll << 30).wholeRounds);
+static_assert(frg::defaultLaunchShape(8, 25ll << 20).bytes == 8ll << 20);
+static_assert(frg::defaultLaunchShape(8, 25ll << 20).wholeRounds);
 static_assert(frg::defaultLaunchShape(8, 100ll << 20).bytes == 8ll << 20);
 static_assert(frg::defaultLaunchShape(8, 100ll << 20).blocksPerCu == 4);
 static_assert(frg::defaultLaunchShape(4, 1ll << 30).bytes == 16ll << 20);
 static_assert(frg::defaultLaunchShape(5, 1ll << 30).bytes == 12ll << 20);
 static_assert(frg::defaultLaunchShape(7, 1ll << 30).bytes == 12ll << 20);
-static_assert(frg::defaultLaunchShape(3, 1ll << 30).bytes == 20ll << 20);
-static_assert(frg::defaultLaunchShape(2, 1ll << 30).blocksPerCu == 6);
-static_assert(frg::defaultLaunchShape(2, 1ll << 20).blocksPerCu == 0);
-static_assert(frg::defaultLaunchShape(3, 1ll << 20).bytes == 13107200);
 static_assert(frg::defaultLaunchShape(9, 1ll << 20).bytes == 8ll << 20);
 static_assert(frg::defaultLaunchShape(12, 1ll << 30).bytes == 8ll << 20);
 static_assert(frg::defaultLaunchShape(13, 1ll << 30).bytes == 4ll << 20);
 static_assert(frg::defaultLaunchShape(16, 1ll << 30).bytes == 4ll << 20);
 static_assert(frg::defaultLaunchShape(64, 1ll << 30).bytes == 4ll << 20);
-static_assert(frg::defaultLaunchShape(64, 1ll << 30).blocksPerCu == 4);
+static_assert(frg::defaultLaunchShape(64, 1ll << 30).wholeRounds);
 // the compressed reduction: whole rounds of 2 MiB of wire, about 80 MB per launch; a bucket is one launch
 static_assert(frg::defaultCompressedLaunchBytes(8, true, true, 1ll << 30) == 8ll << 20);
 static_assert(frg::defaultCompressedLaunchBytes(8, true, true, 12ll << 20) == 16ll << 20);
@@ -241,6 +242,99 @@ int64_t launchesSoFar(frg_ctx* ctx) {
   return p.launches;
 }
 
+void scenarioWholeRoundPlan() {
+  std::puts("aligned launch plan: whole rounds placed on the output's multiples of a round");
+  const int64_t MiB = 1 << 20;
+  auto sizes = [](const std::vector<frg::LaunchPart>& v) {
+    std::vector<std::vector<int64_t>> out;
+    for (auto& p : v) out.push_back({p.bytes, p.blocksPerCu, p.leadBytes});
+    return out;
+  };
+  using P = std::vector<std::vector<int64_t>>;
+  // 256 CUs: a round of the 4-blocks-per-CU grid is 4 MiB
+  CHECK(frg::alignedRoundBytes(256) == 4 * MiB);
+  // a bucket on a multiple of a round: 2 + 2 + 2 rounds, 1 MiB left to the last launch
+  CHECK(sizes(frg::planAlignedLaunches(25 * MiB, 0, 8 * MiB, 256)) ==
+        (P{{8 * MiB, 4, 0}, {8 * MiB, 4, -1}, {9 * MiB, 4, -1}}));
+  CHECK(sizes(frg::planAlignedLaunches(24 * MiB, 0, 8 * MiB, 256)) ==
+        (P{{8 * MiB, 4, 0}, {8 * MiB, 4, -1}, {8 * MiB, 4, -1}}));
+  // 1 MiB past a multiple: 3 MiB ahead of the first round go to the first launch, five
+  // whole rounds follow (2 + 3), 2 MiB behind them go to the last
+  CHECK(sizes(frg::planAlignedLaunches(25 * MiB, 3 * MiB, 8 * MiB, 256)) ==
+        (P{{11 * MiB, 4, 3 * MiB}, {14 * MiB, 4, -1}}));
+  // an odd round goes to the last launch; a lead of less than a tile is like any other
+  CHECK(sizes(frg::planAlignedLaunches(28 * MiB + 1536 + 100, 1536, 8 * MiB, 256)) ==
+        (P{{8 * MiB + 1536, 4, 1536}, {8 * MiB, 4, -1}, {12 * MiB + 100, 4, -1}}));
+  // fewer than two whole rounds: one launch, everything left to the kernel
+  CHECK(sizes(frg::planAlignedLaunches(7 * MiB, 0, 8 * MiB, 256)) == (P{{7 * MiB, 0, -1}}));
+  CHECK(sizes(frg::planAlignedLaunches(10 * MiB, 3 * MiB, 8 * MiB, 256)) == (P{{10 * MiB, 0, -1}}));
+  CHECK(sizes(frg::planAlignedLaunches(0, 0, 8 * MiB, 256)) == (P{{0, 0, -1}}));
+  CHECK(sizes(frg::planAlignedLaunches(100, 3000, 8 * MiB, 256)) == (P{{100, 0, -1}}));
+  CHECK(sizes(frg::planAlignedLaunches(8 * MiB, 0, 8 * MiB, 256)) == (P{{8 * MiB, 4, 0}}));
+  // more contributions aim at one round per launch; few at four
+  CHECK(frg::planAlignedLaunches(25 * MiB, 0, 4 * MiB, 256).size() == 6);
+  CHECK(sizes(frg::planAlignedLaunches(41 * MiB, 0, 16 * MiB, 256)) ==
+        (P{{20 * MiB, 4, 0}, {21 * MiB, 4, -1}}));  // ten rounds as 5 + 5, 1 MiB left over
+  // every size: the parts add up, every launch but the last is whole rounds past its lead
+  for (int64_t lead : {int64_t(0), int64_t(1536), 3 * MiB + 512}) {
+    for (int64_t m = 1; m <= 70; ++m) {
+      const int64_t bytes = m * MiB + 12345 * 16;
+      const auto plan = frg::planAlignedLaunches(bytes, lead, 8 * MiB, 256);
+      int64_t sum = 0;
+      for (size_t i = 0; i < plan.size(); ++i) {
+        sum += plan[i].bytes;
+        if (plan.size() > 1 && i + 1 < plan.size()) {
+          CHECK((plan[i].bytes - (i == 0 ? lead : 0)) % (4 * MiB) == 0);
+        }
+      }
+      CHECK(sum == bytes);
+    }
+  }
+  // a whole gradient: 8 MiB launches throughout
+  const auto big = frg::planAlignedLaunches(5480000000ll, 0, 8 * MiB, 256);
+  int64_t sum = 0;
+  for (auto& p : big) sum += p.bytes;
+  CHECK(sum == 5480000000ll && big.size() == 653);
+  CHECK(big.front().bytes == 8 * MiB && big[big.size() / 2].bytes == 8 * MiB);
+  // where the rounds start: at the output's next multiple of a round within its
+  // allocation, on the 4 KiB grid of the first contribution
+  CHECK(frg::alignedLeadBytes(0, 0x7f0000000000ull, 256) == 0);
+  CHECK(frg::alignedLeadBytes(1 * MiB, 0x7f0000100000ull, 256) == 3 * MiB);
+  CHECK(frg::alignedLeadBytes(4 * MiB - 1536, 0x7f0000000a00ull, 256) == 1536);
+  CHECK(frg::alignedLeadBytes(2 * MiB + 2560, 0x7f0000000a00ull, 256) == 2 * MiB - 2560);
+  // the output 512 bytes off the first contribution's 4 KiB grid: the tile grid wins
+  CHECK(frg::alignedLeadBytes(1 * MiB + 512, 0x7f0000100000ull, 256) == 3 * MiB - 4096);
+  // through the ABI, in elements
+  int64_t elems[8];
+  int32_t bpc[8];
+  int n = 0;
+  CHECK(frg_plan_launches(8, 6553600, 4, 0, 0, 1, 256, elems, bpc, 8, &n) == FRG_OK);
+  CHECK(n == 3 && elems[0] == 2097152 && elems[1] == 2097152 && elems[2] == 2359296);
+  CHECK(bpc[0] == 4 && bpc[2] == 4);
+  // a short operation is not aligned unless the caller says that its neighbours are too
+  CHECK(frg_plan_launches(8, 6553600, 4, 0, 0, 0, 256, elems, bpc, 8, &n) == FRG_OK);
+  CHECK(n == 2 && elems[0] == 3276800 && bpc[0] == 0);
+  // 3 MiB short of a multiple, 5 whole rounds: aligning does not pay, two equal launches
+  CHECK(frg_plan_launches(8, 6553600, 4, 0x7f0000100000ull, 1 * MiB, 1, 256, elems, bpc, 8,
+                          &n) == FRG_OK);
+  CHECK(n == 2 && elems[0] == 3276800 && elems[1] == 3276800 && bpc[0] == 0);
+  // 1 MiB short of one: it does (the first launch takes that MiB ahead of its rounds)
+  CHECK(frg_plan_launches(8, 6553600, 4, 0x7f0000300000ull, 3 * MiB, 1, 256, elems, bpc, 8,
+                          &n) == FRG_OK);
+  CHECK(n == 3 && elems[0] == 9 * MiB / 4 && elems[1] == 2 * MiB && elems[2] == 2 * MiB);
+  // a large operation is aligned wherever it starts
+  CHECK(frg_plan_launches(8, 100 << 20, 4, 0x7f0000200000ull, 2 * MiB, 0, 256, elems, bpc, 8,
+                          &n) == FRG_OK);
+  CHECK(n == 49 && elems[0] == 10 * MiB / 4 && elems[1] == 2 * MiB && bpc[0] == 4);
+  // more than 8 contributions far from a multiple: whole rounds from the start
+  CHECK(frg_plan_launches(16, 6553600, 4, 0x7f0000200000ull, 2 * MiB, 1, 256, elems, bpc, 8,
+                          &n) == FRG_OK);
+  CHECK(n == 6 && elems[0] == 1 * MiB && bpc[0] == 4);
+  CHECK(frg_plan_launches(2, 100 << 20, 4, 0, 0, 0, 256, elems, bpc, 8, &n) == FRG_OK);  // 400 MiB
+  CHECK(n == 8 && elems[0] == 12582912 && bpc[0] == 6);
+  CHECK(frg_plan_launches(0, 10, 4, 0, 0, 0, 256, elems, bpc, 8, &n) == FRG_ERR_INVALID);
+}
+
 void scenarioLaunchPartition() {
   std::puts("launch partition: sizes cut from the tensor on tile boundaries, 1.5x rule, per slice");
   struct Case {
@@ -327,6 +421,31 @@ void scenarioWaitGivesUp() {
   CHECK(frg_destroy(ctx) == FRG_OK);
 }
 
+void scenarioIdleProducer() {
+  std::puts("no event is recorded on a producer stream that has drained");
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  auto c = randomContribs(3, 3000, 31);
+  Vec out(3000);
+  auto t = table(c);
+  frg_work* w = nullptr;
+  CHECK(hipStreamSynchronize(nullptr) == hipSuccess);
+  long records = fake_hip_calls("hipEventRecord");
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
+  CHECK(fake_hip_calls("hipEventRecord") == records);
+  frg_work_release(w);
+  fake_hip_occupy(nullptr, 30);  // busy: the event is recorded and waited for
+  records = fake_hip_calls("hipEventRecord");
+  CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
+                      nullptr, nullptr, nullptr, &w) == FRG_OK);
+  CHECK(fake_hip_calls("hipEventRecord") == records + 1);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  frg_work_release(w);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
 void scenarioProducerOrdering() {
   std::puts("the pipeline waits for the producer stream");
   frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
@@ -397,6 +516,28 @@ std::vector<hipStream_t> streamsOf(frg_ctx* ctx) {
   std::vector<hipStream_t> v;
   for (int i = 0; i < n && i < 16; ++i) v.push_back(static_cast<hipStream_t>(raw[i]));
   return v;
+}
+
+void scenarioStreamsAreReused() {
+  std::puts("contexts created one after the other run on the same streams");
+  frg_ctx* a = makeCtx(8192, 4096, 2, 0);
+  const std::vector<hipStream_t> first = streamsOf(a);
+  CHECK(first.size() == 2);
+  CHECK(frg_destroy(a) == FRG_OK);
+  const long created = fake_hip_calls("hipStreamCreateWithFlags");
+  frg_ctx* b = makeCtx(8192, 4096, 2, 0);
+  CHECK(streamsOf(b) == first);                       // handed back, handed out again
+  frg_ctx* c = makeCtx(8192, 4096, 2, 0);             // while b lives: streams of its own
+  const std::vector<hipStream_t> other = streamsOf(c);
+  CHECK(other.size() == 2 && other[0] != first[0] && other[0] != first[1] &&
+        other[1] != first[0] && other[1] != first[1]);
+  CHECK(frg_destroy(b) == FRG_OK);
+  CHECK(frg_destroy(c) == FRG_OK);
+  frg_ctx* d = makeCtx(8192, 4096, 3, 0);             // three: the oldest idle ones first
+  const std::vector<hipStream_t> three = streamsOf(d);
+  CHECK(three.size() == 3 && three[0] == first[0] && three[1] == first[1]);
+  CHECK(frg_destroy(d) == FRG_OK);
+  CHECK(fake_hip_calls("hipStreamCreateWithFlags") <= created + 2);
 }
 
 void scenarioOrderBetweenOperations() {
@@ -697,6 +838,8 @@ void scenarioErrors() {
   CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
   frg_work_release(w);
   // recording the initial event fails on the caller's thread: the call itself reports it
+  // (the producer's stream must be busy: nothing is recorded on a stream that has drained)
+  fake_hip_occupy(nullptr, 50);
   fake_hip_fail_call("hipEventRecord", 1);
   CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3000, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
                       nullptr, nullptr, nullptr, &w) == FRG_ERR_HIP);
@@ -834,12 +977,15 @@ void runAll() {
   };
   const Scenario all[] = {
       {"resident", scenarioResident},
+      {"aligned launch plan", scenarioWholeRoundPlan},
       {"launch partition", scenarioLaunchPartition},
       {"pre-scale and compressed", scenarioPreScaleAndCompressed},
       {"busy producer", scenarioBusyProducer},
       {"wait gives up", scenarioWaitGivesUp},
       {"block stream gives up", scenarioBlockStreamGivesUp},
+      {"idle producer", scenarioIdleProducer},
       {"producer ordering", scenarioProducerOrdering},
+      {"streams are reused", scenarioStreamsAreReused},
       {"order between operations", scenarioOrderBetweenOperations},
       {"host staged", scenarioHostStaged},
       {"callback", scenarioCallback},

@@ -39,9 +39,9 @@ def test_defaults_are_the_headline_configuration():
     (1_300_000_000, 13_107_200, 2, 0, 4_194_304),  # bf16: the same 8 MiB
     (1_370_000_000, 819_196, 4, 0, 2_097_152),     # default layout (3,276,784 B slices): the same
     (1_370_000_000, 6_553_600, 4, -1, 6_553_600),  # one launch per slice
-    (6_553_600, 6_553_600, 4, 0, 3_276_800),       # one 25 MiB bucket: two launches
+    (6_553_600, 6_553_600, 4, 0, 3_276_800),       # one 25 MiB bucket on its own: two launches
     (262_144, 6_553_600, 4, 0, 262_144),           # the 1 MiB bucket: one launch
-    (4_000_000, 6_553_600, 4, 0, 4_000_000),       # up to 1.5 x the target: still one launch
+    (4_000_000, 6_553_600, 4, 0, 4_000_000),       # up to 1.5 x the launch size: still one launch
     (1_370_000_000, 6_553_600, 4, 6 * MiB, 1_572_864),
 ])
 def test_launch_elems_follows_the_pipeline_rule(op_elems, slice_elems, elsize, lb, want):
