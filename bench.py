@@ -693,10 +693,15 @@ def run_small_ops(args, torch, fa):
 
     dev = fa.DeviceFairring(0)
 
+    # Operations on distinct tensors, like the buckets of a gradient: the pipeline
+    # lets them overlap. (Operations that share a tensor are ordered with an event
+    # between the streams; "in_place_chain" below is that case.)
+    import itertools
+
     def submit_abi(numel):
         xs = [torch.zeros(numel, device="cuda:0") for _ in range(k)]
-        out = torch.empty(numel, device="cuda:0")
-        return lambda: dev.allreduce(out, xs)
+        outs = itertools.cycle([torch.empty(numel, device="cuda:0") for _ in range(4)])
+        return lambda: dev.allreduce(next(outs), xs)
 
     report = {"abi_ctypes": measure(submit_abi, lambda w: w.wait())}
     dev.close()
@@ -714,13 +719,16 @@ def run_small_ops(args, torch, fa):
             timeout=datetime.timedelta(seconds=60), slice_size_in_bytes=args.slice_bytes)
         pg = _fairring.ProcessGroup(dist.HashStore(), 0, k, o)
 
-        def submit_pg(numel):
-            own = torch.zeros(numel, device="cuda:0")
+        def submit_pg(numel, distinct=4):
+            owns = itertools.cycle([[torch.zeros(numel, device="cuda:0")]
+                                    for _ in range(distinct)])
             pg._set_simulated_peer_contributions(
                 [torch.zeros(numel, device="cuda:0") for _ in range(k - 1)])
-            return lambda: pg.allreduce([own])
+            return lambda: pg.allreduce(next(owns))
 
         report["process_group"] = measure(submit_pg, lambda w: w.wait())
+        report["process_group_in_place_chain"] = measure(lambda n: submit_pg(n, 1),
+                                                         lambda w: w.wait())
     # the one-launch entry point on the caller's stream: eager, and the same loop captured
     # once into a HIP graph and replayed (it allocates nothing and records no event)
     nb = 64

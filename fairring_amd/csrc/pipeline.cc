@@ -58,9 +58,21 @@ const char* lastError() { return tlsError.c_str(); }
 
 namespace {
 
-// How long a thread polls for something it expects within microseconds before
-// it goes to sleep on a condition variable.
-constexpr std::chrono::microseconds kSpinBeforeSleep{60};
+// How long a thread polls for something it expects soon before it goes to sleep
+// on a condition variable: the buckets of a backward pass arrive some tens to
+// hundreds of microseconds apart, and waking a sleeping thread costs the caller
+// a system call and the operation 20 to 30 microseconds.
+constexpr int64_t kDefaultSpinMicros = 200;
+
+// FAIRRING_SPIN_US overrides it (0: sleep at once), read once.
+std::chrono::microseconds spinBeforeSleep() {
+  static const std::chrono::microseconds v = [] {
+    const char* e = std::getenv("FAIRRING_SPIN_US");
+    const long long us = e != nullptr ? std::atoll(e) : kDefaultSpinMicros;
+    return std::chrono::microseconds(us < 0 ? 0 : (us > 100000 ? 100000 : us));
+  }();
+  return v;
+}
 
 inline void cpuRelax() {
 #if defined(__x86_64__) || defined(__i386__)
@@ -70,11 +82,11 @@ inline void cpuRelax() {
 #endif
 }
 
-// Polls `ready` for at most kSpinBeforeSleep; true as soon as it holds.
+// Polls `ready` for at most spinBeforeSleep(); true as soon as it holds.
 template <typename F>
 bool spinFor(F&& ready) {
   if (ready()) return true;
-  const auto until = std::chrono::steady_clock::now() + kSpinBeforeSleep;
+  const auto until = std::chrono::steady_clock::now() + spinBeforeSleep();
   for (;;) {
     for (int i = 0; i < 32; ++i) {
       if (ready()) return true;
@@ -803,7 +815,18 @@ void Context::orderAfterConflicts(const OpSpans& op, const std::vector<size_t>& 
           break;
         }
       }
-      if (hit) joinTail(s, t);
+      if (!hit) continue;
+      // What has already finished orders nothing: a stream that has drained is
+      // behind everything and its history can go (a host-side question to the
+      // runtime, asked only on a conflict; a join costs an event packet on
+      // either stream).
+      if (hipStreamQuery(reduceStreams_[s]) == hipSuccess) {
+        for (size_t u = 0; u < n; ++u) orderedAfter_[u][s] = history_[s].back().seq;
+        history_[s].clear();
+        break;
+      }
+      (void)hipGetLastError();
+      joinTail(s, t);
     }
   }
 }

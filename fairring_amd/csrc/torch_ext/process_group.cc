@@ -150,7 +150,12 @@ void ProcessGroupFairring::WorkFairring::awaitCompletion() {
   // short while before sleeping on the future (a sleeping thread takes tens of
   // microseconds to wake).
   {
-    const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(60);
+    static const long long spinMicros = [] {
+      const char* e = std::getenv("FAIRRING_SPIN_US");
+      const long long us = e != nullptr ? std::atoll(e) : 200;
+      return us < 0 ? 0ll : (us > 100000 ? 100000ll : us);
+    }();
+    const auto until = std::chrono::steady_clock::now() + std::chrono::microseconds(spinMicros);
     while (!future_->completed() && std::chrono::steady_clock::now() < until) {
 #if defined(__x86_64__)
       __builtin_ia32_pause();
@@ -311,8 +316,46 @@ void ProcessGroupFairring::recordOnPipelineStreams(
 }
 
 void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor> peers) {
-  std::lock_guard<std::mutex> g(mutex_);
-  peers_ = std::move(peers);
+  // Checked and flattened here, once, rather than by every operation that uses them.
+  bool fromHost = false;
+  for (size_t i = 0; i < peers.size(); ++i) {
+    at::Tensor& p = peers[i];
+    TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense(),
+                "fairring: peer contribution must be dense");
+    if (i == 0) fromHost = !p.is_cuda();
+    TORCH_CHECK(fromHost == !p.is_cuda(), "fairring: peers must be all on the GPU or all pinned");
+    if (fromHost) {
+      TORCH_CHECK(p.is_pinned(), "fairring: host-side peer contributions must be pinned");
+    }
+    p = viewAsFlat(p);
+  }
+  std::vector<at::Tensor> old;
+  bool drainFirst = false;
+  {
+    std::lock_guard<std::mutex> g(mutex_);
+    // pinned tensors cannot be recorded on a stream: what may still be copied
+    // from them is waited for before they go
+    drainFirst = peersUsed_ && peersFromHost_ && !peers_.empty();
+  }
+  if (drainFirst) synchronizeAll();
+  {
+    std::lock_guard<std::mutex> g(mutex_);
+    old.swap(peers_);
+    peers_ = std::move(peers);
+    peersFromHost_ = fromHost;
+    // The group holds its peers' tensors for as long as they are in use, so an
+    // operation does not record them on the pipeline's streams; the ones that
+    // go now may still be read by operations in flight, and are recorded here.
+    if (peersUsed_) {
+      for (const at::Tensor& t : old) {
+        if (!t.is_cuda()) continue;
+        auto it = streams_.find(t.device().index());
+        if (it == streams_.end()) continue;
+        for (const c10::Stream& st : it->second) t.record_stream(st);
+      }
+    }
+    peersUsed_ = false;
+  }
 }
 
 void ProcessGroupFairring::setFusedDivide(bool on) {
@@ -447,55 +490,53 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
   const int rank = getRank();
   const int64_t n = out.numel();
   const int64_t elsize = out.element_size();
-  std::vector<int64_t> peerOffsets;
-  std::vector<at::Tensor> peers = peers_;
+  const std::vector<at::Tensor>& peers = peers_;  // checked and flattened when they were set
   TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
               "fairring: this build runs on one GPU without a transport; a group of size ",
               size, " needs ", size - 1, " simulated peer contributions, got ", peers.size());
-  bool fromHost = false;
-  for (size_t i = 0; i < peers.size(); ++i) {
-    at::Tensor& p = peers[i];
-    TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense(),
-                "fairring: peer contribution must be dense");
-    TORCH_CHECK(p.scalar_type() == out.scalar_type() &&
-                    (p.numel() == n || p.numel() == peerNumel),
-                "fairring: peer contribution must match the operation's dtype and hold ", n,
-                " or ", peerNumel, " elements, got ", p.numel());
-    // a whole flat input: the chunk meant for this rank; otherwise just that chunk
-    peerOffsets.push_back(p.numel() == n ? 0 : n * rank);
-    p = viewAsFlat(p);
-    if (i == 0) fromHost = !p.is_cuda();
-    TORCH_CHECK(fromHost == !p.is_cuda(), "fairring: peers must be all on the GPU or all pinned");
-    if (fromHost) {
-      // Switched off by default: one run of this path through the process group
-      // (pinned peers, 2 staging slots, completion through the future) stopped
-      // making progress on an MI355X and no cause has been found. The same
-      // staging through the C ABI (frg_allreduce_host) is unaffected.
-      static const bool allowed = std::getenv("FAIRRING_PINNED_PEERS") != nullptr;
-      TORCH_CHECK(allowed, "fairring: peer contributions in pinned host memory are switched off "
-                           "in the process group (set FAIRRING_PINNED_PEERS=1 to enable them); "
-                           "hand them in as GPU tensors, or use frg_allreduce_host");
-      TORCH_CHECK(p.is_pinned(), "fairring: host-side peer contributions must be pinned");
-    } else {
-      TORCH_CHECK(p.device() == out.device(), "fairring: peer contribution on another device");
-    }
+  const bool fromHost = !peers.empty() && peersFromHost_;
+  if (fromHost) {
+    // Switched off by default: one run of this path through the process group
+    // (pinned peers, 2 staging slots, completion through the future) stopped
+    // making progress on an MI355X and no cause has been found. The same
+    // staging through the C ABI (frg_allreduce_host) is unaffected.
+    static const bool allowed = std::getenv("FAIRRING_PINNED_PEERS") != nullptr;
+    TORCH_CHECK(allowed, "fairring: peer contributions in pinned host memory are switched off "
+                         "in the process group (set FAIRRING_PINNED_PEERS=1 to enable them); "
+                         "hand them in as GPU tensors, or use frg_allreduce_host");
   }
+  const at::ScalarType outType = out.scalar_type();
+  const int64_t rankOffset = n * rank;
+  for (const at::Tensor& p : peers) {
+    const int64_t pn = p.numel();
+    TORCH_CHECK(p.scalar_type() == outType && (pn == n || pn == peerNumel),
+                "fairring: peer contribution must match the operation's dtype and hold ", n,
+                " or ", peerNumel, " elements, got ", pn);
+    TORCH_CHECK(fromHost || p.device() == out.device(),
+                "fairring: peer contribution on another device");
+  }
+  peersUsed_ = true;
 
   // Contribution table in rank order, this rank's own chunk at its index.
   const char* ownPtr = static_cast<const char*>(own.data_ptr()) + chunkOffset * elsize;
   std::vector<const void*> table;
   table.reserve(size);
   for (int r = 0, pi = 0; r < size; ++r) {
-    table.push_back(r == rank ? static_cast<const void*>(ownPtr)
-                              : static_cast<const char*>(peers[pi].data_ptr()) +
-                                    peerOffsets[pi] * elsize);
-    if (r != rank) ++pi;
+    if (r == rank) {
+      table.push_back(ownPtr);
+      continue;
+    }
+    // a whole flat input: the chunk meant for this rank; otherwise just that chunk
+    const at::Tensor& p = peers[pi++];
+    table.push_back(static_cast<const char*>(p.data_ptr()) +
+                    (p.numel() == n ? 0 : rankOffset) * elsize);
   }
 
+  // the caller's tensors; the peers' are held by the group (setSimulatedPeerContributions)
   if (own.data_ptr() == out.data_ptr()) {  // in place: one storage
-    recordOnPipelineStreams(device, fromHost, {&out}, fromHost ? nullptr : &peers);
+    recordOnPipelineStreams(device, fromHost, {&out}, nullptr);
   } else {
-    recordOnPipelineStreams(device, fromHost, {&out, &own}, fromHost ? nullptr : &peers);
+    recordOnPipelineStreams(device, fromHost, {&out, &own}, nullptr);
   }
 
   auto future = c10::make_intrusive<c10::ivalue::Future>(
@@ -530,7 +571,6 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
 
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
   keepAlive.push_back(own);
-  for (at::Tensor& p : peers) keepAlive.push_back(p);
   auto* pending = new Pending{future, out, std::move(keepAlive), device};
   int rc;
   if (fromHost) {
@@ -637,30 +677,29 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
   const int size = getSize();
   const int rank = getRank();
   const int64_t n = t.numel();
-  std::vector<at::Tensor> peers = peers_;
+  const std::vector<at::Tensor>& peers = peers_;
   TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
               "fairring: this build runs on one GPU without a transport; a group of size ",
               size, " needs ", size - 1, " simulated peer contributions, got ", peers.size());
-  for (at::Tensor& p : peers) {
-    TORCH_CHECK(p.layout() == at::kStrided && p.is_non_overlapping_and_dense() && p.is_cuda() &&
-                    p.device() == t.device(),
+  for (const at::Tensor& p : peers) {
+    TORCH_CHECK(p.is_cuda() && p.device() == t.device(),
                 "fairring: a compressed peer contribution must be a dense tensor on the bucket's "
                 "device");
     TORCH_CHECK(p.scalar_type() == wire && p.numel() == n,
                 "fairring: a compressed peer contribution must hold ", n, " elements of ", wire);
-    p = viewAsFlat(p);
   }
+  peersUsed_ = true;
   std::vector<const void*> table;
   table.reserve(size);
   for (int r = 0, pi = 0; r < size; ++r) {
     table.push_back(r == rank ? t.data_ptr() : peers[pi].data_ptr());
     if (r != rank) ++pi;
   }
-  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&t}, &peers);
+  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&t}, nullptr);
   auto future = c10::make_intrusive<c10::ivalue::Future>(
       c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
-  auto* pending = new Pending{future, t, std::move(peers), device};
+  auto* pending = new Pending{future, t, {}, device};
   // buffer.to(wire).div_(size): on the GPU a multiply by the reciprocal, in
   // the wire type's arithmetic
   const int rc = frg_allreduce_compressed(

@@ -179,7 +179,9 @@ class ProcessGroupFairring : public c10d::Backend {
   void recordOnPipelineStreams(c10::DeviceIndex device, bool copyStreamsToo,
                                std::initializer_list<const at::Tensor*> tensors,
                                const std::vector<at::Tensor>* more);
-  std::vector<at::Tensor> peers_;
+  std::vector<at::Tensor> peers_;     // flat views, checked when they were set
+  bool peersFromHost_ = false;
+  bool peersUsed_ = false;             // by an operation since they were set
   bool fusedDivide_ = false;
 };
 
