@@ -17,7 +17,7 @@ SCALE_PRE_MUL, SCALE_PRE_DIV = 3, 4
 
 # every symbol include/fairring_hip.h declares
 EXPORTS = (
-    "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_plan_launches", "frg_reduce_slice",
+    "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_plan_launches", "frg_reduce_slice", "frg_reduce_slice_static",
     "frg_reduce_slice_compressed", "frg_allreduce_compressed",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
@@ -87,6 +87,7 @@ def lib():
                                     ctypes.POINTER(i64),
                                     ctypes.POINTER(ctypes.c_int32), i32, ctypes.POINTER(i32)]
     L.frg_reduce_slice.argtypes = [vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp]
+    L.frg_reduce_slice_static.argtypes = [vp, pvp, i32, i64, i32, i32, i32, f32, vp]
     L.frg_create.argtypes = [i32, ctypes.POINTER(Options), pvp]
     L.frg_destroy.argtypes = [vp]
     L.frg_get_layout.argtypes = [vp, ctypes.POINTER(Layout)]

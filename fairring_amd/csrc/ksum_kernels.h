@@ -44,6 +44,19 @@ struct ReduceArgs {
   hipEvent_t stopEvent = nullptr;
 };
 
+// Where inside a scratch region a chain of launches parks its partial result so
+// that the vector variant of the kernel still runs: at the same position within
+// 16 bytes as `like` for a buffer of the storage type, or, for fp32 accumulators
+// of a 2-byte type (`acc`), such that it reaches a 16-byte boundary after as
+// many elements as `like` does. `base` is 16-byte aligned and the region has 16
+// bytes to spare.
+inline char* placeInScratch(char* base, const void* like, bool acc, int64_t elsize) {
+  const uintptr_t pos = reinterpret_cast<uintptr_t>(like) & 15;
+  if (!acc) return base + pos;
+  const uintptr_t headElems = ((16 - pos) & 15) / static_cast<uintptr_t>(elsize);
+  return base + ((16 - (4 * headElems) % 16) % 16);
+}
+
 // Validates the arguments, picks the kernel variant that fits K and the
 // pointers' alignment, and enqueues one launch on `stream`. Returns an FRG_*
 // status; on failure `err` says why. Never synchronises.

@@ -280,6 +280,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
       c->slotFilledEvents_.push_back(b);
     }
     c->slotUsed_.assign(static_cast<size_t>(c->numSlots_), 0);
+    prepareStaticScratch(device);  // for frg_reduce_slice_static; failures are left to that call
     c->streamLaunches_.assign(c->reduceStreams_.size(), 0);
     c->streamElems_.assign(c->reduceStreams_.size(), 0);
     c->history_.resize(c->reduceStreams_.size());
@@ -689,10 +690,7 @@ void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
 // 16-byte boundary after as many elements as `like` does.
 char* Context::scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize) {
   char* base = carryScratch_ + streamIdx * static_cast<size_t>(carryScratchBytes_ + 16);
-  const uintptr_t pos = reinterpret_cast<uintptr_t>(like) & 15;
-  if (!acc) return base + pos;
-  const uintptr_t headElems = ((16 - pos) & 15) / static_cast<uintptr_t>(elsize);
-  return base + ((16 - (4 * headElems) % 16) % 16);
+  return placeInScratch(base, like, acc, elsize);
 }
 
 // One part of a slice with more contributions than a launch takes, chained

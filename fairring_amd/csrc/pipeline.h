@@ -255,6 +255,10 @@ class Context {
   std::thread thread_;
 };
 
+// Looks up the static scratch of frg_reduce_slice_static on `device` ahead of
+// the first call (static_scratch.hip).
+void prepareStaticScratch(int device);
+
 // Process-wide limit of frg_work_wait in seconds (0: none).
 void setWaitTimeout(double seconds);
 

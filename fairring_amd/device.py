@@ -116,6 +116,21 @@ def reduce_slice(out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, carry=
         scale, 1 if carry else 0, stream.cuda_stream))
 
 
+def reduce_slice_static(out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+    """reduce_slice for any number of contributions without any allocation
+    (frg_reduce_slice_static): chains of more than 64 park their partial result
+    in the library's static device array."""
+    import torch
+    stream = torch.cuda.current_stream(out.device) if stream is None else stream
+    for c in contribs:
+        if c.numel() != out.numel() or c.dtype != out.dtype:
+            raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+    tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+    _capi.check(_capi.lib().frg_reduce_slice_static(
+        out.data_ptr(), tab, len(contribs), out.numel(), _dtype_code(out), op, scale_mode, scale,
+        stream.cuda_stream))
+
+
 def _check_compressed(out, contribs, raw_index):
     """Shapes and types of the reduction with compression folded in; returns
     the wire dtype code."""

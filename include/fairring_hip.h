@@ -148,6 +148,34 @@ FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);
 
+/* No counterpart in the reference. frg_reduce_slice for any number of
+ * contributions, for callers that cannot allocate: a stream that is being
+ * captured into a HIP graph, a tight serving loop, a harness that forbids
+ * hipMalloc. More than 64 contributions are folded by a chain of launches on
+ * `stream` with the result of one fold over all of them, as frg_allreduce gives
+ * (one rounding for bf16 / fp16, whose partial sums travel as fp32; exact also
+ * when `out` is one of the later contributions). Where frg_allreduce parks the
+ * partial result of such a chain in a scratch buffer that its context
+ * allocates, this call parks it in an array that is part of the library's
+ * device code (FRG_STATIC_SCRATCH_BYTES per GPU, there for the life of the
+ * process), so the call allocates nothing, creates no event and no stream, and
+ * clears no memory. A chain that needs the array (a bf16 / fp16 SUM, or `out`
+ * among contributions 64 and up) is limited to what it holds:
+ * FRG_STATIC_SCRATCH_BYTES / 4 elements for the fp32 accumulators of a 2-byte
+ * type, FRG_STATIC_SCRATCH_BYTES / element size otherwise; beyond that, and
+ * beyond FRG_STATIC_MAX_CONTRIBUTIONS, the call fails with FRG_ERR_INVALID and
+ * says so. Everything else (up to 64 contributions; chains of fp32, fp64,
+ * integers or MAX, which carry their exact partial result in `out`) takes any
+ * size. All calls on one GPU share that GPU's array: two of them that overlap
+ * in time (different streams, or two graphs replayed at once) race on it; calls
+ * on one stream do not. The array's address is looked up on the first call on a
+ * device (frg_create does it for its device beforehand). */
+#define FRG_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+#define FRG_STATIC_MAX_CONTRIBUTIONS 4096
+FRG_API int frg_reduce_slice_static(void* out, const void* const* contribs, int K,
+                                    int64_t n, int dtype, int op, int scale_mode,
+                                    float scale, void* stream);
+
 /* The same reduction with torch's gradient-compression hooks folded in
  * (bf16_compress_hook / fp16_compress_hook,
  * torch:distributed/algorithms/ddp_comm_hooks/default_hooks.py:57-134, wrapped

@@ -41,6 +41,8 @@ void setTuning(int) {}
 
 int computeUnits(int) { return 4; }  // what the stand-in runtime reports
 
+void prepareStaticScratch(int) {}  // device code: not part of the host build
+
 namespace {
 
 struct Job {

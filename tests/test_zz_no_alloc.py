@@ -1,0 +1,94 @@
+"""frg_reduce_slice_static: the entry point that allocates nothing, against
+frg_allreduce, whose context allocates the scratch buffer of the same chains.
+Bit-exact; two calls in a row, the second one smaller."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+fa = pytest.importorskip("fairring_amd")
+from fairring_amd import _capi  # noqa: E402
+
+DEV = "cuda:0"
+MiB = 1024 * 1024
+
+
+def bits16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def test_static_scratch_chain_matches_the_pipeline_on_two_calls_in_a_row():
+    print("[case] no-alloc entry point, bf16 K = 100, two sizes", flush=True)
+    k = 100
+    g = torch.Generator(device=DEV)
+    g.manual_seed(71)
+    dev = fa.DeviceFairring(0)
+    try:
+        for n in (1_000_003, 70_001):          # the second call is the smaller one
+            xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g).to(torch.bfloat16)
+                  for _ in range(k)]
+            want = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+            dev.allreduce(want, xs, scale_mode=fa.SCALE_DIV, scale=float(k)).wait()
+            got = torch.full((n,), 7.0, dtype=torch.bfloat16, device=DEV)
+            fa.reduce_slice_static(got, xs, scale_mode=fa.SCALE_DIV, scale=float(k))
+            torch.cuda.synchronize()
+            assert_bits_equal(bits16(got), bits16(want), "n = %d" % n)
+            # and both against the oracle (one rounding at the end of the chain)
+            host = [bits16(x) for x in xs]
+            assert_bits_equal(bits16(got), oracle.sum_bf16(host, oracle.SCALE_DIV, float(k),
+                                                           threads=8), "oracle, n = %d" % n)
+    finally:
+        dev.close()
+
+
+def test_static_scratch_in_place_into_a_late_contribution_and_plain_cases():
+    print("[case] no-alloc entry point, fp32 in place at rank 80; K <= 64; fp32 chain", flush=True)
+    k, n = 100, 300_007
+    g = torch.Generator(device=DEV)
+    g.manual_seed(72)
+    dev = fa.DeviceFairring(0)
+    try:
+        xs = [torch.empty(n, device=DEV).normal_(0, 1.0, generator=g) for _ in range(k)]
+        want = torch.empty(n, device=DEV)
+        dev.allreduce(want, xs).wait()
+        target = xs[80]                        # read only by the second launch of the chain
+        fa.reduce_slice_static(target, xs)
+        torch.cuda.synchronize()
+        assert_bits_equal(target.cpu().numpy(), want.cpu().numpy(), "in place at rank 80")
+        # a chain that carries its partial result in `out` (fp32, separate output): any size
+        xs[80] = torch.empty(n, device=DEV).normal_(0, 1.0, generator=g)
+        dev.allreduce(want, xs, scale_mode=fa.SCALE_MUL, scale=0.01).wait()
+        got = torch.empty(n, device=DEV)
+        fa.reduce_slice_static(got, xs, scale_mode=fa.SCALE_MUL, scale=0.01)
+        torch.cuda.synchronize()
+        assert_bits_equal(got.cpu().numpy(), want.cpu().numpy(), "fp32 chain")
+        # up to 64 contributions it is frg_reduce_slice
+        fa.reduce_slice_static(got, xs[:8], op=fa.MAX)
+        fa.reduce_slice(want, xs[:8], op=fa.MAX)
+        torch.cuda.synchronize()
+        assert_bits_equal(got.cpu().numpy(), want.cpu().numpy(), "K = 8 max")
+    finally:
+        dev.close()
+
+
+def test_static_scratch_rejects_what_it_cannot_hold():
+    print("[case] no-alloc entry point, limits", flush=True)
+    cap = 8 * MiB // 4                         # fp32 accumulators of a 2-byte type
+    n = cap + 1
+    x = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(fa.FairringError) as e:
+        fa.reduce_slice_static(out, [x] * 65)
+    assert e.value.code == _capi.ERR_INVALID and "at most %d elements" % cap in str(e.value)
+    fa.reduce_slice_static(out[:cap], [x[:cap]] * 65)       # exactly what it holds
+    fa.reduce_slice_static(out, [x] * 64)                   # one launch: no scratch, any size
+    f = torch.zeros(3 * cap, device=DEV)
+    fa.reduce_slice_static(torch.empty_like(f), [f] * 65)   # fp32 carries in `out`: any size
+    torch.cuda.synchronize()
+    with pytest.raises(fa.FairringError) as e:
+        fa.reduce_slice_static(out[:16], [x[:16]] * 4097)
+    assert e.value.code == _capi.ERR_INVALID and "4096" in str(e.value)
