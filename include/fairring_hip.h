@@ -213,24 +213,26 @@ typedef struct frg_options {
   int64_t max_launch_bytes;               /* bytes of one contribution that a single reduction
                                              launch covers: device-resident tensors are cut into
                                              launches of this size on 4 KiB boundaries (the last
-                                             one up to 1.5 times as long), dealt round-robin to the
-                                             reduce streams. 0 = default: size and grid chosen
-                                             together (whole rounds of a 4-blocks-per-CU grid,
-                                             about 80 MB per launch, for operations of at least
-                                             100 MiB per contribution and for more than 8
-                                             contributions; 12.5 MiB for smaller operations of
-                                             3 to 8; 48 MiB for fewer), < 0 = one launch per
-                                             slice */
+                                             one up to 1.5 times as long). 0 = default: the
+                                             library's own partition (frg_plan_launches: from 4
+                                             contributions on, whole rounds of a 4-blocks-per-CU
+                                             grid placed on the 4 MiB multiples of the output's
+                                             allocation, about 80 MB per launch), < 0 = one launch
+                                             per slice */
 } frg_options;
 
 /* DeviceFairring ctor: fairring/device.cc:213-284 (streams, staging pool,
  * per-slot events, command thread). No padding pool: ragged tails are handled
- * inside the kernel. */
+ * inside the kernel. The streams come from a pool that lives as long as the
+ * process: a context created after another one was destroyed runs on that
+ * one's streams. Every device allocation a context ever makes (staging pool,
+ * chain scratch) is made here. */
 FRG_API int frg_create(int device, const frg_options* opts, frg_ctx** out);
 
 /* DeviceFairring dtor: fairring/device.cc:286-289 (drain the command queue,
- * join the thread). Streams are deliberately leaked, as machine.cc:162-175
- * requires for streams that consumers may still hold events on. */
+ * join the thread). Streams are never destroyed, as machine.cc:162-175
+ * requires for streams that consumers may still hold events on: they go back
+ * to the process's pool. */
 FRG_API int frg_destroy(frg_ctx* ctx);
 
 /* The layout in force (slice size, number of staging slots). */
@@ -262,9 +264,9 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
  * Device-resident contributions: `contribs[k]` are device pointers to `numel`
  * elements each. The slices of the layout only count here (they advance the
  * slot cursor): resident contributions need no slot, so the tensor is reduced
- * by launches of frg_options.max_launch_bytes per contribution, cut on 4 KiB
- * boundaries from its start, whatever the slice size (max_launch_bytes < 0:
- * one launch per slice). An operation of up to 8 launches (a DDP bucket) runs
+ * by launches cut as frg_options.max_launch_bytes says (by default the
+ * partition of frg_plan_launches), whatever the slice size (max_launch_bytes
+ * < 0: one launch per slice). An operation of up to 8 launches (a DDP bucket) runs
  * on one reduce stream and the next operation on the next one; a longer one
  * deals its launches over all reduce streams. Operations are ordered as on one
  * stream wherever that can be observed: one that writes memory an earlier
