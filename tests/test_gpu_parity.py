@@ -744,3 +744,105 @@ def test_max_against_amax_on_the_gpu(tdt):
             assert bool(strict.all()), "%s K=%d bits" % (tdt, k)
         else:
             assert bool(torch.equal(out, ref)), "%s K=%d" % (tdt, k)
+
+
+# ---- where the rounds lie: launches placed on the 4 MiB multiples of the output's allocation ----
+
+def _offset_in_allocation(t):
+    """Bytes from the start of the hipMalloc allocation that holds `t` to its first element."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")     # the runtime torch has loaded already
+    base, size = ctypes.c_void_p(), ctypes.c_size_t()
+    rc = hip.hipMemGetAddressRange(ctypes.byref(base), ctypes.byref(size), ctypes.c_void_p(t.data_ptr()))
+    assert rc == 0 and base.value is not None
+    return t.data_ptr() - base.value
+
+
+def _view_at_residue(buf, residue_bytes, n, elsize):
+    """n elements of `buf` whose first byte lies `residue_bytes` past a 4 MiB multiple of the allocation."""
+    off = _offset_in_allocation(buf)
+    start = (residue_bytes - off) % (4 * MiB)
+    assert start % elsize == 0
+    return buf[start // elsize: start // elsize + n]
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+def test_large_operation_at_any_offset_within_its_allocation(kind):
+    # An operation of 16 rounds or more starts its rounds where the output reaches a 4 MiB multiple
+    # of its allocation: the first launch takes up to a whole round ahead of that point as pieces
+    # (the kernel's lead), the last one what lies behind the last whole round. Offsets that leave
+    # nothing, a few vectors, most of a round, and an odd number of elements ahead of the rounds.
+    tdt = torch.float32 if kind == "f32" else torch.bfloat16
+    elsize = 4 if kind == "f32" else 2
+    k, n = 4, 100 * MiB // elsize + 12345
+    g = torch.Generator(device=DEV)
+    g.manual_seed(81)
+    room = n + 8 * MiB // elsize
+    bufs = [torch.empty(room, device=DEV).normal_(0, 0.01, generator=g).to(tdt) for _ in range(k)]
+    outbuf = torch.zeros(room, dtype=tdt, device=DEV)
+    dev = fa.DeviceFairring(0)
+    try:
+        for residue in (0, 2560, 1 * MiB + 4 * elsize, 2 * MiB, 3 * MiB + 2560, 4 * MiB - 16):
+            _print_case("large operation", kind, "residue", residue)
+            xs = [_view_at_residue(b, residue, n, elsize) for b in bufs]
+            out = _view_at_residue(outbuf, residue, n, elsize)
+            outbuf.zero_()
+            before = dev.progress()["launches"]
+            dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=0.25).wait()
+            plan = fa.plan_launches(k, n, elsize, xs[0].data_ptr(), _offset_in_allocation(out))
+            assert dev.progress()["launches"] - before == len(plan) >= 6
+            assert all(b == 4 for _, b in plan)
+            chain = xs[0].to(torch.float32, copy=True)   # (.float() of an fp32 tensor is the tensor)
+            for x in xs[1:]:
+                chain.add_(x.float())
+            chain.mul_(0.25)
+            want = chain.to(tdt)
+            it = torch.int32 if kind == "f32" else torch.int16
+            assert bool(torch.equal(out.view(it), want.view(it))), residue
+            # nothing outside the view was written
+            lo = out.data_ptr() - outbuf.data_ptr()
+            assert int(torch.count_nonzero(outbuf)) == int(torch.count_nonzero(out))
+            assert lo % elsize == 0
+            # and the oracle on the range around the end of the first launch's lead and rounds
+            first = plan[0][0]
+            a, b = max(0, first - 5000), min(n, first + 5000)
+            if kind == "f32":
+                host = [x[a:b].cpu().numpy() for x in xs]
+                assert_bits_equal(out[a:b].cpu().numpy(), oracle.sum_f32(host, oracle.SCALE_MUL, 0.25))
+            else:
+                host = [bf16_bits(x[a:b]) for x in xs]
+                assert_bits_equal(bf16_bits(out[a:b]), oracle.sum_bf16(host, oracle.SCALE_MUL, 0.25))
+    finally:
+        dev.close()
+
+
+def test_stream_of_buckets_keeps_one_shape_and_switches_only_after_a_run_of_aligned_ones():
+    # short operations are aligned to the 4 MiB multiples only when the four before them could be
+    # too; one that cannot ends the run. 28 MiB buckets: 8 + 8 + 12 MiB aligned, 12.5 + 15.5 otherwise.
+    _print_case("bucket stream: aligned after a run of four")
+    k, n = 8, 28 * MiB // 4
+    g = torch.Generator(device=DEV)
+    g.manual_seed(82)
+    room = n + 2 * MiB
+    bufs = [torch.empty(room, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    outbuf = torch.zeros(12 * room, device=DEV)
+    dev = fa.DeviceFairring(0)
+    try:
+        residues = [0] * 7 + [2 * MiB] + [0] * 6       # the eighth bucket starts 2 MiB off
+        launches = []
+        outs, xss = [], []
+        for i, residue in enumerate(residues):
+            xs = [_view_at_residue(b, residue, n, 4) for b in bufs]
+            out = _view_at_residue(outbuf[(i % 12) * room:], residue, n, 4)
+            before = dev.progress()["launches"]
+            w = dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+            w.wait()
+            launches.append(dev.progress()["launches"] - before)
+            chain = xs[0].clone()
+            for x in xs[1:]:
+                chain.add_(x)
+            chain.mul_(0.125)
+            assert bool(torch.equal(out.view(torch.int32), chain.view(torch.int32))), i
+        assert launches == [2, 2, 2, 2, 3, 3, 3, 2, 2, 2, 2, 2, 3, 3], launches
+    finally:
+        dev.close()
