@@ -167,6 +167,34 @@ def test_group_destroyed_while_python_callbacks_are_pending():
     assert float(own[0]) == 41.0 and float(own[-1]) == 41.0   # 1, plus the peer's 1 forty times
 
 
+def test_result_and_synchronize_wait_without_holding_the_interpreter_lock():
+    # Python's bindings of Work.result() and Work.synchronize() keep the global lock (those of
+    # Work.wait() and Future.wait() let go of it). The completion callback on the command thread
+    # needs that lock here (a Python `then` callback; the last reference to a tensor Python made),
+    # so a wait inside result() that held on to it would stop both threads for good.
+    print("[case] pg result() with Python callbacks pending", flush=True)
+    import warnings
+    n = 1 << 22
+    pg = make_pg(0, 2)
+    seen = []
+    for i in range(20):
+        own = torch.full((n,), float(i), device=DEV)
+        pg._set_simulated_peer_contributions([torch.ones(n, device=DEV)])
+        work = pg.allreduce([own])
+        fut = work.get_future().then(lambda f, i=i: seen.append((i, float(f.value()[0][0]))))
+        del own                                  # the future's value holds the last reference
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            if i % 2:
+                res = work.result()              # binding keeps the lock while it waits
+                assert float(res[0][-1]) == float(i) + 1.0
+            else:
+                work.synchronize()
+        fut.wait()
+    torch.cuda.synchronize()
+    assert seen == [(i, float(i) + 1.0) for i in range(20)]
+
+
 def test_data_moving_collectives_exist_for_a_group_of_one_only():
     print("[case] pg broadcast/allgather/barrier", flush=True)
     pg = make_pg(0, 1)
