@@ -666,6 +666,59 @@ void scenarioOrderBetweenOperations() {
   }
 }
 
+void scenarioRandomDependentOperations() {
+  std::puts("random sequences of operations over shared buffers equal their sequential execution");
+  for (unsigned seed = 0; seed < 6; ++seed) {
+    std::mt19937 rng(7000 + seed);
+    const int nbuf = 4;
+    const int64_t size = 6000;
+    const int streams = 2 + static_cast<int>(seed % 2);
+    frg_ctx* ctx = makeCtx(8192, 4096, streams, seed % 3 == 0 ? 0 : 2048);
+    const std::vector<hipStream_t> ss = streamsOf(ctx);
+    auto bufs = randomContribs(nbuf, size, 8000 + seed);
+    auto shadow = bufs;
+    std::uniform_int_distribution<int> pickBuf(0, nbuf - 1), pickK(2, 5), pickDelay(0, 3);
+    std::vector<std::vector<const void*>> tables;  // kept alive until the operations have run
+    for (int op = 0; op < 60; ++op) {
+      const int64_t n = 200 + static_cast<int64_t>(rng() % 1500);
+      const int ob = pickBuf(rng);
+      const int64_t olo = static_cast<int64_t>(rng() % static_cast<unsigned>(size - n));
+      const int k = pickK(rng);
+      std::vector<std::pair<int, int64_t>> terms;
+      for (int t = 0; t < k; ++t) {
+        if (rng() % 4 == 0) {
+          terms.emplace_back(ob, olo);  // in place
+          continue;
+        }
+        for (;;) {
+          const int cb = pickBuf(rng);
+          const int64_t clo = static_cast<int64_t>(rng() % static_cast<unsigned>(size - n));
+          if (cb != ob || clo + n <= olo || olo + n <= clo) {
+            terms.emplace_back(cb, clo);
+            break;
+          }
+        }
+      }
+      // hold one of the streams up now and then, so that an unordered operation runs too early
+      if (pickDelay(rng) == 0) fake_hip_occupy(ss[rng() % ss.size()], 2);
+      std::vector<const void*> tab;
+      for (auto& t : terms) tab.push_back(bufs[t.first].data() + t.second);
+      tables.push_back(tab);
+      CHECK(frg_allreduce(ctx, bufs[ob].data() + olo, tables.back().data(), k, n, FRG_F32, FRG_SUM,
+                          FRG_SCALE_MUL, 0.5f, nullptr, nullptr, nullptr, nullptr) == FRG_OK);
+      Vec acc(shadow[terms[0].first].begin() + terms[0].second,
+              shadow[terms[0].first].begin() + terms[0].second + n);
+      for (size_t t = 1; t < terms.size(); ++t) {
+        for (int64_t i = 0; i < n; ++i) acc[i] = acc[i] + shadow[terms[t].first][terms[t].second + i];
+      }
+      for (int64_t i = 0; i < n; ++i) shadow[ob][olo + i] = acc[i] * 0.5f;
+    }
+    CHECK(frg_synchronize(ctx) == FRG_OK);
+    for (int b = 0; b < nbuf; ++b) CHECK(same(bufs[b], shadow[b]));
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
 // What the c10d extension does around the ABI, with a mutex standing in for
 // Python's global lock: the caller holds it except inside the calls that let go
 // of it (submitting, waiting); the completion callback, on the command thread,
@@ -987,6 +1040,7 @@ void runAll() {
       {"producer ordering", scenarioProducerOrdering},
       {"streams are reused", scenarioStreamsAreReused},
       {"order between operations", scenarioOrderBetweenOperations},
+      {"random dependent operations", scenarioRandomDependentOperations},
       {"host staged", scenarioHostStaged},
       {"callback", scenarioCallback},
       {"process-group-shaped", scenarioProcessGroupShaped},

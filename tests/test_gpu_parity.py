@@ -846,3 +846,54 @@ def test_stream_of_buckets_keeps_one_shape_and_switches_only_after_a_run_of_alig
         assert launches == [2, 2, 2, 2, 3, 3, 3, 2, 2, 2, 2, 2, 3, 3], launches
     finally:
         dev.close()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_sequences_of_dependent_operations_match_sequential_execution(seed):
+    # Operations over ranges of a few shared buffers, submitted back to back without a wait: every
+    # read-after-write, write-after-read and write-after-write between them must resolve as if they
+    # ran one after the other, whichever reduce streams they land on. Ranges are 1 to 6 MiB, so
+    # neighbouring operations do overlap in time when nothing orders them.
+    _print_case("random dependent operations", seed)
+    rng = np.random.default_rng(9100 + seed)
+    nbuf, size = 5, 6 * MiB // 4 * 3                      # five buffers of 18 MiB
+    g = torch.Generator(device=DEV)
+    g.manual_seed(9100 + seed)
+    bufs = [torch.empty(size, device=DEV).normal_(0, 1.0, generator=g) for _ in range(nbuf)]
+    shadow = [b.clone() for b in bufs]                    # the sequential execution, by torch
+    streams = int(rng.choice([2, 3]))
+    dev = fa.DeviceFairring(0, num_reduce_streams=streams)
+    torch.cuda.synchronize()
+    try:
+        works = []
+        for _ in range(50):
+            n = int(rng.integers(MiB // 4, 6 * MiB // 4))
+            ob = int(rng.integers(nbuf))
+            olo = int(rng.integers(0, size - n)) // 4 * 4
+            k = int(rng.integers(2, 6))
+            terms = []
+            for _ in range(k):
+                if rng.random() < 0.25:
+                    terms.append((ob, olo))               # in place: the output's own range
+                    continue
+                while True:
+                    cb = int(rng.integers(nbuf))
+                    clo = int(rng.integers(0, size - n)) // 4 * 4
+                    if cb != ob or clo + n <= olo or olo + n <= clo:   # no partial overlap with `out`
+                        break
+                terms.append((cb, clo))
+            scale = float(rng.choice([0.5, 0.25, 1.0, 2.0]))
+            out = bufs[ob][olo:olo + n]
+            works.append(dev.allreduce(out, [bufs[b][lo:lo + n] for b, lo in terms],
+                                       scale_mode=fa.SCALE_MUL, scale=scale))
+            acc = shadow[terms[0][0]][terms[0][1]:terms[0][1] + n].clone()
+            for b, lo in terms[1:]:
+                acc.add_(shadow[b][lo:lo + n])
+            acc.mul_(scale)
+            shadow[ob][olo:olo + n] = acc
+        for w in works:
+            w.wait()
+        for i in range(nbuf):
+            assert bool(torch.equal(bufs[i].view(torch.int32), shadow[i].view(torch.int32))), i
+    finally:
+        dev.close()
