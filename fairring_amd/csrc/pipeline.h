@@ -209,7 +209,7 @@ class Context {
   std::mutex copyMu_;  // guards the creation of copyStreams_
 
   char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
-  // Allocated on first use, one region per reduce stream: carries the partial
+  // Allocated with the context, one region per reduce stream: carries the partial
   // result of a chain of launches that must not, or not yet, land in `out`
   // (reduced in place into a late contribution; bf16 / fp16 sums, kept in fp32).
   // 8 MiB per stream by default: with 1 MiB a 100-way bf16 sum ran at 2.4 TB/s

@@ -137,3 +137,13 @@ def test_hook_entry_points_exist_and_refuse_other_backends():
                  ddp_comm_hooks.fp16_compress_hook):
         with pytest.raises(RuntimeError, match="'fairring' backend"):
             hook(object(), Bucket())
+
+
+def test_simulated_peers_are_checked_when_they_are_set():
+    # the peers' tensors are validated and flattened once, by the setter, not by every operation
+    pg = make_pg(0, 3)
+    with pytest.raises(RuntimeError, match="dense"):
+        pg._set_simulated_peer_contributions([torch.zeros(8)[::2], torch.zeros(4)])
+    with pytest.raises(RuntimeError, match="pinned"):
+        pg._set_simulated_peer_contributions([torch.zeros(4), torch.zeros(4)])   # pageable memory
+    pg._set_simulated_peer_contributions([])                                      # clears them
