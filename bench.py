@@ -807,10 +807,14 @@ def main():
             try:
                 r = measure(sub, name, np, torch, fa, oracle,
                             shared=shared if name in ("c5", "c5pg") else None)
-                extra[name] = {key: r[key] for key in ("metric", "value", "unit", "steps",
-                                                       "ms_per_step", "dtype", "pct_of_hbm_peak",
-                                                       "parity", "roofline")}
-                extra[name]["workload"] = r["config"]["workload"]
+                # compact: the whole record stays one line of a few KB
+                roof = {key: r["roofline"][key] for key in (
+                    "bound", "achieved", "peak", "unit", "frac", "traffic", "launch_bytes",
+                    "avg_launch_us", "concurrency", "kernel") if key in r["roofline"]}
+                extra[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"],
+                               "steps": r["steps"], "ms_per_step": r["ms_per_step"],
+                               "dtype": r["dtype"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
+                               "parity": r["parity"].split(";")[0], "roofline": roof}
                 if "host_link_GBps" in r["config"]:
                     extra[name]["host_link_GBps"] = r["config"]["host_link_GBps"]
             except (SystemExit, Exception) as e:  # noqa: BLE001  (reported, and the run fails)
