@@ -297,6 +297,7 @@ int frg_get_progress(frg_ctx* ctx, frg_progress* out) {
   out->started = p.started.load();
   out->enqueued = p.enqueued.load();
   out->launches = p.launches.load();
+  out->on_callers_stream = p.onCallersStream.load();
   return FRG_OK;
 }
 

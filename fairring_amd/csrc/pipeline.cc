@@ -188,6 +188,47 @@ StreamPool& streamPool() {
   return *pool;
 }
 
+// Events for a caller's stream to wait on an operation (frg_work_block_stream):
+// kept per device and never destroyed, since a work handle may outlive its
+// context and creating and destroying an event per wait costs more than the
+// record and the wait themselves. An event goes back as soon as the wait on it
+// is enqueued: the wait holds what it needs of the record.
+class WaitEventPool {
+ public:
+  hipEvent_t take(int device) {
+    {
+      std::lock_guard<std::mutex> g(mu_);
+      for (size_t i = 0; i < idle_.size(); ++i) {
+        if (idle_[i].device != device) continue;
+        hipEvent_t e = idle_[i].event;
+        idle_[i] = idle_.back();
+        idle_.pop_back();
+        return e;
+      }
+    }
+    hipEvent_t e;
+    FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    return e;
+  }
+  void give(int device, hipEvent_t e) {
+    std::lock_guard<std::mutex> g(mu_);
+    idle_.push_back(Entry{e, device});
+  }
+
+ private:
+  struct Entry {
+    hipEvent_t event;
+    int device;
+  };
+  std::mutex mu_;
+  std::vector<Entry> idle_;
+};
+
+WaitEventPool& waitEventPool() {
+  static WaitEventPool* pool = new WaitEventPool();
+  return *pool;
+}
+
 }  // namespace
 
 int Context::create(int device, const frg_options& o, Context** out, std::string* err) {
@@ -244,6 +285,10 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
   if (const char* v = std::getenv("FAIRRING_IDLE_PRODUCER_CHECK")) {
     c->idleProducerCheck_ = std::atoi(v) != 0;
+  }
+  if (const char* v = std::getenv("FAIRRING_INLINE_BYTES")) {
+    const long long b = std::atoll(v);
+    if (b >= 0) c->inlineTrafficBytes_ = b;
   }
   if (const char* v = std::getenv("FAIRRING_ONE_STREAM_LAUNCHES")) {
     const long long m = std::atoll(v);
@@ -317,6 +362,10 @@ Context::~Context() {
   (void)hipSetDevice(device_);
   for (hipStream_t s : reduceStreams_) (void)hipStreamSynchronize(s);
   for (hipStream_t s : copyStreams_) (void)hipStreamSynchronize(s);
+  if (inlinePending_) {
+    (void)(inlineRecorded_ ? hipEventSynchronize(inlineEvent_) : hipStreamSynchronize(nullptr));
+  }
+  if (inlineEvent_ != nullptr) (void)hipEventDestroy(inlineEvent_);
   if (stagingPool_) (void)hipFree(stagingPool_);
   if (carryScratch_) (void)hipFree(carryScratch_);
   for (hipEvent_t e : slotFreeEvents_) (void)hipEventDestroy(e);
@@ -472,6 +521,8 @@ int Context::waitWork(Work* w, std::string* err) {
 
 int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
   const double limit = waitTimeoutSeconds();
+  // a small operation is enqueued within microseconds: poll before sleeping
+  spinFor([&] { return w->enqueuedFlag.load(std::memory_order_acquire); });
   {
     std::unique_lock<std::mutex> lock(w->mu);
     if (limit > 0.0) {
@@ -495,20 +546,143 @@ int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
   }
   try {
     DeviceGuard g(w->device);
-    for (hipStream_t s : w->doneStreams) {
+    Progress& p = *w->progress;
+    for (size_t i = 0; i < w->doneStreams.size(); ++i) {
+      hipStream_t s = w->doneStreams[i];
       if (s == stream) continue;
-      hipEvent_t e;
-      FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      const int idx = i < w->doneIndices.size() ? w->doneIndices[i] : -1;
+      // The event goes behind whatever the stream holds now, this operation
+      // included. The null stream remembers how far that is.
+      const bool remember = stream == nullptr && idx >= 0 && idx < Progress::kMaxStreams;
+      std::unique_lock<std::mutex> known(p.nullWaitMu, std::defer_lock);
+      int64_t upTo = 0;
+      if (remember) {
+        known.lock();
+        if (w->donePositions[i] <= p.nullStreamWaitsFor[idx]) continue;
+        upTo = p.streamPosition[idx].load(std::memory_order_acquire);
+      }
+      hipEvent_t e = waitEventPool().take(w->device);
       hipError_t r = hipEventRecord(e, s);
       if (r == hipSuccess) r = hipStreamWaitEvent(stream, e, 0);
-      (void)hipEventDestroy(e);  // released once the recorded work has passed
+      waitEventPool().give(w->device, e);
       FRG_HIP_CHECK(r);
+      if (remember && upTo > p.nullStreamWaitsFor[idx]) p.nullStreamWaitsFor[idx] = upTo;
     }
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;
   }
   return FRG_OK;
+}
+
+// What was launched on a caller's stream is ahead of whatever comes from the
+// same stream (it takes the producer's event, or finds that stream drained).
+// Coming from another stream, the producer waits for it first.
+void Context::orderAfterInline(hipStream_t producer) {
+  std::lock_guard<std::mutex> g(inlineMu_);
+  if (!inlinePending_ || inlineStream_ == producer) return;
+  if (!inlineRecorded_) {
+    // the null stream, which is always there to record on: behind whatever it
+    // holds by now, the launch included
+    if (inlineEvent_ == nullptr) {
+      FRG_HIP_CHECK(hipEventCreateWithFlags(&inlineEvent_, hipEventDisableTiming));
+    }
+    FRG_HIP_CHECK(hipEventRecord(inlineEvent_, nullptr));
+    inlineRecorded_ = true;
+  }
+  if (hipEventQuery(inlineEvent_) == hipSuccess) {
+    inlinePending_ = false;
+    return;
+  }
+  (void)hipGetLastError();
+  FRG_HIP_CHECK(hipStreamWaitEvent(producer, inlineEvent_, 0));
+}
+
+// Launches a small operation on the producer stream itself, if it is one the
+// rule covers and the reduce streams have drained, marks the work and calls
+// the completion callback (on this, the caller's, thread). Returns false when
+// the operation is to go through the pipeline instead.
+bool Context::tryInline(const Request& req, Work* work) {
+  if (inlineTrafficBytes_ <= 0 || req.fromHost || req.compressed || !launchBytesByContribs_) {
+    return false;
+  }
+  const int total = static_cast<int>(req.contribs.size());
+  if (total > kMaxContribsPerLaunch || req.numel <= 0) return false;
+  const int64_t elsize = elementSize(req.dtype);
+  if ((total + 1) * req.numel * elsize > inlineTrafficBytes_) return false;
+  if (profiling_.load(std::memory_order_relaxed)) return false;  // its records are per reduce stream
+  if (total == 1 && req.contribs[0] == req.out && req.scaleMode == FRG_SCALE_NONE) return false;
+  if (inlineSkips_.load(std::memory_order_relaxed) > 0) {
+    inlineSkips_.fetch_sub(1, std::memory_order_relaxed);
+    return false;
+  }
+  for (hipStream_t s : reduceStreams_) {
+    if (hipStreamQuery(s) != hipSuccess) {
+      (void)hipGetLastError();
+      inlineSkips_.store(kBusyProducerSkips, std::memory_order_relaxed);
+      return false;
+    }
+  }
+  ReduceArgs a;
+  a.out = req.out;
+  a.contribs = req.contribs.data();
+  a.K = total;
+  a.n = req.numel;
+  a.dtype = req.dtype;
+  a.op = req.op;
+  a.scale_mode = req.scaleMode;
+  a.scale = req.scale;
+  // From here on the operation is this function's; a failure is the work's
+  // status, as it would be on the command thread.
+  int status = FRG_OK;
+  std::string error;
+  try {
+    std::lock_guard<std::mutex> g(inlineMu_);
+    status = launchReduce(a, req.producerStream, &error);
+    if (status == FRG_OK) {
+      // The event that orders other streams after this launch. A stream of the
+      // caller's may be gone by the time it is needed, so it is recorded now;
+      // the null stream is always there, and a record on it now would make it
+      // look busy to the next operation's idle check for no reason: it is
+      // recorded when another stream turns up.
+      inlineRecorded_ = req.producerStream != nullptr;
+      if (inlineRecorded_) {
+        if (inlineEvent_ == nullptr) {
+          FRG_HIP_CHECK(hipEventCreateWithFlags(&inlineEvent_, hipEventDisableTiming));
+        }
+        FRG_HIP_CHECK(hipEventRecord(inlineEvent_, req.producerStream));
+      }
+      inlineStream_ = req.producerStream;
+      inlinePending_ = true;
+      inlineExplainsBusy_ = true;
+      work->doneStreams.assign(1, req.producerStream);
+      work->doneIndices.assign(1, -1);
+      work->donePositions.assign(1, -1);
+      progress_->launches.fetch_add(1);
+      progress_->onCallersStream.fetch_add(1);
+    }
+  } catch (const std::exception& e) {
+    status = FRG_ERR_HIP;
+    error = e.what();
+  }
+  if (status != FRG_OK) {
+    std::fprintf(stderr, "[fairring] operation #%lld failed: %s\n",
+                 static_cast<long long>(work->seq), error.c_str());
+  }
+  // every slice takes its turn in the slot rotation (fairring/device.cc:482)
+  nextStagingSlot_ += numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
+  progress_->started.fetch_add(1);
+  progress_->enqueued.fetch_add(1);
+  {
+    std::lock_guard<std::mutex> lock(work->mu);
+    work->status = status;
+    work->error = error;
+    work->lastStream = req.producerStream;
+    work->enqueued = true;
+    work->enqueuedFlag.store(true, std::memory_order_release);
+  }
+  if (req.done) req.done(req.user, status, req.producerStream);
+  return true;
 }
 
 int Context::submit(Request req, Work** workOut, std::string* err) {
@@ -602,23 +776,59 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   Work* work = new Work();
   work->device = device_;
   work->progress = progress_;
+  // nothing of the pipeline in flight, as far as the host can tell without asking
+  const bool nothingQueued = progress_->enqueued.load() == progress_->submitted.load();
   work->seq = progress_->submitted.fetch_add(1);
   hipEvent_t initial = nullptr;
   try {
     DeviceGuard g(device_);
+    orderAfterInline(req.producerStream);
+    if (nothingQueued && tryInline(req, work)) {
+      if (workOut) {
+        work->refs.fetch_add(1);
+        *workOut = work;
+      }
+      releaseWork(work);  // the share the command thread would have held
+      return FRG_OK;
+    }
     // Orders the pipeline after whatever produced the inputs
     // (fairring/device.cc:294-295). A producer stream that has already drained
     // has nothing to wait for, and no event is recorded on it: a record is a
     // packet on the producer's hardware queue, and two hundred of them per step
     // (one per bucket) are work for the command processor that the reduction's
     // own queues then wait behind.
+    // Asking an idle stream costs 0.1 us, asking a busy one over 10 (the
+    // runtime flushes its queue to find out) against 1 for the record: after a
+    // "busy" the next operations from that stream record without asking.
     bool producerIdle = false;
     if (idleProducerCheck_) {
-      const hipError_t q = hipStreamQuery(req.producerStream);
-      if (q == hipSuccess) {
-        producerIdle = true;
+      if (busyProducer_.load(std::memory_order_relaxed) == req.producerStream &&
+          busyProducerSkips_.load(std::memory_order_relaxed) > 0) {
+        busyProducerSkips_.fetch_sub(1, std::memory_order_relaxed);
       } else {
-        (void)hipGetLastError();  // "not ready" (or a failure the record below will report)
+        const hipError_t q = hipStreamQuery(req.producerStream);
+        if (q == hipSuccess) {
+          producerIdle = true;
+          std::lock_guard<std::mutex> ig(inlineMu_);
+          if (inlineStream_ == req.producerStream) {  // and with it what was launched there
+            inlinePending_ = false;
+            inlineExplainsBusy_ = false;
+          }
+        } else {
+          (void)hipGetLastError();  // "not ready" (or a failure the record below will report)
+          // (what keeps it busy may be a small operation of this context's own,
+          // launched there a moment ago and gone by the next time: ask again then)
+          bool ownLaunch = false;
+          {
+            std::lock_guard<std::mutex> ig(inlineMu_);
+            ownLaunch = inlineExplainsBusy_ && inlineStream_ == req.producerStream;
+            inlineExplainsBusy_ = false;  // once per launch
+          }
+          if (!ownLaunch) {
+            busyProducer_.store(req.producerStream, std::memory_order_relaxed);
+            busyProducerSkips_.store(kBusyProducerSkips, std::memory_order_relaxed);
+          }
+        }
       }
     }
     if (!producerIdle) {
@@ -1239,6 +1449,19 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
     // Without a callback nothing needs a single stream, and the streams keep
     // running independently of each other.
     work->doneStreams = used;
+    // where the operation stands on each of them, for waits that are remembered
+    for (hipStream_t s : used) {
+      int idx = -1;
+      for (size_t i = 0; i < reduceStreams_.size(); ++i) {
+        if (reduceStreams_[i] == s) idx = static_cast<int>(i);
+      }
+      int64_t position = -1;
+      if (idx >= 0 && idx < Progress::kMaxStreams) {
+        position = progress_->streamPosition[idx].fetch_add(1, std::memory_order_acq_rel) + 1;
+      }
+      work->doneIndices.push_back(idx);
+      work->donePositions.push_back(position);
+    }
   } catch (const ContractFailure& e) {
     status = e.code;
     error = e.what();
@@ -1284,6 +1507,12 @@ int Context::synchronize(std::string* err) {
     DeviceGuard g(device_);
     for (hipStream_t s : reduceStreams_) FRG_HIP_CHECK(hipStreamSynchronize(s));
     for (hipStream_t s : copyStreams_) FRG_HIP_CHECK(hipStreamSynchronize(s));
+    std::lock_guard<std::mutex> ig(inlineMu_);
+    if (inlinePending_) {  // what went to a caller's stream
+      FRG_HIP_CHECK(inlineRecorded_ ? hipEventSynchronize(inlineEvent_)
+                                    : hipStreamSynchronize(nullptr));
+      inlinePending_ = false;
+    }
   } catch (const std::exception& e) {
     *err = e.what();
     return FRG_ERR_HIP;

@@ -45,6 +45,16 @@ struct Progress {
   std::atomic<int64_t> started{0};    // operations the command thread has begun
   std::atomic<int64_t> enqueued{0};   // operations whose GPU work is all enqueued
   std::atomic<int64_t> launches{0};   // kernel launches issued
+  std::atomic<int64_t> onCallersStream{0};  // operations launched by submit() on the producer stream
+  // Per reduce stream: how many operations it has been given, and up to which
+  // of them the device's null stream already waits (the null stream is never
+  // destroyed, so what it was once told to wait for stays waited for: a step's
+  // worth of Work.wait() calls on it costs one event per reduce stream, not
+  // one per operation).
+  static constexpr int kMaxStreams = 8;
+  std::atomic<int64_t> streamPosition[kMaxStreams] = {};
+  std::mutex nullWaitMu;
+  int64_t nullStreamWaitsFor[kMaxStreams] = {};
 };
 
 // Completion state of one submitted operation (what the reference keeps in an
@@ -58,10 +68,15 @@ struct Work {
   std::string error;
   // The streams the operation's work ended on. No event is recorded per
   // operation (an event record is a packet on the stream, between two launches
-  // that would otherwise run back to back): waiting is done against the
-  // streams themselves, which are in order, so it covers the operation and
-  // whatever was enqueued on them up to the moment of the wait.
+  // that would otherwise run back to back: one per 25 MiB bucket cost a stream
+  // of buckets 4 %): waiting is done against the streams themselves, which are
+  // in order, so it covers the operation and whatever was enqueued on them up
+  // to the moment of the wait. donePositions[i] counts the operations
+  // doneStreams[i] had been given when this one was (Progress::streamPosition),
+  // for reduce streams; -1 for a caller's stream.
   std::vector<hipStream_t> doneStreams;
+  std::vector<int> doneIndices;        // which reduce stream, -1 for a caller's
+  std::vector<int64_t> donePositions;
   hipStream_t lastStream = nullptr;
   int device = 0;
   int64_t seq = 0;  // position among the context's operations
@@ -200,6 +215,30 @@ class Context {
   // Ask the runtime whether the producer stream has drained before recording
   // the initial event on it (FAIRRING_IDLE_PRODUCER_CHECK=0 records always).
   bool idleProducerCheck_ = true;
+  // The producer stream that last answered "busy", and how many more of its
+  // operations record their event without asking again (any thread may submit).
+  static constexpr int kBusyProducerSkips = 15;
+  std::atomic<hipStream_t> busyProducer_{nullptr};
+  std::atomic<int> busyProducerSkips_{0};
+  // Small operations on the caller's stream. With nothing of the pipeline in
+  // flight, an operation of one launch that moves at most this many bytes is
+  // launched by submit() itself on the producer stream: handing it to the
+  // reduce streams costs two cross-stream waits of 6 to 13 us of host time each
+  // (producer -> reduce stream, reduce stream -> consumer), several times what
+  // the kernel takes. FAIRRING_INLINE_BYTES overrides it (0: never).
+  int64_t inlineTrafficBytes_ = 16ll << 20;
+  std::atomic<int> inlineSkips_{0};  // attempts to leave out after a reduce stream answered "busy"
+  // The last such launch: an event recorded behind it and the stream it went
+  // to (kept for comparison only, never used after the call that set it).
+  // Whatever is submitted from another stream is ordered after that event.
+  std::mutex inlineMu_;
+  hipEvent_t inlineEvent_ = nullptr;
+  hipStream_t inlineStream_ = nullptr;
+  bool inlinePending_ = false;
+  bool inlineExplainsBusy_ = false;  // the idle check has not been answered since that launch
+  bool inlineRecorded_ = false;  // inlineEvent_ stands behind that launch (else: the null stream, not yet recorded)
+  bool tryInline(const Request& req, Work* work);
+  void orderAfterInline(hipStream_t producer);
 
   std::vector<hipStream_t> reduceStreams_;
   // Slot s is filled on copy stream s % copyStreams_.size(): while one stream works through the
@@ -222,7 +261,7 @@ class Context {
   std::vector<hipEvent_t> slotFreeEvents_;    // recorded after a slot's last consumer
   std::vector<hipEvent_t> slotFilledEvents_;  // recorded after the copy into a slot
   std::vector<char> slotUsed_;
-  int64_t nextStagingSlot_ = 0;  // round-robin cursor (fairring/device.cc:482)
+  std::atomic<int64_t> nextStagingSlot_{0};  // round-robin cursor (fairring/device.cc:482)
   int64_t nextSeq_ = 0;          // operation counter for log lines
   std::shared_ptr<Progress> progress_ = std::make_shared<Progress>();
 

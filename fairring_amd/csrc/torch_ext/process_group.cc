@@ -105,6 +105,62 @@ class GilRelease {
   PyThreadState* saved_ = nullptr;
 };
 
+
+}  // namespace
+
+// The state of one operation in flight. The result tensor and the status are
+// written before `done` is set and not changed after it; the future is made by
+// the first getFuture(), and completed by whoever finds both it and `done`:
+// the completion callback if the future was there first, else getFuture().
+struct ProcessGroupFairring::OpState {
+  std::mutex mu;
+  std::atomic<bool> done{false};
+  int status = FRG_OK;
+  hipStream_t lastStream = nullptr;
+  c10::intrusive_ptr<c10::ivalue::Future> future;
+  at::Tensor tensor;               // the result tensor (the caller's, reduced in place)
+  std::vector<at::Tensor> inputs;  // kept alive until the operation is enqueued
+  c10::DeviceIndex device = 0;
+};
+
+namespace {
+
+using OpState = ProcessGroupFairring::OpState;
+
+std::string failureText(int status) {
+  return "fairring: allreduce failed with status " + std::to_string(status);
+}
+
+// Completes the future under a guard of the operation's last stream, so that
+// consumers are ordered after it on the GPU without a host wait
+// (fairring/device.cc:337-348).
+void completeFuture(const OpState& st, const c10::intrusive_ptr<c10::ivalue::Future>& future) {
+  c10::Stream s = c10::hip::getStreamFromExternalMasqueradingAsCUDA(st.lastStream, st.device);
+  c10::StreamGuard g(s);
+  if (st.status == FRG_OK) {
+    future->markCompleted(std::vector<at::Tensor>{st.tensor});
+  } else {
+    future->setError(std::make_exception_ptr(std::runtime_error(failureText(st.status))));
+  }
+}
+
+// Runs on the pipeline's command thread once the last slice is enqueued.
+void onEnqueued(void* user, int status, void* lastStream) {
+  std::unique_ptr<std::shared_ptr<OpState>> holder(static_cast<std::shared_ptr<OpState>*>(user));
+  OpState& st = **holder;
+  c10::intrusive_ptr<c10::ivalue::Future> future;
+  std::vector<at::Tensor> inputs;
+  {
+    std::lock_guard<std::mutex> g(st.mu);
+    st.status = status;
+    st.lastStream = static_cast<hipStream_t>(lastStream);
+    st.done.store(true, std::memory_order_release);
+    future = st.future;
+    inputs.swap(st.inputs);
+  }
+  if (future) completeFuture(st, future);
+}
+
 }  // namespace
 
 // ---- WorkFairring ---------------------------------------------------------
@@ -117,25 +173,68 @@ ProcessGroupFairring::WorkFairring::WorkFairring(
       group_(std::move(group)),
       ctx_(ctx) {}
 
-ProcessGroupFairring::WorkFairring::~WorkFairring() = default;
+ProcessGroupFairring::WorkFairring::WorkFairring(
+    c10d::OpType opType, std::shared_ptr<OpState> state, frg_work* handle,
+    c10::intrusive_ptr<c10d::Backend> group, frg_ctx* ctx)
+    : c10d::Work(-1, opType),
+      state_(std::move(state)),
+      handle_(handle),
+      group_(std::move(group)),
+      ctx_(ctx) {}
 
-bool ProcessGroupFairring::WorkFairring::isCompleted() { return future_->completed(); }
+ProcessGroupFairring::WorkFairring::~WorkFairring() {
+  if (handle_ != nullptr) (void)frg_work_release(handle_);
+}
 
-bool ProcessGroupFairring::WorkFairring::isSuccess() const { return future_->hasValue(); }
+bool ProcessGroupFairring::WorkFairring::isCompleted() {
+  return state_ ? state_->done.load(std::memory_order_acquire) : future_->completed();
+}
+
+bool ProcessGroupFairring::WorkFairring::isSuccess() const {
+  if (!state_) return future_->hasValue();
+  return state_->done.load(std::memory_order_acquire) && state_->status == FRG_OK;
+}
 
 std::exception_ptr ProcessGroupFairring::WorkFairring::exception() const {
-  return future_->exception_ptr();
+  if (!state_) return future_->exception_ptr();
+  if (state_->done.load(std::memory_order_acquire) && state_->status != FRG_OK) {
+    return std::make_exception_ptr(std::runtime_error(failureText(state_->status)));
+  }
+  return nullptr;
 }
 
 std::vector<at::Tensor> ProcessGroupFairring::WorkFairring::result() {
   awaitCompletion();
+  if (state_) return {state_->tensor};
   return future_->value().toTensorVector();
+}
+
+// The caller's current stream waits for the operation; the host only until the
+// command thread has enqueued it (what waiting on the reference's future does:
+// fairring/process_group.cc:64-68). A limit set with FAIRRING_WAIT_TIMEOUT_S
+// applies inside the handle's own wait.
+void ProcessGroupFairring::WorkFairring::awaitCompletion() {
+  if (!state_) {
+    awaitFuture();
+    return;
+  }
+  hipStream_t current =
+      c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(state_->device).stream();
+  int rc;
+  {
+    GilRelease unlocked;
+    rc = frg_work_block_stream(handle_, current);
+  }
+  if (rc == FRG_ERR_NOT_READY) {
+    TORCH_CHECK(false, "fairring: ", frg_last_error());
+  }
+  if (rc != FRG_OK) throw std::runtime_error(failureText(rc));
 }
 
 // FAIRRING_WAIT_TIMEOUT_S (seconds, unset or 0: no limit, as in the reference):
 // a wait that sees no completion for that long raises with a report of where
 // the pipeline stands, instead of blocking for good.
-void ProcessGroupFairring::WorkFairring::awaitCompletion() {
+void ProcessGroupFairring::WorkFairring::awaitFuture() {
   static const double limit = [] {
     const char* v = std::getenv("FAIRRING_WAIT_TIMEOUT_S");
     const double s = v ? std::atof(v) : 0.0;
@@ -196,7 +295,22 @@ bool ProcessGroupFairring::WorkFairring::wait(std::chrono::milliseconds /*timeou
 void ProcessGroupFairring::WorkFairring::abort() {}
 
 c10::intrusive_ptr<c10::ivalue::Future> ProcessGroupFairring::WorkFairring::getFuture() {
-  return future_;
+  if (!state_) return future_;
+  c10::intrusive_ptr<c10::ivalue::Future> future;
+  bool completeHere = false;
+  {
+    std::lock_guard<std::mutex> g(state_->mu);
+    if (!state_->future) {
+      state_->future = c10::make_intrusive<c10::ivalue::Future>(
+          c10::ListType::ofTensors(),
+          std::vector<c10::Device>{c10::Device(c10::kCUDA, state_->device)});
+      // enqueued already: the callback has been and gone
+      completeHere = state_->done.load(std::memory_order_acquire);
+    }
+    future = state_->future;
+  }
+  if (completeHere) completeFuture(*state_, future);
+  return future;
 }
 
 // ---- OptionsFairring -------------------------------------------------------
@@ -539,9 +653,6 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     recordOnPipelineStreams(device, fromHost, {&out, &own}, nullptr);
   }
 
-  auto future = c10::make_intrusive<c10::ivalue::Future>(
-      c10::ListType::ofTensors(), std::vector<c10::Device>{out.device()});
-
   const bool divide = fusedDivide_ && op == c10d::ReduceOp::SUM && size > 1;
   const bool pow2 = (size & (size - 1)) == 0;
   int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
@@ -571,21 +682,26 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
 
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
   keepAlive.push_back(own);
-  auto* pending = new Pending{future, out, std::move(keepAlive), device};
+  auto state = std::make_shared<OpState>();
+  state->tensor = out;
+  state->inputs = std::move(keepAlive);
+  state->device = device;
+  auto* holder = new std::shared_ptr<OpState>(state);
+  frg_work* handle = nullptr;
   int rc;
   if (fromHost) {
     rc = frg_allreduce_host(ctx, out.data_ptr(), table.data() + 1, size - 1, n, dtype, frgOp,
-                            scaleMode, scale, /*carry=*/1, current, &onDone, pending, nullptr);
+                            scaleMode, scale, /*carry=*/1, current, &onEnqueued, holder, &handle);
   } else {
     rc = frg_allreduce(ctx, out.data_ptr(), table.data(), size, n, dtype, frgOp, scaleMode,
-                       scale, current, &onDone, pending, nullptr);
+                       scale, current, &onEnqueued, holder, &handle);
   }
   if (rc != FRG_OK) {
-    delete pending;
+    delete holder;
     TORCH_CHECK(false, "fairring: ", frg_last_error());
   }
   return c10::make_intrusive<WorkFairring>(
-      opType, std::move(future),
+      opType, std::move(state), handle,
       c10::intrusive_ptr<c10d::Backend>::unsafe_reclaim_from_nonowning(this), ctx);
 }
 

@@ -13,7 +13,9 @@
 #include <torch/csrc/distributed/c10d/Work.hpp>
 #include <torch/torch.h>
 
+#include <atomic>
 #include <map>
+#include <memory>
 #include <mutex>
 
 #include "../../../include/fairring_hip.h"
@@ -25,12 +27,24 @@ constexpr const char* kPgName = "fairring";
 class ProcessGroupFairring : public c10d::Backend {
  public:
   // fairring/process_group.h:24-50, fairring/process_group.cc:35-75
+  // What an operation in flight shares between its Work and the pipeline's
+  // completion callback.
+  struct OpState;
+
   class WorkFairring : public c10d::Work {
    public:
-    // `group` and `ctx` (optional) let a wait that gives up say where the
-    // pipeline stands; the work keeps the group, and so the context, alive.
+    // A work that is its future (already completed, or completed by a callback
+    // of its own). `group` and `ctx` (optional) let a wait that gives up say
+    // where the pipeline stands; the work keeps the group, and so the context,
+    // alive.
     WorkFairring(c10d::OpType opType, c10::intrusive_ptr<c10::ivalue::Future> future,
                  c10::intrusive_ptr<c10d::Backend> group = {}, frg_ctx* ctx = nullptr);
+    // A work over the pipeline's own handle: wait() orders the caller's stream
+    // after the operation through that handle, and the device-aware future
+    // (an event created, recorded and waited for per operation) is only made if
+    // getFuture() asks for it. Takes over `handle`.
+    WorkFairring(c10d::OpType opType, std::shared_ptr<OpState> state, frg_work* handle,
+                 c10::intrusive_ptr<c10d::Backend> group, frg_ctx* ctx);
     ~WorkFairring() override;
 
     bool isCompleted() override;
@@ -44,7 +58,10 @@ class ProcessGroupFairring : public c10d::Backend {
 
    private:
     void awaitCompletion();
-    const c10::intrusive_ptr<c10::ivalue::Future> future_;
+    void awaitFuture();
+    const c10::intrusive_ptr<c10::ivalue::Future> future_;  // null with a handle
+    const std::shared_ptr<OpState> state_;
+    frg_work* const handle_ = nullptr;
     const c10::intrusive_ptr<c10d::Backend> group_;
     frg_ctx* const ctx_;
   };

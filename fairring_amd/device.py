@@ -358,11 +358,13 @@ class DeviceFairring:
         return submit
 
     def progress(self):
-        """Operations submitted / started by the command thread / fully
-        enqueued, and kernel launches issued, so far."""
-        out = (ctypes.c_int64 * 4)()
+        """Operations submitted / started / fully enqueued, kernel launches
+        issued, and operations launched by the call itself on the producer
+        stream (small ones, with nothing in flight), so far."""
+        out = (ctypes.c_int64 * 5)()
         _capi.check(_capi.lib().frg_get_progress(self._h, ctypes.byref(out)))
-        return dict(submitted=out[0], started=out[1], enqueued=out[2], launches=out[3])
+        return dict(submitted=out[0], started=out[1], enqueued=out[2], launches=out[3],
+                    on_callers_stream=out[4])
 
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))

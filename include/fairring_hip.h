@@ -253,10 +253,12 @@ FRG_API int frg_get_streams(frg_ctx* ctx, void** streams, int capacity, int* cou
  * submits a host-staged operation (they write `out`). */
 FRG_API int frg_get_copy_streams(frg_ctx* ctx, void** streams, int capacity, int* count);
 
-/* Called on the command thread once the last slice of an operation has been
- * enqueued (status FRG_OK) or enqueueing failed; `last_stream` is the stream
- * on which completion is ordered (device.cc:337-340 marks the future under a
- * guard of that stream). */
+/* Called once the last slice of an operation has been enqueued (status FRG_OK)
+ * or enqueueing failed; `last_stream` is the stream on which completion is
+ * ordered (device.cc:337-340 marks the future under a guard of that stream).
+ * It runs on the command thread, or, for a small operation that frg_allreduce
+ * launches itself (see there), on the calling thread before that call returns:
+ * it must not take a lock the caller holds across the call. */
 typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
 
 /* DeviceFairring::allReduce: fairring/device.cc:291-353, with the
@@ -280,7 +282,17 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
  * one of the contributions. `producer_stream` is the stream the caller's
  * producer work was enqueued on (the reference records its initial event on
  * the current stream, device.cc:294-295). Returns immediately; `*work`
- * (optional) receives a handle to wait on. */
+ * (optional) receives a handle to wait on.
+ * A small operation (one launch that moves at most 16 MiB, contributions and
+ * output together; FAIRRING_INLINE_BYTES overrides the figure, 0 switches the
+ * rule off) that arrives while nothing of this context is queued or running is
+ * launched by this call on `producer_stream` itself, behind the producer's
+ * work: handing it to a reduce stream and the result back costs two
+ * cross-stream waits of 6 to 13 us of host time each, against 3 us for the
+ * launch. Its completion is then ordered on `producer_stream`
+ * (frg_work_block_stream on that stream is free); whatever this context is
+ * handed afterwards from another stream is ordered after it with an event, and
+ * frg_synchronize covers it. */
 FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
                           int K, int64_t numel, int dtype, int op,
                           int scale_mode, float scale, void* producer_stream,
@@ -325,12 +337,15 @@ FRG_API int frg_work_wait(frg_work* work);
 FRG_API int frg_set_wait_timeout(double seconds);
 
 /* Where the pipeline stands, for such reports: operations accepted, begun by
- * the command thread and fully enqueued, and kernel launches issued so far. */
+ * the command thread and fully enqueued, and kernel launches issued so far;
+ * and how many of the operations were small enough, with nothing in flight, to
+ * be launched by the call itself on the producer stream (see frg_allreduce). */
 typedef struct frg_progress {
   int64_t submitted;
   int64_t started;
   int64_t enqueued;
   int64_t launches;
+  int64_t on_callers_stream;
 } frg_progress;
 FRG_API int frg_get_progress(frg_ctx* ctx, frg_progress* out);
 

@@ -897,3 +897,140 @@ def test_random_sequences_of_dependent_operations_match_sequential_execution(see
             assert bool(torch.equal(bufs[i].view(torch.int32), shadow[i].view(torch.int32))), i
     finally:
         dev.close()
+
+
+def _hold(stream, ballast, times=30):
+    """Keeps `stream` busy for a few milliseconds (elementwise passes over 256 MiB)."""
+    with torch.cuda.stream(stream):
+        for _ in range(times):
+            ballast.add_(1.0)
+
+
+def test_small_operation_with_nothing_in_flight_runs_on_the_callers_stream():
+    # One launch that moves at most 16 MiB, with the pipeline idle, is launched by the call itself
+    # on the producer stream (no reduce stream, no event between streams). Whatever comes next
+    # from another stream is still ordered after it, and synchronize() covers it.
+    _print_case("small operation on the caller's stream")
+    g = torch.Generator(device=DEV)
+    g.manual_seed(77)
+    small, big, k = 100_003, 8_000_000, 4
+    xs = [torch.empty(big, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    ballast = [torch.zeros(64 * MiB, device=DEV) for _ in range(2)]
+    p, q = torch.cuda.Stream(), torch.cuda.Stream()
+    dev = fa.DeviceFairring(0)
+    torch.cuda.synchronize()
+    try:
+        # read after write across streams: the small result feeds a large operation
+        mid = torch.zeros(big, device=DEV)
+        out = torch.zeros(big, device=DEV)
+        torch.cuda.synchronize()
+        _hold(p, ballast[0])
+        before = dev.progress()
+        w0 = dev.allreduce(mid[:small], [x[:small] for x in xs], scale_mode=fa.SCALE_MUL,
+                           scale=0.25, stream=p)
+        after = dev.progress()
+        assert after["on_callers_stream"] == before["on_callers_stream"] + 1
+        assert after["submitted"] == after["enqueued"] == before["submitted"] + 1
+        assert w0.is_completed()                       # enqueued, on p, behind the ballast
+        w1 = dev.allreduce(out, [mid, xs[1]], stream=q)   # 96 MB: through the pipeline
+        assert dev.progress()["on_callers_stream"] == after["on_callers_stream"]
+        w1.wait()
+        want_mid = xs[0][:small] + xs[1][:small]
+        want_mid.add_(xs[2][:small]).add_(xs[3][:small]).mul_(0.25)
+        assert bool(torch.equal(out[:small].view(torch.int32),
+                                (want_mid + xs[1][:small]).view(torch.int32)))
+        assert bool(torch.equal(out[small:].view(torch.int32), xs[1][small:].view(torch.int32)))
+        host = [x[:small].cpu().numpy() for x in xs]
+        assert_bits_equal(mid[:small].cpu().numpy(), oracle.sum_f32(host, oracle.SCALE_MUL, 0.25))
+        dev.synchronize()
+        torch.cuda.synchronize()
+
+        # two small in-place operations on one tensor from two streams, the first held up
+        own = xs[0][:small].clone()
+        torch.cuda.synchronize()
+        _hold(p, ballast[0])
+        before = dev.progress()["on_callers_stream"]
+        dev.allreduce(own, [own] + [x[:small] for x in xs[1:]], scale_mode=fa.SCALE_MUL, scale=0.5,
+                      stream=p)
+        w = dev.allreduce(own, [own] + [x[:small] for x in xs[1:]], scale_mode=fa.SCALE_MUL,
+                          scale=2.0, stream=q)
+        assert dev.progress()["on_callers_stream"] == before + 2
+        w.wait()                                       # q, which waited for p's operation
+        acc = host[0]
+        for s in (0.5, 2.0):
+            acc = oracle.sum_f32([acc] + host[1:], oracle.SCALE_MUL, s)
+        assert_bits_equal(own.cpu().numpy(), acc)
+
+        # synchronize() covers what went to a caller's stream
+        res = torch.zeros(small, device=DEV)
+        torch.cuda.synchronize()
+        _hold(q, ballast[1])
+        dev.allreduce(res, [x[:small] for x in xs], stream=q)
+        dev.synchronize()
+        assert_bits_equal(res.cpu().numpy(), oracle.sum_f32(host))
+        torch.cuda.synchronize()
+    finally:
+        dev.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_mix_of_small_and_large_operations_from_two_streams(seed):
+    # Small operations (launched on the caller's stream when nothing is in flight) and large ones
+    # (through the reduce streams), from two producer streams that are held up at random, over
+    # shared buffers: the result is that of running them one after the other.
+    _print_case("random small and large operations from two streams", seed)
+    rng = np.random.default_rng(9300 + seed)
+    nbuf, size = 4, 4 * MiB                               # four buffers of 16 MiB
+    g = torch.Generator(device=DEV)
+    g.manual_seed(9300 + seed)
+    bufs = [torch.empty(size, device=DEV).normal_(0, 1.0, generator=g) for _ in range(nbuf)]
+    shadow = [b.clone() for b in bufs]
+    ballast = [torch.zeros(64 * MiB, device=DEV) for _ in range(2)]
+    producers = [torch.cuda.Stream(), torch.cuda.Stream()]
+    dev = fa.DeviceFairring(0)
+    torch.cuda.synchronize()
+    try:
+        works = []
+        for step in range(60):
+            if rng.random() < 0.2:
+                dev.synchronize()                         # lets the pipeline run empty
+                torch.cuda.synchronize()
+            small = rng.random() < 0.6
+            n = int(rng.integers(1024, 200_000)) if small else int(rng.integers(MiB, 3 * MiB))
+            which = int(rng.integers(2))
+            if rng.random() < 0.3:
+                _hold(producers[which], ballast[which], times=8)
+            ob = int(rng.integers(nbuf))
+            olo = int(rng.integers(0, size - n)) // 4 * 4
+            k = int(rng.integers(2, 5))
+            terms = []
+            for _ in range(k):
+                if rng.random() < 0.3:
+                    terms.append((ob, olo))
+                    continue
+                while True:
+                    cb = int(rng.integers(nbuf))
+                    clo = int(rng.integers(0, size - n)) // 4 * 4
+                    if cb != ob or clo + n <= olo or olo + n <= clo:
+                        break
+                terms.append((cb, clo))
+            scale = float(rng.choice([0.5, 0.25, 1.0, 2.0]))
+            works.append(dev.allreduce(bufs[ob][olo:olo + n],
+                                       [bufs[b][lo:lo + n] for b, lo in terms],
+                                       scale_mode=fa.SCALE_MUL, scale=scale,
+                                       stream=producers[which]))
+            acc = shadow[terms[0][0]][terms[0][1]:terms[0][1] + n].clone()
+            for b, lo in terms[1:]:
+                acc.add_(shadow[b][lo:lo + n])
+            acc.mul_(scale)
+            shadow[ob][olo:olo + n] = acc
+        for w in works:
+            w.wait()
+        dev.synchronize()
+        torch.cuda.synchronize()
+        done = dev.progress()
+        assert 0 < done["on_callers_stream"] < done["submitted"] == 60
+        for i in range(nbuf):
+            assert bool(torch.equal(bufs[i].view(torch.int32), shadow[i].view(torch.int32))), i
+    finally:
+        dev.close()

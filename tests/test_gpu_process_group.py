@@ -74,6 +74,83 @@ def test_allreduce_fused_divide_and_future():
     assert pg._layout() == [3276672, 3276672, 16, 16]
 
 
+def test_future_asked_for_late_or_twice_or_never():
+    """The work waits through the pipeline's own handle; the future is made by
+    the first get_future(), also when the operation has long been enqueued, and
+    orders its consumers after the reduction all the same."""
+    print("[case] pg future made on demand", flush=True)
+    size, rank, n = 8, 1, 2_000_003
+    rng = np.random.default_rng(15)
+    x = (rng.standard_normal((size, n)) * 0.01).astype(np.float32)
+    want = oracle.sum_f32(list(x))
+    pg = make_pg(rank, size)
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(x[r].copy()).to(DEV) for r in range(size) if r != rank])
+
+    # never: wait() alone orders the current stream after the result
+    own = torch.from_numpy(x[rank].copy()).to(DEV)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        side.wait_stream(torch.cuda.default_stream())
+        work = pg.allreduce([own])
+        assert work.wait() is True
+        twice = own * 2          # on `side`, after the reduction
+    side.synchronize()
+    assert_bits_equal(twice.cpu().numpy(), want * np.float32(2))
+    assert work.is_completed() and work.is_success()
+
+    # a small operation goes to the caller's stream; a wait on another stream
+    # orders that one after it, and so does the future
+    ns = 50_001
+    small_want = oracle.sum_f32([r[:ns] for r in x])
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(x[r, :ns].copy()).to(DEV) for r in range(size) if r != rank])
+    own = torch.from_numpy(x[rank, :ns].copy()).to(DEV)
+    ballast = torch.zeros(64 * MiB, device=DEV)
+    pg._synchronize()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(20):
+            ballast.add_(1.0)           # the operation queues up behind this
+        work = pg.allreduce([own])
+    work.wait()                         # the default stream waits for `side`'s operation
+    plus = own + 1
+    fut = work.get_future()
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):
+        times = fut.then(lambda f: f.value()[0] * 3).wait()
+    torch.cuda.synchronize()
+    assert_bits_equal(own.cpu().numpy(), small_want)
+    assert_bits_equal(plus.cpu().numpy(), small_want + np.float32(1))
+    assert_bits_equal(times.cpu().numpy(), small_want * np.float32(3))
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(x[r].copy()).to(DEV) for r in range(size) if r != rank])
+
+    # late: the operation is enqueued and finished before anyone asks
+    own = torch.from_numpy(x[rank].copy()).to(DEV)
+    work = pg.allreduce([own])
+    work.wait()
+    torch.cuda.synchronize()
+    fut = work.get_future()
+    assert fut.done()
+    assert work.get_future() is fut or work.get_future().done()
+    got = fut.then(lambda f: f.value()[0] + 1).wait()
+    torch.cuda.synchronize()
+    assert fut.value()[0].data_ptr() == own.data_ptr()
+    assert_bits_equal(own.cpu().numpy(), want)
+    assert_bits_equal(got.cpu().numpy(), want + np.float32(1))
+
+    # at once, then dropped together with the work: the callback still runs
+    seen = []
+    for i in range(20):
+        own = torch.from_numpy(x[rank].copy()).to(DEV)
+        pg.allreduce([own]).get_future().then(lambda f, i=i: seen.append(i))
+        del own
+    pg._synchronize()
+    torch.cuda.synchronize()
+    assert sorted(seen) == list(range(20))
+
+
 def test_allreduce_non_power_of_two_divide():
     print("[case] pg divide by 3", flush=True)
     size, rank, n = 3, 1, 50_001
