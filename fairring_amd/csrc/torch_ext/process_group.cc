@@ -466,9 +466,13 @@ void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor>
         auto it = streams_.find(t.device().index());
         if (it == streams_.end()) continue;
         for (const c10::Stream& st : it->second) t.record_stream(st);
+        for (const c10::Stream& st : peersUsedFrom_) {
+          if (st.device_index() == t.device().index()) t.record_stream(st);
+        }
       }
     }
     peersUsed_ = false;
+    peersUsedFrom_.clear();
   }
 }
 
@@ -680,7 +684,14 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     }
   }
 
-  hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
+  const auto currentStream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
+  hipStream_t current = currentStream.stream();
+  {
+    const c10::Stream asStream = currentStream.unwrap();
+    bool seen = false;
+    for (const c10::Stream& st : peersUsedFrom_) seen = seen || st == asStream;
+    if (!seen) peersUsedFrom_.push_back(asStream);
+  }
   keepAlive.push_back(own);
   auto state = std::make_shared<OpState>();
   state->tensor = out;

@@ -199,6 +199,9 @@ class ProcessGroupFairring : public c10d::Backend {
   std::vector<at::Tensor> peers_;     // flat views, checked when they were set
   bool peersFromHost_ = false;
   bool peersUsed_ = false;             // by an operation since they were set
+  // The callers' streams those operations came from: a small operation runs on
+  // its caller's stream, so that stream reads the peers' tensors too.
+  std::vector<c10::Stream> peersUsedFrom_;
   bool fusedDivide_ = false;
 };
 
