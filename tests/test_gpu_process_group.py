@@ -532,3 +532,39 @@ def test_random_process_group_case(seed):
         zero = (want == 0) if kind in ("f32", "f64") else ((want & 0x7FFF) == 0)
         got, want = got[~zero], want[~zero]
     assert_bits_equal(got, want, str(case), half=kind == "f16")
+
+
+@pytest.mark.parametrize("consumer", ["default", "side"])
+def test_waiting_on_every_bucket_orders_the_consumer_after_all_of_them(consumer):
+    """DDP's end of backward: every bucket's work is waited for on one stream,
+    which then reads the results with no host synchronisation in between. On
+    the default (null) stream the pipeline tells that stream only once per
+    reduce stream what to wait for; the results must be complete all the same."""
+    print("[case] pg waits on every bucket, consumer on the", consumer, "stream", flush=True)
+    size, rank, nb, n = 4, 1, 24, 16 * MiB          # 24 buckets of 64 MiB
+    g = torch.Generator(device=DEV)
+    g.manual_seed(33)
+    peers = [torch.empty(n, device=DEV).normal_(0, 1.0, generator=g) for _ in range(size - 1)]
+    owns = [torch.empty(n, device=DEV).normal_(0, 1.0, generator=g) for _ in range(nb)]
+    want = []
+    for o in owns:                                   # rank order: peer 0, own, peers 1 and 2
+        acc = peers[0] + o
+        acc.add_(peers[1]).add_(peers[2])
+        want.append(acc)
+    pg = make_pg(rank, size, slice_bytes=25 * MiB)
+    pg._set_simulated_peer_contributions(peers)
+    stream = torch.cuda.default_stream() if consumer == "default" else torch.cuda.Stream()
+    with torch.cuda.stream(stream):                  # the comparison's kernels loaded beforehand:
+        torch.equal(want[0].view(torch.int32), want[1].view(torch.int32))   # the first call takes 0.1 s
+    torch.cuda.synchronize()
+    works = [pg.allreduce([o]) for o in owns]        # 7.7 GB of traffic: still running below
+    with torch.cuda.stream(stream):
+        for w in works:
+            assert w.wait() is True
+        # reads on `stream`, right behind the waits; the bucket submitted last first,
+        # which is the one still furthest from done
+        same = [torch.equal(o.view(torch.int32), w_.view(torch.int32))
+                for o, w_ in zip(reversed(owns), reversed(want))]
+    assert all(same)
+    pg._synchronize()
+    torch.cuda.synchronize()
