@@ -612,14 +612,15 @@ bool Context::tryInline(const Request& req, Work* work) {
   if ((total + 1) * req.numel * elsize > inlineTrafficBytes_) return false;
   if (profiling_.load(std::memory_order_relaxed)) return false;  // its records are per reduce stream
   if (total == 1 && req.contribs[0] == req.out && req.scaleMode == FRG_SCALE_NONE) return false;
-  if (inlineSkips_.load(std::memory_order_relaxed) > 0) {
-    inlineSkips_.fetch_sub(1, std::memory_order_relaxed);
-    return false;
-  }
+  // Asking a busy stream costs 12 us: after a "busy" nobody asks again for a while.
+  const int64_t now = std::chrono::duration_cast<std::chrono::nanoseconds>(
+                          std::chrono::steady_clock::now().time_since_epoch())
+                          .count();
+  if (now < inlineRetryAtNs_.load(std::memory_order_relaxed)) return false;
   for (hipStream_t s : reduceStreams_) {
     if (hipStreamQuery(s) != hipSuccess) {
       (void)hipGetLastError();
-      inlineSkips_.store(kBusyProducerSkips, std::memory_order_relaxed);
+      inlineRetryAtNs_.store(now + kInlineRetryNs, std::memory_order_relaxed);
       return false;
     }
   }

@@ -227,7 +227,9 @@ class Context {
   // (producer -> reduce stream, reduce stream -> consumer), several times what
   // the kernel takes. FAIRRING_INLINE_BYTES overrides it (0: never).
   int64_t inlineTrafficBytes_ = 16ll << 20;
-  std::atomic<int> inlineSkips_{0};  // attempts to leave out after a reduce stream answered "busy"
+  // After a reduce stream answered "busy" the rule is not tried again before this time.
+  static constexpr int64_t kInlineRetryNs = 200 * 1000;
+  std::atomic<int64_t> inlineRetryAtNs_{0};
   // The last such launch: an event recorded behind it and the stream it went
   // to (kept for comparison only, never used after the call that set it).
   // Whatever is submitted from another stream is ordered after that event.

@@ -923,6 +923,15 @@ def test_small_operation_with_nothing_in_flight_runs_on_the_callers_stream():
         # read after write across streams: the small result feeds a large operation
         mid = torch.zeros(big, device=DEV)
         out = torch.zeros(big, device=DEV)
+        # Every kind of call once beforehand: a first call takes milliseconds (code objects are
+        # loaded), longer than the producer is held up below, and would hide a missing order.
+        for s_ in (p, q):
+            dev.allreduce(mid[:small], [x[:small] for x in xs], stream=s_).wait()
+            dev.allreduce(out, [mid, xs[1]], stream=s_).wait()
+            _hold(s_, ballast[0], times=2)
+        dev.synchronize()
+        mid.zero_()
+        out.zero_()
         torch.cuda.synchronize()
         _hold(p, ballast[0])
         before = dev.progress()
@@ -974,63 +983,82 @@ def test_small_operation_with_nothing_in_flight_runs_on_the_callers_stream():
 
 
 @pytest.mark.parametrize("seed", range(4))
-def test_random_mix_of_small_and_large_operations_from_two_streams(seed):
+def test_random_mix_of_small_and_large_operations_from_two_streams(seed, monkeypatch):
     # Small operations (launched on the caller's stream when nothing is in flight) and large ones
-    # (through the reduce streams), from two producer streams that are held up at random, over
-    # shared buffers: the result is that of running them one after the other.
+    # (through the reduce streams) from two producer streams over ranges of four 4 MiB buffers, so
+    # that neighbouring operations often share memory. Each episode starts from an idle pipeline
+    # with a small operation behind a held-up producer (it sits on that stream for milliseconds),
+    # followed by up to four operations of either kind from either stream; the result is that of
+    # running them one after the other. "Small" is up to 1 MiB moved here.
     _print_case("random small and large operations from two streams", seed)
     rng = np.random.default_rng(9300 + seed)
-    nbuf, size = 4, 4 * MiB                               # four buffers of 16 MiB
+    nbuf, size = 4, MiB
     g = torch.Generator(device=DEV)
     g.manual_seed(9300 + seed)
     bufs = [torch.empty(size, device=DEV).normal_(0, 1.0, generator=g) for _ in range(nbuf)]
     shadow = [b.clone() for b in bufs]
     ballast = [torch.zeros(64 * MiB, device=DEV) for _ in range(2)]
     producers = [torch.cuda.Stream(), torch.cuda.Stream()]
+    monkeypatch.setenv("FAIRRING_INLINE_BYTES", str(MiB))
     dev = fa.DeviceFairring(0)
+    warm = torch.zeros(MiB, device=DEV)
+    for s_ in producers:                                  # first calls take milliseconds: not in the mix
+        dev.allreduce(warm[:4096], [warm[:4096], warm[4096:8192]], stream=s_).wait()
+        dev.allreduce(warm, [warm, warm], stream=s_).wait()
+        _hold(s_, ballast[0], times=2)
+    dev.synchronize()
     torch.cuda.synchronize()
-    try:
-        works = []
-        for step in range(60):
-            if rng.random() < 0.2:
-                dev.synchronize()                         # lets the pipeline run empty
-                torch.cuda.synchronize()
-            small = rng.random() < 0.6
-            n = int(rng.integers(1024, 200_000)) if small else int(rng.integers(MiB, 3 * MiB))
-            which = int(rng.integers(2))
+    before = dev.progress()
+    submitted = 0
+
+    def submit(small, which):
+        n = int(rng.integers(256, 50_000)) if small else int(rng.integers(100_000, 500_000))
+        ob = int(rng.integers(2))                          # two of the buffers take the results,
+        olo = int(rng.integers(0, size - n)) // 4 * 4      # so that ranges meet often
+        k = int(rng.integers(2, 5))
+        terms = []
+        for _ in range(k):
             if rng.random() < 0.3:
-                _hold(producers[which], ballast[which], times=8)
-            ob = int(rng.integers(nbuf))
-            olo = int(rng.integers(0, size - n)) // 4 * 4
-            k = int(rng.integers(2, 5))
-            terms = []
-            for _ in range(k):
-                if rng.random() < 0.3:
-                    terms.append((ob, olo))
-                    continue
-                while True:
-                    cb = int(rng.integers(nbuf))
-                    clo = int(rng.integers(0, size - n)) // 4 * 4
-                    if cb != ob or clo + n <= olo or olo + n <= clo:
-                        break
-                terms.append((cb, clo))
-            scale = float(rng.choice([0.5, 0.25, 1.0, 2.0]))
-            works.append(dev.allreduce(bufs[ob][olo:olo + n],
-                                       [bufs[b][lo:lo + n] for b, lo in terms],
-                                       scale_mode=fa.SCALE_MUL, scale=scale,
-                                       stream=producers[which]))
-            acc = shadow[terms[0][0]][terms[0][1]:terms[0][1] + n].clone()
-            for b, lo in terms[1:]:
-                acc.add_(shadow[b][lo:lo + n])
-            acc.mul_(scale)
-            shadow[ob][olo:olo + n] = acc
-        for w in works:
-            w.wait()
+                terms.append((ob, olo))
+                continue
+            while True:
+                cb = int(rng.integers(nbuf))
+                clo = int(rng.integers(0, size - n)) // 4 * 4
+                if cb != ob or clo + n <= olo or olo + n <= clo:
+                    break
+            terms.append((cb, clo))
+        scale = float(rng.choice([0.5, 0.25, 1.0, 2.0]))
+        w = dev.allreduce(bufs[ob][olo:olo + n], [bufs[b][lo:lo + n] for b, lo in terms],
+                          scale_mode=fa.SCALE_MUL, scale=scale, stream=producers[which])
+        acc = shadow[terms[0][0]][terms[0][1]:terms[0][1] + n].clone()
+        for b, lo in terms[1:]:
+            acc.add_(shadow[b][lo:lo + n])
+        acc.mul_(scale)
+        shadow[ob][olo:olo + n] = acc
+        return w
+
+    try:
+        for episode in range(30):
+            dev.synchronize()                              # the pipeline runs empty
+            torch.cuda.synchronize()
+            first = int(rng.integers(2))
+            _hold(producers[first], ballast[first], times=20)
+            works = [submit(True, first)]
+            for _ in range(int(rng.integers(1, 5))):
+                which = int(rng.integers(2))
+                if rng.random() < 0.2:
+                    _hold(producers[which], ballast[which], times=10)
+                works.append(submit(rng.random() < 0.5, which))
+            submitted += len(works)
+            for w in works:
+                w.wait()
         dev.synchronize()
         torch.cuda.synchronize()
         done = dev.progress()
-        assert 0 < done["on_callers_stream"] < done["submitted"] == 60
         for i in range(nbuf):
             assert bool(torch.equal(bufs[i].view(torch.int32), shadow[i].view(torch.int32))), i
+        assert done["submitted"] - before["submitted"] == submitted
+        # every episode's first operation at least
+        assert 30 <= done["on_callers_stream"] - before["on_callers_stream"] < submitted
     finally:
         dev.close()
