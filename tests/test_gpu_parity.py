@@ -470,51 +470,61 @@ def test_pipeline_many_small_operations_in_order():
     dev.close()
 
 
-def test_operations_sharing_a_tensor_keep_their_order_across_streams():
-    # Bucket-sized operations alternate between the reduce streams. Operations that share a
-    # tensor must still run in submission order: six in-place reductions of one 20 M-element
-    # tensor (80 MiB, several launches each, long enough to overlap if nothing orders them),
-    # each with a scale of its own so that the order shows in the bits; then the output of one
-    # operation as a contribution of the next, and an operation that overwrites a contribution
-    # of the one before. None is waited for until the end.
-    _print_case("order between operations")
-    k, n = 4, 20_000_003
+@pytest.mark.parametrize("n", [6_553_600 + 3, 14_000_003, 20_000_003])
+def test_operations_sharing_a_tensor_keep_their_order_across_streams(n):
+    # Bucket-sized operations (25 MiB: a few launches on one reduce stream, the next operation on
+    # the other) and larger ones (53 and 76 MiB: launches dealt over both streams) that share a
+    # tensor must run in submission order: six in-place reductions of one tensor, each with a scale
+    # of its own so that the order shows in the bits; then the output of one operation as a
+    # contribution of the next, and an operation that overwrites a contribution of the one before.
+    # The calls are marshalled beforehand and issued back to back (a few microseconds apart, a
+    # fraction of what one of them runs), and none is waited for until the end: whatever is not
+    # ordered overlaps.
+    _print_case("order between operations", n)
+    k = 4
     g = torch.Generator(device=DEV)
     g.manual_seed(61)
     xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
     own = xs[0].clone()
     dev = fa.DeviceFairring(0)
-    torch.cuda.synchronize()
-    scales = [0.5, 0.25, 2.0, 1.0, 4.0, 0.125]
-    works = [dev.allreduce(own, [own] + xs[1:], scale_mode=fa.SCALE_MUL, scale=s) for s in scales]
-    works[-1].wait()            # covers the earlier ones: they share its tensor
-    want = xs[0].clone()
-    for s in scales:
-        for x in xs[1:]:
-            want.add_(x)
-        want.mul_(s)
-    assert bool(torch.equal(own.view(torch.int32), want.view(torch.int32)))
-    lo, hi = n - 70_001, n
-    acc = xs[0][lo:hi].cpu().numpy()
-    host = [x[lo:hi].cpu().numpy() for x in xs[1:]]
-    for s in scales:
-        acc = oracle.sum_f32([acc] + host, oracle.SCALE_MUL, s)
-    assert_bits_equal(own[lo:hi].cpu().numpy(), acc)
-    # read after write, then write after read
-    mid = torch.zeros(n, device=DEV)
-    out = torch.zeros(n, device=DEV)
-    spare = xs[3].clone()
-    w1 = dev.allreduce(mid, xs)                       # mid = x0 + x1 + x2 + x3
-    w2 = dev.allreduce(out, [mid, spare])             # reads mid
-    w3 = dev.allreduce(spare, [xs[1], xs[2]])         # overwrites what w2 reads
-    for w in (w1, w2, w3):
-        w.wait()
-    want_mid = xs[0] + xs[1]
-    want_mid.add_(xs[2]).add_(xs[3])
-    assert bool(torch.equal(mid.view(torch.int32), want_mid.view(torch.int32)))
-    assert bool(torch.equal(out.view(torch.int32), (want_mid + xs[3]).view(torch.int32)))
-    assert bool(torch.equal(spare.view(torch.int32), (xs[1] + xs[2]).view(torch.int32)))
-    dev.close()
+    try:
+        scales = [0.5, 0.25, 2.0, 1.0, 4.0, 0.125]
+        calls = [dev.prepare(own, [own] + xs[1:], scale_mode=fa.SCALE_MUL, scale=s) for s in scales]
+        warm = torch.zeros(n, device=DEV)
+        dev.allreduce(warm, [warm, warm]).wait()      # the first launch loads the code object
+        torch.cuda.synchronize()
+        works = [call() for call in calls]
+        works[-1].wait()            # covers the earlier ones: they share its tensor
+        want = xs[0].clone()
+        for s_ in scales:
+            for x in xs[1:]:
+                want.add_(x)
+            want.mul_(s_)
+        assert bool(torch.equal(own.view(torch.int32), want.view(torch.int32)))
+        lo, hi = n - 70_001, n
+        acc = xs[0][lo:hi].cpu().numpy()
+        host = [x[lo:hi].cpu().numpy() for x in xs[1:]]
+        for s_ in scales:
+            acc = oracle.sum_f32([acc] + host, oracle.SCALE_MUL, s_)
+        assert_bits_equal(own[lo:hi].cpu().numpy(), acc)
+        # read after write, then write after read
+        mid = torch.zeros(n, device=DEV)
+        out = torch.zeros(n, device=DEV)
+        spare = xs[3].clone()
+        calls = [dev.prepare(mid, xs),                        # mid = x0 + x1 + x2 + x3
+                 dev.prepare(out, [mid, spare]),              # reads mid
+                 dev.prepare(spare, [xs[1], xs[2]])]          # overwrites what the second reads
+        torch.cuda.synchronize()
+        works = [call() for call in calls]
+        for w in works:
+            w.wait()
+        want_mid = xs[0] + xs[1]
+        want_mid.add_(xs[2]).add_(xs[3])
+        assert bool(torch.equal(mid.view(torch.int32), want_mid.view(torch.int32)))
+        assert bool(torch.equal(out.view(torch.int32), (want_mid + xs[3]).view(torch.int32)))
+        assert bool(torch.equal(spare.view(torch.int32), (xs[1] + xs[2]).view(torch.int32)))
+    finally:
+        dev.close()
 
 
 def test_pipeline_empty_tensor_and_layout_errors():
@@ -850,24 +860,28 @@ def test_stream_of_buckets_keeps_one_shape_and_switches_only_after_a_run_of_alig
 
 @pytest.mark.parametrize("seed", range(6))
 def test_random_sequences_of_dependent_operations_match_sequential_execution(seed):
-    # Operations over ranges of a few shared buffers, submitted back to back without a wait: every
+    # Operations over ranges of a few shared buffers, issued back to back without a wait: every
     # read-after-write, write-after-read and write-after-write between them must resolve as if they
-    # ran one after the other, whichever reduce streams they land on. Ranges are 1 to 6 MiB, so
-    # neighbouring operations do overlap in time when nothing orders them.
+    # ran one after the other, whichever reduce streams they land on. Ranges are 8 to 40 MiB and
+    # the calls are marshalled beforehand, so that an operation runs for several times the gap to
+    # the next call and neighbouring operations do overlap when nothing orders them.
     _print_case("random dependent operations", seed)
     rng = np.random.default_rng(9100 + seed)
-    nbuf, size = 5, 6 * MiB // 4 * 3                      # five buffers of 18 MiB
+    nbuf, size = 5, 16 * MiB                              # five buffers of 64 MiB
     g = torch.Generator(device=DEV)
     g.manual_seed(9100 + seed)
     bufs = [torch.empty(size, device=DEV).normal_(0, 1.0, generator=g) for _ in range(nbuf)]
     shadow = [b.clone() for b in bufs]                    # the sequential execution, by torch
     streams = int(rng.choice([2, 3]))
     dev = fa.DeviceFairring(0, num_reduce_streams=streams)
-    torch.cuda.synchronize()
     try:
-        works = []
+        dev.allreduce(shadow[0][:MiB], [shadow[0][:MiB], shadow[1][:MiB]],
+                      scale_mode=fa.SCALE_MUL, scale=1.0).wait()     # loads the code object
+        shadow[0][:MiB] = bufs[0][:MiB] + bufs[1][:MiB]
+        shadow[0][:MiB] = bufs[0][:MiB]
+        calls, plan = [], []
         for _ in range(50):
-            n = int(rng.integers(MiB // 4, 6 * MiB // 4))
+            n = int(rng.integers(2 * MiB, 10 * MiB))
             ob = int(rng.integers(nbuf))
             olo = int(rng.integers(0, size - n)) // 4 * 4
             k = int(rng.integers(2, 6))
@@ -883,9 +897,12 @@ def test_random_sequences_of_dependent_operations_match_sequential_execution(see
                         break
                 terms.append((cb, clo))
             scale = float(rng.choice([0.5, 0.25, 1.0, 2.0]))
-            out = bufs[ob][olo:olo + n]
-            works.append(dev.allreduce(out, [bufs[b][lo:lo + n] for b, lo in terms],
-                                       scale_mode=fa.SCALE_MUL, scale=scale))
+            calls.append(dev.prepare(bufs[ob][olo:olo + n], [bufs[b][lo:lo + n] for b, lo in terms],
+                                     scale_mode=fa.SCALE_MUL, scale=scale))
+            plan.append((n, ob, olo, terms, scale))
+        torch.cuda.synchronize()
+        works = [call() for call in calls]
+        for n, ob, olo, terms, scale in plan:
             acc = shadow[terms[0][0]][terms[0][1]:terms[0][1] + n].clone()
             for b, lo in terms[1:]:
                 acc.add_(shadow[b][lo:lo + n])
