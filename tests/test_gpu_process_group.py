@@ -568,3 +568,59 @@ def test_waiting_on_every_bucket_orders_the_consumer_after_all_of_them(consumer)
     assert all(same)
     pg._synchronize()
     torch.cuda.synchronize()
+
+
+def test_collectives_issued_back_to_back_on_one_tensor_run_in_order():
+    """No wait between them, as with any c10d backend. An in-place allreduce of
+    a 64 MiB tensor is followed at once by one of its last quarter (which would
+    otherwise start on the other reduce stream while the first is still at the
+    front of the tensor), three times over; then a reduce-scatter whose output's
+    tail is allreduced at once."""
+    print("[case] pg back-to-back collectives on one tensor", flush=True)
+    size, rank, n = 4, 1, 16 * MiB
+    m = n // 4
+    g = torch.Generator(device=DEV)
+    g.manual_seed(44)
+    peers = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(size - 1)]
+    tails = [p[n - m:] for p in peers]
+    own = torch.empty(n, device=DEV).normal_(0, 0.01, generator=g)
+    start = own.clone()
+    pg = make_pg(rank, size, slice_bytes=25 * MiB)
+    pg._set_simulated_peer_contributions(peers)
+    warm = torch.zeros(n, device=DEV)
+    pg.allreduce([warm]).wait()                       # the first launch loads the code object
+    torch.cuda.synchronize()
+
+    def fold(mine, others):                           # rank order: peer 0, this rank, peers 1 and 2
+        acc = others[0] + mine
+        return acc.add_(others[1]).add_(others[2])
+
+    works = []
+    for _ in range(3):
+        pg._set_simulated_peer_contributions(peers)
+        works.append(pg.allreduce([own]))
+        pg._set_simulated_peer_contributions(tails)
+        works.append(pg.allreduce([own[n - m:]]))
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    want = start
+    for _ in range(3):
+        want = fold(want, peers)
+        want[n - m:] = fold(want[n - m:], tails)
+    assert bool(torch.equal(own.view(torch.int32), want.view(torch.int32)))
+
+    whole = torch.empty(size * n, device=DEV).normal_(0, 0.01, generator=g)
+    out = torch.zeros(n, device=DEV)
+    torch.cuda.synchronize()
+    pg._set_simulated_peer_contributions(peers)
+    w1 = pg._reduce_scatter_base(out, whole, dist.ReduceScatterOptions())
+    pg._set_simulated_peer_contributions(tails)
+    w2 = pg.allreduce([out[n - m:]])
+    w1.wait()
+    w2.wait()
+    torch.cuda.synchronize()
+    want = fold(whole[rank * n:(rank + 1) * n], peers)
+    want[n - m:] = fold(want[n - m:], tails)
+    assert bool(torch.equal(out.view(torch.int32), want.view(torch.int32)))
+    pg._synchronize()
