@@ -369,23 +369,36 @@ def test_pipeline_host_staged_half_types_round_once(kind, tdt, slots, carry, cha
     dev.close()
 
 
-def test_pipeline_waits_for_producer_stream():
-    _print_case("pipeline producer stream")
-    n = 4_000_000
+@pytest.mark.parametrize("producer", ["side", "default"])
+@pytest.mark.parametrize("n", [4_000_000, 50_000])
+def test_pipeline_waits_for_producer_stream(producer, n):
+    # The contributions are written late by the producer stream (a few milliseconds of other work
+    # first); the operation is handed over at once and must see them. 4 M elements go through the
+    # reduce streams (the producer's event), 50 K are launched on the producer stream itself. One
+    # call of each kind beforehand: a first call takes longer than the producer is busy.
+    _print_case("pipeline producer stream", producer, n)
     dev = fa.DeviceFairring(0, slice_size_in_bytes=MiB, max_memory_allocated_in_bytes=4 * MiB)
-    side = torch.cuda.Stream()
+    stream = torch.cuda.Stream() if producer == "side" else torch.cuda.default_stream()
     a = torch.zeros(n, device=DEV)
     b = torch.zeros(n, device=DEV)
     out = torch.empty(n, device=DEV)
-    torch.cuda.synchronize()
-    with torch.cuda.stream(side):
-        for _ in range(20):  # a long tail of producer work on a side stream
+    ballast = torch.zeros(64 * MiB, device=DEV)
+    try:
+        with torch.cuda.stream(stream):
+            ballast.add_(1.0)
+            a.add_(0.0)
+            dev.allreduce(out, [a, b]).wait()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            for _ in range(30):
+                ballast.add_(1.0)
             a.add_(1.0)
             b.add_(2.0)
-        w = dev.allreduce(out, [a, b])
-    w.wait()
-    assert bool((out == 60.0).all())
-    dev.close()
+            w = dev.allreduce(out, [a, b])
+        w.wait()
+        assert bool((out == 3.0).all())
+    finally:
+        dev.close()
 
 
 @pytest.mark.parametrize("k,slots", [(1, 2), (2, 2), (5, 1), (9, 2), (9, 3), (12, 8), (64, 2)])
