@@ -234,8 +234,10 @@ def roofline_from_records(recs, bytes_per_elem, full_launch_elems, how):
     the recorded launches divided by the time during which at least one of them
     was running (the union of the recorded intervals); avg_launch_us and
     concurrency (sum of durations / union) are reported beside it, so that
-    achieved = launch_bytes * concurrency / avg_launch (up to the ragged last
-    launch of a step)."""
+    achieved = launch_bytes * concurrency / avg_launch. launch_bytes is the
+    mean over the recorded launches (a bucket stream's launches are cut from
+    runs of buckets, so they are not all of the planned size of a lone
+    operation, which is reported as launch_elems)."""
     durs = [r[1] - r[0] for r in recs]
     launches = sum(r[5] for r in recs)
     elems = sum(r[2] for r in recs)
@@ -244,7 +246,8 @@ def roofline_from_records(recs, bytes_per_elem, full_launch_elems, how):
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-        "launch_bytes": full_launch_elems * bytes_per_elem, "launch_elems": full_launch_elems,
+        "launch_bytes": int(round(elems * bytes_per_elem / max(launches, 1))),
+        "launch_elems": full_launch_elems,
         "avg_launch_us": round(sum(durs) / launches * 1e3, 3), "launches_timed": launches,
         "concurrency": round(sum(durs) / busy_ms, 3),
         "streams_used": len({r[4] for r in recs}),

@@ -104,7 +104,7 @@ def lib():
         fn.argtypes = [vp]
     L.frg_work_block_stream.argtypes = [vp, vp]
     L.frg_set_wait_timeout.argtypes = [ctypes.c_double]
-    L.frg_get_progress.argtypes = [vp, ctypes.POINTER(ctypes.c_int64 * 5)]
+    L.frg_get_progress.argtypes = [vp, ctypes.POINTER(ctypes.c_int64 * 6)]
     L.frg_set_profiling.argtypes = [vp, i32]
     L.frg_kernel_times.argtypes = [vp, ctypes.POINTER(ctypes.c_float), i32, ctypes.POINTER(i32)]
     L.frg_launch_records.argtypes = [vp, ctypes.POINTER(LaunchRecord), i32, ctypes.POINTER(i32)]

@@ -298,6 +298,7 @@ int frg_get_progress(frg_ctx* ctx, frg_progress* out) {
   out->enqueued = p.enqueued.load();
   out->launches = p.launches.load();
   out->on_callers_stream = p.onCallersStream.load();
+  out->merged = p.merged.load();
   return FRG_OK;
 }
 

@@ -98,23 +98,49 @@ bool spinFor(F&& ready) {
 
 }  // namespace
 
-void CommandQueue::enqueue(std::function<void()> fn) {
+void CommandQueue::push(Command c) {
   {
     std::unique_lock<std::mutex> lock(mutex_);
-    fns_.push_back(std::move(fn));
+    entries_.push_back(std::move(c));
     pending_.fetch_add(1, std::memory_order_release);
   }
   cv_.notify_one();
 }
 
-std::function<void()> CommandQueue::dequeue() {
+void CommandQueue::enqueue(std::function<void()> fn) { push(Command{std::move(fn), nullptr}); }
+
+void CommandQueue::enqueue(std::shared_ptr<QueuedOp> op) { push(Command{nullptr, std::move(op)}); }
+
+CommandQueue::Command CommandQueue::dequeue() {
   spinFor([&] { return pending_.load(std::memory_order_acquire) > 0; });
   std::unique_lock<std::mutex> lock(mutex_);
-  cv_.wait(lock, [&] { return !fns_.empty(); });
-  std::function<void()> fn = std::move(fns_.front());
-  fns_.pop_front();
+  cv_.wait(lock, [&] { return !entries_.empty(); });
+  Command c = std::move(entries_.front());
+  entries_.pop_front();
   pending_.fetch_sub(1, std::memory_order_relaxed);
-  return fn;
+  return c;
+}
+
+std::vector<std::shared_ptr<QueuedOp>> CommandQueue::takeRun(
+    const QueuedOp& first, const std::function<bool(const QueuedOp&, const QueuedOp&)>& continues,
+    int atLeast, int atMost) {
+  std::vector<std::shared_ptr<QueuedOp>> run;
+  if (pending_.load(std::memory_order_acquire) < atLeast) return run;
+  std::unique_lock<std::mutex> lock(mutex_);
+  size_t n = 0;
+  const QueuedOp* previous = &first;
+  while (n < entries_.size() && static_cast<int>(n) < atMost && entries_[n].op &&
+         continues(*previous, *entries_[n].op)) {
+    previous = entries_[n].op.get();
+    ++n;
+  }
+  if (static_cast<int>(n) < atLeast) return run;
+  for (size_t i = 0; i < n; ++i) {
+    run.push_back(std::move(entries_.front().op));
+    entries_.pop_front();
+  }
+  pending_.fetch_sub(static_cast<int64_t>(n), std::memory_order_relaxed);
+  return run;
 }
 
 namespace {
@@ -286,6 +312,10 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   if (const char* v = std::getenv("FAIRRING_IDLE_PRODUCER_CHECK")) {
     c->idleProducerCheck_ = std::atoi(v) != 0;
   }
+  if (const char* v = std::getenv("FAIRRING_MERGE_OPERATIONS")) {
+    const long long m = std::atoll(v);
+    if (m >= 1 && m <= 1024) c->mergeOperations_ = static_cast<int>(m);
+  }
   if (const char* v = std::getenv("FAIRRING_INLINE_BYTES")) {
     const long long b = std::atoll(v);
     if (b >= 0) c->inlineTrafficBytes_ = b;
@@ -342,9 +372,37 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->thread_ = std::thread([c] {
     (void)hipSetDevice(c->device_);
     while (true) {
-      std::function<void()> fn = c->queue_.dequeue();
-      if (!fn) return;
-      fn();
+      CommandQueue::Command cmd = c->queue_.dequeue();
+      if (cmd.op) {
+        // Neighbouring operations that are already waiting run as one: what
+        // limits a stream of buckets is the ragged ends of each, and a run of
+        // them has only two.
+        // Only a run of several: launches cut from ranges of ever-changing
+        // length (one bucket, then two, then one) run slower than either kind.
+        std::vector<std::shared_ptr<QueuedOp>> group{std::move(cmd.op)};
+        if (c->mergeOperations_ > 1) {
+          int direction = 0;
+          int64_t bytes = group[0]->req.numel * elementSize(group[0]->req.dtype);
+          std::vector<std::shared_ptr<QueuedOp>> more = c->queue_.takeRun(
+              *group[0],
+              [&](const QueuedOp& previous, const QueuedOp& next) {
+                const int64_t nextBytes = next.req.numel * elementSize(next.req.dtype);
+                if (bytes + nextBytes > kMaxMergedBytes ||
+                    !c->adjoins(previous, next, bytes, &direction)) {
+                  return false;
+                }
+                bytes += nextBytes;
+                return true;
+              },
+              kMinMergedOperations - 1, c->mergeOperations_ - 1);
+          for (auto& op : more) group.push_back(std::move(op));
+        }
+        c->runGroup(group);
+      } else if (cmd.fn) {
+        cmd.fn();
+      } else {
+        return;
+      }
     }
   });
   *out = c;
@@ -353,7 +411,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
 
 Context::~Context() {
   if (thread_.joinable()) {
-    queue_.enqueue(nullptr);
+    queue_.enqueue(std::function<void()>());
     thread_.join();
   }
   // Everything submitted has been enqueued; let it finish before the pool goes.
@@ -846,7 +904,11 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     work->refs.fetch_add(1);
     *workOut = work;
   }
-  queue_.enqueue([this, req = std::move(req), initial, work]() { run(req, initial, work); });
+  auto queued = std::make_shared<QueuedOp>();
+  queued->req = std::move(req);
+  queued->initial = initial;
+  queued->work = work;
+  queue_.enqueue(std::move(queued));
   return FRG_OK;
 }
 
@@ -1082,9 +1144,21 @@ void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fir
 // size (or one per slice of fairring/device.cc:315-326 when asked for), dealt
 // round-robin to the reduce streams so that neighbouring launches overlap.
 // Returns the streams the operation's work ended on.
-std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t initialEvent) {
+std::vector<hipStream_t> Context::runResident(const Request& req,
+                                              const std::vector<hipEvent_t>& initialEvents,
+                                              int64_t slices) {
   const int64_t elsize = elementSize(req.dtype);
-  const int64_t nSlices = numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
+  const int64_t nSlices =
+      slices >= 0 ? slices : numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
+  std::vector<char> initialsFired(initialEvents.size(), 0);
+  // the first launch on a stream follows every producer's event
+  auto waitInitials = [&](hipStream_t stream) {
+    for (size_t i = 0; i < initialEvents.size(); ++i) {
+      bool fired = initialsFired[i] != 0;
+      waitInitial(stream, initialEvents[i], &fired);
+      initialsFired[i] = fired ? 1 : 0;
+    }
+  };
   const size_t nStreams = reduceStreams_.size();
   std::vector<char> waited(nStreams, 0);
   std::vector<const void*> ptrs(req.contribs.size());
@@ -1103,7 +1177,6 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   const int64_t launchBytes = shape.bytes;
   const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;
   size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
-  bool initialFired = false;
   // Reduced in place into a contribution that only a later launch of the chain
   // reads: the partial result must not land in `out` before that.
   bool lateAlias = false;
@@ -1216,7 +1289,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
     if (!waited[si]) {
       // Only the first launch on a stream needs the producer's event; later
       // ones follow it in stream order (fairring/device.cc:334-336,507-509).
-      waitInitial(s, initialEvent, &initialFired);
+      waitInitials(s);
       waited[si] = 1;
     }
     for (size_t k = 0; k < ptrs.size(); ++k) {
@@ -1275,7 +1348,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req, hipEvent_t ini
   }
   // The streams that took part, the one of the last launch at the back.
   if (!waited[lastIdx]) {
-    waitInitial(reduceStreams_[lastIdx], initialEvent, &initialFired);
+    waitInitials(reduceStreams_[lastIdx]);
     waited[lastIdx] = 1;
   }
   std::vector<hipStream_t> used;
@@ -1426,17 +1499,104 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
   return {s};
 }
 
-void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
-  const int64_t seq = nextSeq_++;
-  progress_->started.fetch_add(1);
+// Whether `next`, which was submitted right after `last`, continues it: the
+// same reduction over buffers that lie directly below (direction -1) or above
+// (+1) those of `last`, output and every contribution alike, so that the two
+// are one elementwise operation over the joint range. `bytesSoFar`: the length
+// of the run that ends in `last`; `*direction` is 0 until the first pair has
+// set it.
+bool Context::adjoins(const QueuedOp& last, const QueuedOp& next, int64_t bytesSoFar,
+                      int* direction) {
+  const Request& a = last.req;
+  const Request& b = next.req;
+  if (!launchBytesByContribs_ || a.fromHost || b.fromHost || a.compressed || b.compressed) {
+    return false;
+  }
+  if (a.dtype != b.dtype || a.op != b.op || a.scaleMode != b.scaleMode || a.scale != b.scale ||
+      a.contribs.size() != b.contribs.size() || a.numel <= 0 || b.numel <= 0 ||
+      a.contribs.size() > static_cast<size_t>(kMaxContribsPerLaunch)) {
+    return false;
+  }
+  const uintptr_t elsize = static_cast<uintptr_t>(elementSize(a.dtype));
+  const uintptr_t aBytes = static_cast<uintptr_t>(a.numel) * elsize;
+  const uintptr_t bBytes = static_cast<uintptr_t>(b.numel) * elsize;
+  const uintptr_t ao = reinterpret_cast<uintptr_t>(a.out);
+  const uintptr_t bo = reinterpret_cast<uintptr_t>(b.out);
+  int dir = 0;
+  if (bo + bBytes == ao) dir = -1;
+  if (ao + aBytes == bo) dir = +1;
+  if (dir == 0 || (*direction != 0 && dir != *direction)) return false;
+  for (size_t k = 0; k < a.contribs.size(); ++k) {
+    const uintptr_t ap = reinterpret_cast<uintptr_t>(a.contribs[k]);
+    const uintptr_t bp = reinterpret_cast<uintptr_t>(b.contribs[k]);
+    if (dir < 0 ? bp + bBytes != ap : ap + aBytes != bp) return false;
+    // Over the joint range a contribution is the output itself or apart from
+    // it: operations of which one reads what another writes are not one. Every
+    // operation of the run has the same distance between the two, so the
+    // question is whether that distance is shorter than the run.
+    const uintptr_t distance = ap > ao ? ap - ao : ao - ap;
+    if (distance != 0 && distance < static_cast<uintptr_t>(bytesSoFar) + bBytes) return false;
+  }
+  if (allocationBase(a.out) != allocationBase(b.out)) return false;
+  *direction = dir;
+  return true;
+}
+
+// One operation, or several neighbours as one (see adjoins()): enqueues the
+// launches, then marks every work and calls every callback, in submission order.
+void Context::runGroup(const std::vector<std::shared_ptr<QueuedOp>>& group) {
+  const size_t count = group.size();
+  const int64_t firstSeq = nextSeq_;
+  nextSeq_ += static_cast<int64_t>(count);
+  progress_->started.fetch_add(static_cast<int64_t>(count));
+  if (count > 1) progress_->merged.fetch_add(static_cast<int64_t>(count));
   int status = FRG_OK;
   std::string error;
   hipStream_t lastStream = reduceStreams_[0];
+  std::vector<hipStream_t> used;
   try {
-    std::vector<hipStream_t> used =
-        req.fromHost ? runHostStaged(req, initialEvent) : runResident(req, initialEvent);
+    const Request* req = &group[0]->req;
+    Request joint;
+    int64_t slices = -1;
+    if (count > 1) {
+      // the joint range starts where the lowest of them does
+      const QueuedOp* lowest = group[0].get();
+      const int64_t elsize = elementSize(req->dtype);
+      slices = 0;
+      int64_t numel = 0;
+      for (const auto& op : group) {
+        if (op->req.out < lowest->req.out) lowest = op.get();
+        numel += op->req.numel;
+        slices += numSlices(op->req.numel, layout_.sliceSizeInBytes, elsize);
+      }
+      joint = lowest->req;
+      joint.numel = numel;
+      joint.done = nullptr;
+      joint.user = nullptr;
+      req = &joint;
+    }
+    // what the producers recorded: of one stream's events the last covers the others
+    std::vector<hipEvent_t> initials;
+    std::vector<hipStream_t> producers;
+    bool anyCallback = false;
+    for (const auto& op : group) {
+      anyCallback = anyCallback || op->req.done != nullptr;
+      if (op->initial == nullptr) continue;
+      size_t at = producers.size();
+      for (size_t i = 0; i < producers.size(); ++i) {
+        if (producers[i] == op->req.producerStream) at = i;
+      }
+      if (at == producers.size()) {
+        producers.push_back(op->req.producerStream);
+        initials.push_back(op->initial);
+      } else {
+        initials[at] = op->initial;
+      }
+    }
+    used = req->fromHost ? runHostStaged(*req, initials.empty() ? nullptr : initials[0])
+                         : runResident(*req, initials, slices);
     lastStream = used.back();
-    if (req.done != nullptr && used.size() > 1) {
+    if (anyCallback && used.size() > 1) {
       // The callback orders consumers after ONE stream (fairring/device.cc:337-340
       // marks the future under a guard of the last stream): join the others into it.
       for (size_t i = 0; i + 1 < used.size(); ++i) {
@@ -1449,6 +1609,22 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
     }
     // Without a callback nothing needs a single stream, and the streams keep
     // running independently of each other.
+  } catch (const ContractFailure& e) {
+    status = e.code;
+    error = e.what();
+    used.clear();
+  } catch (const std::exception& e) {
+    status = FRG_ERR_HIP;
+    error = e.what();
+    used.clear();
+  }
+  if (status != FRG_OK) {
+    std::fprintf(stderr, "[fairring] operation #%lld%s failed: %s\n",
+                 static_cast<long long>(firstSeq), count > 1 ? " (and its neighbours)" : "",
+                 error.c_str());
+  }
+  for (const auto& op : group) {
+    Work* work = op->work;
     work->doneStreams = used;
     // where the operation stands on each of them, for waits that are remembered
     for (hipStream_t s : used) {
@@ -1463,30 +1639,20 @@ void Context::run(const Request& req, hipEvent_t initialEvent, Work* work) {
       work->doneIndices.push_back(idx);
       work->donePositions.push_back(position);
     }
-  } catch (const ContractFailure& e) {
-    status = e.code;
-    error = e.what();
-  } catch (const std::exception& e) {
-    status = FRG_ERR_HIP;
-    error = e.what();
+    if (op->initial != nullptr) giveEvent(op->initial);
+    progress_->enqueued.fetch_add(1);
+    {
+      std::lock_guard<std::mutex> g(work->mu);
+      work->status = status;
+      work->error = error;
+      work->lastStream = lastStream;
+      work->enqueued = true;
+      work->enqueuedFlag.store(true, std::memory_order_release);
+    }
+    work->cv.notify_all();
+    if (op->req.done) op->req.done(op->req.user, status, lastStream);
+    releaseWork(work);
   }
-  if (status != FRG_OK) {
-    std::fprintf(stderr, "[fairring] operation #%lld failed: %s\n",
-                 static_cast<long long>(seq), error.c_str());
-  }
-  if (initialEvent != nullptr) giveEvent(initialEvent);
-  progress_->enqueued.fetch_add(1);
-  {
-    std::lock_guard<std::mutex> g(work->mu);
-    work->status = status;
-    work->error = error;
-    work->lastStream = lastStream;
-    work->enqueued = true;
-    work->enqueuedFlag.store(true, std::memory_order_release);
-  }
-  work->cv.notify_all();
-  if (req.done) req.done(req.user, status, lastStream);
-  releaseWork(work);
 }
 
 int Context::synchronize(std::string* err) {

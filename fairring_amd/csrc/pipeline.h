@@ -21,20 +21,38 @@
 
 namespace frg {
 
-// Unbounded FIFO of closures drained by one thread; an empty function is the
-// shutdown token (fairring/utils.h:329-351, fairring/device.cc:275-283).
+struct QueuedOp;  // a submitted operation on its way to the command thread
+constexpr int64_t kMaxMergedBytes = 512ll << 20;
+constexpr int kMinMergedOperations = 4;
+
+// Unbounded FIFO drained by one thread: closures, and operations, which the
+// thread may look ahead at (it runs neighbouring ones that are already waiting
+// as one). An entry with neither is the shutdown token (fairring/utils.h:329-351,
+// fairring/device.cc:275-283).
 class CommandQueue {
  public:
+  struct Command {
+    std::function<void()> fn;
+    std::shared_ptr<QueuedOp> op;
+  };
   void enqueue(std::function<void()> fn);
+  void enqueue(std::shared_ptr<QueuedOp> op);
   // Polls for a short while before it sleeps: a sleeping thread takes tens of
   // microseconds to wake, which is most of what a small operation costs.
-  std::function<void()> dequeue();
+  Command dequeue();
+  // Takes the run of operations at the head of which each continues the one
+  // before (`continues(previous, next)`, the first against `first`), at most
+  // `atMost` of them, but only if there are at least `atLeast`; never waits.
+  std::vector<std::shared_ptr<QueuedOp>> takeRun(
+      const QueuedOp& first, const std::function<bool(const QueuedOp&, const QueuedOp&)>& continues,
+      int atLeast, int atMost);
 
  private:
+  void push(Command c);
   std::mutex mutex_;
   std::condition_variable cv_;
-  std::deque<std::function<void()>> fns_;
-  std::atomic<int64_t> pending_{0};  // closures enqueued and not yet taken
+  std::deque<Command> entries_;
+  std::atomic<int64_t> pending_{0};  // entries enqueued and not yet taken
 };
 
 // Progress counters of a context, shared with the works it hands out so that a
@@ -46,6 +64,7 @@ struct Progress {
   std::atomic<int64_t> enqueued{0};   // operations whose GPU work is all enqueued
   std::atomic<int64_t> launches{0};   // kernel launches issued
   std::atomic<int64_t> onCallersStream{0};  // operations launched by submit() on the producer stream
+  std::atomic<int64_t> merged{0};           // operations run together with a neighbour that was waiting
   // Per reduce stream: how many operations it has been given, and up to which
   // of them the device's null stream already waits (the null stream is never
   // destroyed, so what it was once told to wait for stays waited for: a step's
@@ -139,10 +158,16 @@ class Context {
  private:
   Context() = default;
 
-  void run(const Request& req, hipEvent_t initialEvent, Work* work);
+  void runGroup(const std::vector<std::shared_ptr<QueuedOp>>& group);
+  bool adjoins(const QueuedOp& last, const QueuedOp& next, int64_t bytesSoFar, int* direction);
   // Both return the streams the operation's work ended on, the last one used
   // at the back.
-  std::vector<hipStream_t> runResident(const Request& req, hipEvent_t initialEvent);
+  // `initialEvents`: what the producers recorded (one operation: at most one);
+  // `slices` >= 0 overrides the count of slices the operation advances the
+  // slot cursor by (several operations run as one keep their own counts).
+  std::vector<hipStream_t> runResident(const Request& req,
+                                       const std::vector<hipEvent_t>& initialEvents,
+                                       int64_t slices);
   std::vector<hipStream_t> runHostStaged(const Request& req, hipEvent_t initialEvent);
   // Makes `stream` wait for `initialEvent` unless that event has already fired.
   void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
@@ -226,6 +251,12 @@ class Context {
   // reduce streams costs two cross-stream waits of 6 to 13 us of host time each
   // (producer -> reduce stream, reduce stream -> consumer), several times what
   // the kernel takes. FAIRRING_INLINE_BYTES overrides it (0: never).
+  // Operations waiting in the queue whose buffers continue one another's (the
+  // buckets of one gradient, handed over faster than they run) are run as one
+  // operation over the whole range: at least kMinMergedOperations, at most this
+  // many at a time (FAIRRING_MERGE_OPERATIONS; 1: never) and kMaxMergedBytes of
+  // output.
+  int mergeOperations_ = 16;
   int64_t inlineTrafficBytes_ = 16ll << 20;
   // After a reduce stream answered "busy" the rule is not tried again before this time.
   static constexpr int64_t kInlineRetryNs = 200 * 1000;
@@ -305,5 +336,12 @@ void setWaitTimeout(double seconds);
 
 void setLastError(const std::string& msg);
 const char* lastError();
+
+// What submit() hands to the command thread.
+struct QueuedOp {
+  Context::Request req;
+  hipEvent_t initial = nullptr;  // recorded on the producer stream, or null if that was idle
+  Work* work = nullptr;
+};
 
 }  // namespace frg

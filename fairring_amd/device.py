@@ -359,12 +359,13 @@ class DeviceFairring:
 
     def progress(self):
         """Operations submitted / started / fully enqueued, kernel launches
-        issued, and operations launched by the call itself on the producer
-        stream (small ones, with nothing in flight), so far."""
-        out = (ctypes.c_int64 * 5)()
+        issued, operations launched by the call itself on the producer stream
+        (small ones, with nothing in flight) and operations run as one with
+        neighbours that were waiting in the queue, so far."""
+        out = (ctypes.c_int64 * 6)()
         _capi.check(_capi.lib().frg_get_progress(self._h, ctypes.byref(out)))
         return dict(submitted=out[0], started=out[1], enqueued=out[2], launches=out[3],
-                    on_callers_stream=out[4])
+                    on_callers_stream=out[4], merged=out[5])
 
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))

@@ -292,7 +292,17 @@ typedef void (*frg_done_fn)(void* user, int status, void* last_stream);
  * launch. Its completion is then ordered on `producer_stream`
  * (frg_work_block_stream on that stream is free); whatever this context is
  * handed afterwards from another stream is ordered after it with an event, and
- * frg_synchronize covers it. */
+ * frg_synchronize covers it.
+ * Operations that wait in the queue while the command thread is busy and
+ * continue one another (the same reduction over buffers that lie directly
+ * below or above the previous operation's, output and every contribution
+ * alike: the buckets of one gradient, handed over faster than they run) are
+ * run as one operation over the joint range, 4 to 16 at a time
+ * (FAIRRING_MERGE_OPERATIONS sets the upper limit, 1 switches this off): a
+ * bucket's launches have ragged ends, a run of buckets has only two. Every
+ * operation keeps its own work handle and callback (called in submission
+ * order); all of the run complete together. Operations of which one reads what
+ * another writes are never joined. */
 FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
                           int K, int64_t numel, int dtype, int op,
                           int scale_mode, float scale, void* producer_stream,
@@ -346,6 +356,7 @@ typedef struct frg_progress {
   int64_t enqueued;
   int64_t launches;
   int64_t on_callers_stream;
+  int64_t merged; /* operations run as one with neighbours that were waiting (see frg_allreduce) */
 } frg_progress;
 FRG_API int frg_get_progress(frg_ctx* ctx, frg_progress* out);
 

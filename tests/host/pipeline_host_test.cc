@@ -6,6 +6,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <condition_variable>
 #include <cstdio>
 #include <cstdlib>
 #include <chrono>
@@ -660,6 +661,205 @@ void scenarioNullStreamRemembersItsWaits() {
   CHECK(hipStreamDestroy(consumer) == hipSuccess);
 }
 
+// A completion callback that holds the command thread until the test lets go.
+struct Gate {
+  std::mutex mu;
+  std::condition_variable cv;
+  bool open = false;
+  bool reached = false;
+};
+void waitAtGate(void* user, int, void*) {
+  auto* g = static_cast<Gate*>(user);
+  std::unique_lock<std::mutex> lock(g->mu);
+  g->reached = true;
+  g->cv.notify_all();
+  g->cv.wait(lock, [&] { return g->open; });
+}
+struct Order {
+  std::mutex mu;
+  std::vector<int> seen;
+};
+struct OrderNote {
+  Order* order;
+  int index;
+};
+void noteOrder(void* user, int status, void*) {
+  auto* n = static_cast<OrderNote*>(user);
+  std::lock_guard<std::mutex> g(n->order->mu);
+  n->order->seen.push_back(status == FRG_OK ? n->index : -1);
+}
+
+void scenarioNeighboursRunAsOne() {
+  std::puts("operations that are waiting and continue one another run as one");
+  const int64_t piece = 3000, pieces = 8;
+  for (int variant = 0; variant < 4; ++variant) {
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    // one tensor per contribution, cut into pieces like a gradient into buckets
+    auto c = randomContribs(3, piece * pieces, 90 + variant);
+    Vec out(piece * pieces, -1.f);
+    Vec own = c[0];
+    // hold the command thread in the callback of an operation of its own
+    Gate gate;
+    auto other = randomContribs(2, 100, 99);
+    Vec otherOut(100);
+    auto ot = table(other);
+    CHECK(frg_allreduce(ctx, otherOut.data(), ot.data(), 2, 100, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                        1.f, nullptr, &waitAtGate, &gate, nullptr) == FRG_OK);
+    {
+      std::unique_lock<std::mutex> lock(gate.mu);
+      gate.cv.wait(lock, [&] { return gate.reached; });
+    }
+    frg_progress before = {};
+    CHECK(frg_get_progress(ctx, &before) == FRG_OK);
+    Order order;
+    std::vector<OrderNote> notes(pieces);
+    std::vector<frg_work*> w(pieces, nullptr);
+    for (int i = 0; i < pieces; ++i) {
+      // variant 0: from the end of the tensor to its start (DDP's order), a separate output;
+      // 1: from start to end, in place into the first contribution; 2: the order changes
+      // direction half way; 3: every second piece, then the others (nothing continues anything)
+      int at = variant == 1 ? i : pieces - 1 - i;
+      if (variant == 2 && i >= 4) at = i - 4;                      // 7 6 5 4, then 0 1 2 3
+      if (variant == 3) at = i < 4 ? 2 * i : 2 * (i - 4) + 1;      // 0 2 4 6 1 3 5 7
+      const int64_t off = at * piece;
+      const void* tab[3] = {variant == 1 ? own.data() + off : c[0].data() + off,
+                            c[1].data() + off, c[2].data() + off};
+      float* dst = variant == 1 ? own.data() + off : out.data() + off;
+      notes[i] = OrderNote{&order, i};
+      CHECK(frg_allreduce(ctx, dst, tab, 3, piece, FRG_F32, FRG_SUM, FRG_SCALE_MUL, 0.5f, nullptr,
+                          &noteOrder, &notes[i], &w[i]) == FRG_OK);
+    }
+    {
+      std::lock_guard<std::mutex> lock(gate.mu);
+      gate.open = true;
+    }
+    gate.cv.notify_all();
+    for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
+    CHECK(frg_synchronize(ctx) == FRG_OK);
+    frg_progress after = {};
+    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    CHECK(after.enqueued - before.enqueued == pieces);
+    if (variant <= 1) {
+      CHECK(after.merged - before.merged == pieces);           // one run of eight
+      CHECK(after.launches - before.launches < pieces);        // cut from the joint range
+    } else if (variant == 2) {
+      CHECK(after.merged - before.merged == pieces);           // two runs of four
+    } else {
+      CHECK(after.merged == before.merged);
+      CHECK(after.launches - before.launches >= pieces);
+    }
+    const Vec want = fold(c, FRG_SCALE_MUL, 0.5f);
+    CHECK(same(variant == 1 ? own : out, want));
+    {
+      std::lock_guard<std::mutex> g(order.mu);
+      CHECK(static_cast<int>(order.seen.size()) == pieces);
+      for (int i = 0; i < pieces; ++i) CHECK(order.seen[i] == i);  // callbacks in submission order
+    }
+    for (frg_work* x : w) frg_work_release(x);
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+  // Two operations that continue one another but each read what the other
+  // writes are not one elementwise operation: they stay apart, and in order.
+  {
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    const int64_t n = 2000;
+    Vec z(3 * n);
+    for (int64_t i = 0; i < 3 * n; ++i) z[i] = static_cast<float>(i % 97) * 0.25f;
+    const Vec z0 = z;
+    Gate gate;
+    auto other = randomContribs(2, 100, 98);
+    Vec otherOut(100);
+    auto ot = table(other);
+    CHECK(frg_allreduce(ctx, otherOut.data(), ot.data(), 2, 100, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                        1.f, nullptr, &waitAtGate, &gate, nullptr) == FRG_OK);
+    {
+      std::unique_lock<std::mutex> lock(gate.mu);
+      gate.cv.wait(lock, [&] { return gate.reached; });
+    }
+    frg_progress before = {};
+    CHECK(frg_get_progress(ctx, &before) == FRG_OK);
+    // pieces of n/4 from the top of z[n, 2n) downwards, each written from the piece n below it
+    // and added to itself: z[n + j] += z[j]; the four would join into z[n, 2n) += z[0, n),
+    // fine; then the same one step further down, z[j] += z[j - ...] is what must not join:
+    // here output z[n/2 + ...] reads z[...] that a neighbour writes
+    std::vector<frg_work*> w;
+    const int64_t q = n / 4;
+    for (int i = 0; i < 4; ++i) {
+      // output piece [2n - (i+1)q, 2n - iq), contribution one piece lower: [.. - q, ..)
+      float* dst = z.data() + 2 * n - (i + 1) * q;
+      const void* tab[2] = {dst, dst - q};  // in place, plus the piece directly below
+      frg_work* x = nullptr;
+      CHECK(frg_allreduce(ctx, dst, tab, 2, q, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f, nullptr,
+                          nullptr, nullptr, &x) == FRG_OK);
+      w.push_back(x);
+    }
+    {
+      std::lock_guard<std::mutex> lock(gate.mu);
+      gate.open = true;
+    }
+    gate.cv.notify_all();
+    for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
+    frg_progress after = {};
+    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    CHECK(after.merged == before.merged);
+    // sequentially: piece i adds the ORIGINAL piece below it (that one is updated only later)
+    Vec want = z0;
+    for (int i = 0; i < 4; ++i) {
+      const int64_t lo = 2 * n - (i + 1) * q;
+      for (int64_t j = 0; j < q; ++j) want[lo + j] = want[lo + j] + want[lo - q + j];
+    }
+    CHECK(same(z, want));
+    for (frg_work* x : w) frg_work_release(x);
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+  // The same with the contribution four and a half pieces below the output:
+  // a run of four neighbours is apart from what it reads, a run of five is not,
+  // so the eight waiting operations run as two runs of four.
+  {
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    const int64_t q = 500, count = 8, gap = 9 * q / 2;
+    Vec z(gap + count * q);
+    for (size_t i = 0; i < z.size(); ++i) z[i] = static_cast<float>(i % 89) * 0.5f;
+    const Vec z0 = z;
+    Gate gate;
+    auto other = randomContribs(2, 100, 97);
+    Vec otherOut(100);
+    auto ot = table(other);
+    CHECK(frg_allreduce(ctx, otherOut.data(), ot.data(), 2, 100, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                        1.f, nullptr, &waitAtGate, &gate, nullptr) == FRG_OK);
+    {
+      std::unique_lock<std::mutex> lock(gate.mu);
+      gate.cv.wait(lock, [&] { return gate.reached; });
+    }
+    std::vector<frg_work*> w;
+    for (int i = 0; i < count; ++i) {   // from the top down; each adds what lies `gap` below it
+      float* dst = z.data() + gap + (count - 1 - i) * q;
+      const void* tab[2] = {dst, dst - gap};
+      frg_work* x = nullptr;
+      CHECK(frg_allreduce(ctx, dst, tab, 2, q, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f, nullptr,
+                          nullptr, nullptr, &x) == FRG_OK);
+      w.push_back(x);
+    }
+    {
+      std::lock_guard<std::mutex> lock(gate.mu);
+      gate.open = true;
+    }
+    gate.cv.notify_all();
+    for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
+    frg_progress after = {};
+    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    CHECK(after.merged == count);
+    Vec want = z0;
+    for (int i = 0; i < count; ++i) {
+      const int64_t lo = gap + (count - 1 - i) * q;
+      for (int64_t j = 0; j < q; ++j) want[lo + j] = want[lo + j] + want[lo - gap + j];
+    }
+    CHECK(same(z, want));
+    for (frg_work* x : w) frg_work_release(x);
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
 void scenarioProducerOrdering() {
   std::puts("the pipeline waits for the producer stream");
   frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
@@ -1251,6 +1451,7 @@ void runAll() {
       {"wait gives up", scenarioWaitGivesUp},
       {"block stream gives up", scenarioBlockStreamGivesUp},
       {"idle producer", scenarioIdleProducer},
+      {"neighbours run as one", scenarioNeighboursRunAsOne},
       {"the null stream remembers its waits", scenarioNullStreamRemembersItsWaits},
       {"small operations on the caller's stream", scenarioSmallOperationsOnTheCallersStream},
       {"producer ordering", scenarioProducerOrdering},

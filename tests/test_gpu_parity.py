@@ -1092,3 +1092,75 @@ def test_random_mix_of_small_and_large_operations_from_two_streams(seed, monkeyp
         assert 30 <= done["on_callers_stream"] - before["on_callers_stream"] < submitted
     finally:
         dev.close()
+
+
+@pytest.mark.parametrize("order", ["descending", "ascending", "in_place"])
+def test_neighbouring_buckets_waiting_in_the_queue_run_as_one(order):
+    # A gradient handed over bucket by bucket faster than the buckets run (calls marshalled
+    # beforehand, issued a few microseconds apart): the command thread finds runs of buckets that
+    # continue one another waiting in its queue and cuts its launches from their joint range.
+    # Every bucket still completes, and the result is the one of running them separately.
+    _print_case("neighbouring buckets run as one", order)
+    k, bucket, count = 4, 6_553_600, 40                      # 40 buckets of 25 MiB: 1 GB per tensor
+    n = bucket * count + 12_345                              # and a ragged first one
+    g = torch.Generator(device=DEV)
+    g.manual_seed(17)
+    xs = [torch.empty(n, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    want = (xs[0] + xs[1]).add_(xs[2]).add_(xs[3]).mul_(0.25)
+    out = xs[0].clone() if order == "in_place" else torch.zeros(n, device=DEV)
+    spans = [(n - 12_345, n)] + [(n - 12_345 - (i + 1) * bucket, n - 12_345 - i * bucket)
+                                 for i in range(count)]
+    if order == "ascending":
+        spans.reverse()
+    dev = fa.DeviceFairring(0)
+    try:
+        calls = [dev.prepare(out[lo:hi], ([out[lo:hi]] if order == "in_place" else [xs[0][lo:hi]])
+                             + [x[lo:hi] for x in xs[1:]], scale_mode=fa.SCALE_MUL, scale=0.25)
+                 for lo, hi in spans]
+        warm = torch.zeros(bucket, device=DEV)
+        dev.allreduce(warm, [warm, warm]).wait()
+        torch.cuda.synchronize()
+        before = dev.progress()
+        works = [call() for call in calls]
+        for w in works:
+            assert w.wait() is True
+        after = dev.progress()
+        assert after["enqueued"] - before["enqueued"] == len(spans)
+        assert after["merged"] - before["merged"] >= 8       # most of them, in practice
+        assert bool(torch.equal(out.view(torch.int32), want.view(torch.int32)))
+        lo, hi = n - 100_000, n
+        assert_bits_equal(out[lo:hi].cpu().numpy(),
+                          oracle.sum_f32([x[lo:hi].cpu().numpy() for x in xs], oracle.SCALE_MUL, 0.25))
+    finally:
+        dev.close()
+
+
+def test_neighbouring_operations_that_read_each_others_output_stay_apart():
+    # z[i] += z[i - gap], bucket by bucket from the top down, with the gap four and a half buckets:
+    # up to four neighbours are one elementwise operation, five are not (the fifth writes what the
+    # first reads). Run one after the other, every bucket adds the ORIGINAL values below it.
+    _print_case("neighbouring operations with a hazard")
+    q, count = 2 * MiB, 24
+    gap = 9 * q // 2
+    g = torch.Generator(device=DEV)
+    g.manual_seed(18)
+    z = torch.empty(gap + count * q, device=DEV).normal_(0, 1.0, generator=g)
+    want = z.clone()
+    for i in range(count):
+        lo = gap + (count - 1 - i) * q
+        want[lo:lo + q] = want[lo:lo + q] + want[lo - gap:lo - gap + q]
+    dev = fa.DeviceFairring(0)
+    try:
+        calls = []
+        for i in range(count):
+            lo = gap + (count - 1 - i) * q
+            calls.append(dev.prepare(z[lo:lo + q], [z[lo:lo + q], z[lo - gap:lo - gap + q]]))
+        warm = torch.zeros(q, device=DEV)
+        dev.allreduce(warm, [warm, warm]).wait()
+        torch.cuda.synchronize()
+        works = [call() for call in calls]
+        for w in works:
+            w.wait()
+        assert bool(torch.equal(z.view(torch.int32), want.view(torch.int32)))
+    finally:
+        dev.close()
