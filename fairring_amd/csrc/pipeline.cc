@@ -394,7 +394,9 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
                 bytes += nextBytes;
                 return true;
               },
-              kMinMergedOperations - 1, c->mergeOperations_ - 1);
+              (c->mergeOperations_ < kMinMergedOperations ? c->mergeOperations_
+                                                           : kMinMergedOperations) - 1,
+              c->mergeOperations_ - 1);
           for (auto& op : more) group.push_back(std::move(op));
         }
         c->runGroup(group);
