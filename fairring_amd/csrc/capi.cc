@@ -376,6 +376,6 @@ int frg_set_tuning(int blocks_per_cu) {
 
 const char* frg_last_error(void) { return frg::lastError(); }
 
-const char* frg_version(void) { return "0.1"; }
+const char* frg_version(void) { return "0.2"; }
 
 }  // extern "C"

@@ -422,7 +422,8 @@ FRG_API int frg_set_tuning(int blocks_per_cu);
 /* Message of the last failure on the calling thread (or of the failed work). */
 FRG_API const char* frg_last_error(void);
 
-/* "major.minor" of this ABI. */
+/* "major.minor" of this ABI. 0.2: frg_progress grew (on_callers_stream, merged);
+ * frg_plan_launches, frg_get_copy_streams, frg_reduce_slice_static added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus
