@@ -151,7 +151,7 @@ def test_c_client_builds_and_fails_cleanly_without_a_gpu(tmp_path):
     if torch.cuda.is_available():
         assert r.returncode == 0 and "abi client ok" in r.stdout, r.stderr
     else:
-        assert r.returncode == 2 and "abi 0.1" in r.stdout     # the HIP runtime finds no device
+        assert r.returncode == 2 and "abi 0.2" in r.stdout     # the HIP runtime finds no device
 
 
 def test_a_missing_library_is_a_loud_error_not_a_fallback(tmp_path):
