@@ -1391,9 +1391,20 @@ void scenarioDestroyWithPendingWork() {
   frg_work_release(w);
 }
 
+void concurrentSubmitters(frg_ctx* ctx);
+
 void scenarioConcurrentSubmitters() {
   std::puts("several threads submit to one context");
-  frg_ctx* ctx = makeCtx(8192, 4096, 2, 1024);
+  concurrentSubmitters(makeCtx(8192, 4096, 2, 1024));
+  // the same with the library's own partition, small operations on the callers'
+  // streams and neighbours joined: whatever path an operation takes
+  setenv("FAIRRING_INLINE_BYTES", "65536", 1);
+  frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+  setenv("FAIRRING_INLINE_BYTES", "0", 1);
+  concurrentSubmitters(ctx);
+}
+
+void concurrentSubmitters(frg_ctx* ctx) {
   std::vector<std::thread> threads;
   std::atomic<int> ok{0};
   for (int tix = 0; tix < 4; ++tix) {
