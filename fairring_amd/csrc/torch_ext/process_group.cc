@@ -144,7 +144,11 @@ void completeFuture(const OpState& st, const c10::intrusive_ptr<c10::ivalue::Fut
   }
 }
 
-// Runs on the pipeline's command thread once the last slice is enqueued.
+// Runs once the last slice is enqueued: on the pipeline's command thread, or on
+// the caller's (inside frg_allreduce, before the Work exists) for a small
+// operation launched on the caller's stream. What the caller handed in is let
+// go of here: from now on its memory is protected by stream order (the
+// caller's own stream) or by what was recorded on the reduce streams.
 void onEnqueued(void* user, int status, void* lastStream) {
   std::unique_ptr<std::shared_ptr<OpState>> holder(static_cast<std::shared_ptr<OpState>*>(user));
   OpState& st = **holder;
