@@ -900,6 +900,9 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     *err = e.what();
     if (initial) giveEvent(initial);
     releaseWork(work);
+    // counted as dealt with: the counters stay level for what comes after
+    progress_->started.fetch_add(1);
+    progress_->enqueued.fetch_add(1);
     return FRG_ERR_HIP;
   }
   if (workOut) {
