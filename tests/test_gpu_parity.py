@@ -1164,3 +1164,51 @@ def test_neighbouring_operations_that_read_each_others_output_stay_apart():
         assert bool(torch.equal(z.view(torch.int32), want.view(torch.int32)))
     finally:
         dev.close()
+
+
+@pytest.mark.parametrize("dtype,op,scaled", [(torch.bfloat16, "sum", True), (torch.float16, "sum", False),
+                                             (torch.int32, "max", False), (torch.float64, "sum", True)])
+def test_joined_neighbours_give_the_bits_of_separate_operations(dtype, op, scaled, monkeypatch):
+    # Whatever the element type and operator: a run of buckets that is executed as one operation
+    # leaves the bits that the buckets leave one by one (FAIRRING_MERGE_OPERATIONS=1).
+    _print_case("joined neighbours, other types", dtype, op)
+    k, bucket, count = 5, 3_000_000, 24
+    n = bucket * count
+    g = torch.Generator(device=DEV)
+    g.manual_seed(23)
+    if dtype == torch.int32:
+        xs = [torch.randint(-2**30, 2**30, (n,), device=DEV, dtype=dtype, generator=g) for _ in range(k)]
+    else:
+        xs = [torch.empty(n, device=DEV, dtype=torch.float32).normal_(0, 1.0, generator=g).to(dtype)
+              for _ in range(k)]
+    kwargs = dict(op=fa.MAX if op == "max" else fa.SUM)
+    if scaled:
+        kwargs.update(scale_mode=fa.SCALE_MUL, scale=0.25)
+    spans = [(n - (i + 1) * bucket, n - i * bucket) for i in range(count)]
+    outs = []
+    for limit in ("16", "1"):
+        monkeypatch.setenv("FAIRRING_MERGE_OPERATIONS", limit)
+        dev = fa.DeviceFairring(0)
+        try:
+            out = torch.zeros(n, device=DEV, dtype=dtype)
+            calls = [dev.prepare(out[lo:hi], [x[lo:hi] for x in xs], **kwargs) for lo, hi in spans]
+            dev.allreduce(out[:bucket], [x[:bucket] for x in xs], **kwargs).wait()
+            out.zero_()
+            torch.cuda.synchronize()
+            before = dev.progress()["merged"]
+            works = [call() for call in calls]
+            for w in works:
+                w.wait()
+            joined = dev.progress()["merged"] - before
+            assert (joined >= 4) if limit == "16" else (joined == 0)
+            outs.append(out)
+        finally:
+            dev.close()
+    a, b = (o.view(torch.int16 if o.element_size() == 2 else (torch.int32 if o.element_size() == 4
+                                                              else torch.int64)) for o in outs)
+    assert bool(torch.equal(a, b))
+    lo, hi = 0, 50_000
+    host = [x[lo:hi].cpu() for x in xs]
+    if dtype == torch.int32:
+        want = torch.stack(host).amax(dim=0)
+        assert bool(torch.equal(outs[0][lo:hi].cpu(), want))
