@@ -1119,14 +1119,20 @@ def test_neighbouring_buckets_waiting_in_the_queue_run_as_one(order):
                  for lo, hi in spans]
         warm = torch.zeros(bucket, device=DEV)
         dev.allreduce(warm, [warm, warm]).wait()
+        # something for the command thread to do meanwhile (some hundred launches), so that the
+        # buckets are waiting when it gets to them however slow this thread is today
+        busy = torch.zeros(256 * MiB, device=DEV)
+        occupy = dev.prepare(busy, [busy, busy])
         torch.cuda.synchronize()
         before = dev.progress()
+        occupied = occupy()
         works = [call() for call in calls]
         for w in works:
             assert w.wait() is True
+        occupied.wait()
         after = dev.progress()
-        assert after["enqueued"] - before["enqueued"] == len(spans)
-        assert after["merged"] - before["merged"] >= 8       # most of them, in practice
+        assert after["enqueued"] - before["enqueued"] == len(spans) + 1
+        assert after["merged"] - before["merged"] >= 8       # nearly all of them, in practice
         assert bool(torch.equal(out.view(torch.int32), want.view(torch.int32)))
         lo, hi = n - 100_000, n
         assert_bits_equal(out[lo:hi].cpu().numpy(),
@@ -1194,11 +1200,15 @@ def test_joined_neighbours_give_the_bits_of_separate_operations(dtype, op, scale
             calls = [dev.prepare(out[lo:hi], [x[lo:hi] for x in xs], **kwargs) for lo, hi in spans]
             dev.allreduce(out[:bucket], [x[:bucket] for x in xs], **kwargs).wait()
             out.zero_()
+            busy = torch.zeros(256 * MiB, device=DEV)      # keeps the command thread at work
+            occupy = dev.prepare(busy, [busy, busy])       # while the buckets queue up
             torch.cuda.synchronize()
             before = dev.progress()["merged"]
+            occupied = occupy()
             works = [call() for call in calls]
             for w in works:
                 w.wait()
+            occupied.wait()
             joined = dev.progress()["merged"] - before
             assert (joined >= 4) if limit == "16" else (joined == 0)
             outs.append(out)
