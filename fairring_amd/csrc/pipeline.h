@@ -261,6 +261,10 @@ class Context {
   // After a reduce stream answered "busy" the rule is not tried again before this time.
   static constexpr int64_t kInlineRetryNs = 200 * 1000;
   std::atomic<int64_t> inlineRetryAtNs_{0};
+  // Operations the command thread has taken up, and the value of that count
+  // when the reduce streams were last found idle.
+  std::atomic<int64_t> pipelineOps_{0};
+  std::atomic<int64_t> idleConfirmedAt_{-1};
   // The last such launch: an event recorded behind it and the stream it went
   // to (kept for comparison only, never used after the call that set it).
   // Whatever is submitted from another stream is ordered after that event.

@@ -554,8 +554,12 @@ void scenarioSmallOperationsOnTheCallersStream() {
     fake_hip_occupy(p, 60);
     CHECK(frg_allreduce(ctx, own.data(), tab, 3, n, FRG_F32, FRG_SUM, FRG_SCALE_MUL, 0.5f, p,
                         nullptr, nullptr, &w0) == FRG_OK);
+    // the reduce streams were found idle for the first and nothing has gone to them since:
+    // the second does not ask again
+    const long asked = fake_hip_calls("hipStreamQuery");
     CHECK(frg_allreduce(ctx, own.data(), tab, 3, n, FRG_F32, FRG_SUM, FRG_SCALE_MUL, 0.25f, q,
                         nullptr, nullptr, &w1) == FRG_OK);
+    CHECK(fake_hip_calls("hipStreamQuery") == asked);
     CHECK(frg_work_wait(w1) == FRG_OK);
     CHECK(same(own, want));
     frg_work_release(w0);
