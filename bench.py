@@ -373,6 +373,11 @@ def run_resident(args, np, torch, fa, oracle, dtype, keep=None):
     return value, elapsed, cfg, roof, checked, base, dtype
 
 
+def _capi_lib():
+    from fairring_amd import _capi
+    return _capi.lib()
+
+
 def run_c3(args, np, torch, fa, oracle):
     """Server-side accumulation: K = 64 contributions of one 25 MiB fp32 slice in
     pinned host memory, staged through the pool and folded in order."""
@@ -400,12 +405,41 @@ def run_c3(args, np, torch, fa, oracle):
     value = step_bytes * args.steps / elapsed / 1e9
     link = k * numel * 4 * args.steps / elapsed / 1e9
     slots = dev.layout["staging_slots"]
-    batch = max(1, slots // 2)
+    batch = max(1, slots // max(1, len(dev._external_streams(_capi_lib().frg_get_copy_streams))))
+    # What the link gives to bare copies in this run: hipMemcpyAsync (torch's non-blocking
+    # copy_ from pinned memory is that call) of the same pinned buffers into two device
+    # buffers of a slice's size, on the pipeline's own copy streams in turn, nothing else running.
+    copy_streams = dev._external_streams(_capi_lib().frg_get_copy_streams)
+    land = [torch.empty(numel, dtype=torch.float32, device="cuda:0") for _ in copy_streams]
+
+    def bare_copies(streams, rounds):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(rounds):
+            for i, h in enumerate(hs):
+                with torch.cuda.stream(streams[i % len(streams)]):
+                    land[i % len(streams)].copy_(h, non_blocking=True)
+        torch.cuda.synchronize()
+        return k * numel * 4 * rounds / (time.perf_counter() - t0) / 1e9
+
+    bare_copies(copy_streams, 1)
+    ceiling = max(bare_copies(copy_streams, 2), bare_copies(copy_streams[:1], 2))
     # the accumulate kernel of a batch reads `batch` staged slots and `out`, writes `out`
     recs = per_launch_pass(fa, args, step)
     recs = [r for r in recs if r[3] == batch]
-    roof = roofline_from_records(recs, (batch + 2) * 4, numel, LAUNCH_HOW)
-    roof["kernel"] = "ksumKernel<F32Vec, SUM, carry, K=%d>" % batch
+    hbm = roofline_from_records(recs, (batch + 2) * 4, numel, LAUNCH_HOW)
+    hbm["kernel"] = "ksumKernel<F32Vec, SUM, carry, K=%d>" % batch
+    roof = {
+        "bound": "host_link", "achieved": round(link, 2), "peak": round(ceiling, 2),
+        "nominal": 64.0, "unit": "GB/s", "frac": round(link / ceiling, 4), "traffic": None,
+        "how": "achieved: bytes of the K contributions crossing the host link per second of the "
+               "timed region; peak: bare hipMemcpyAsync of the same pinned buffers on the same copy "
+               "streams in this run (best of both streams in turn and one alone); nominal: PCIe "
+               "Gen5 x16 per direction",
+        "kernel": hbm["kernel"],
+        "hbm": {key: hbm[key] for key in ("achieved", "peak", "frac", "launch_bytes",
+                                          "avg_launch_us", "launches_timed")},
+    }
     step(dev).wait()
     want = oracle.sum_f32([h.numpy() for h in hs], oracle.SCALE_MUL, 1.0 / k,
                           threads=os.cpu_count() or 1)
@@ -812,8 +846,9 @@ def main():
                             shared=shared if name in ("c5", "c5pg") else None)
                 # compact: the whole record stays one line of a few KB
                 roof = {key: r["roofline"][key] for key in (
-                    "bound", "achieved", "peak", "unit", "frac", "traffic", "launch_bytes",
-                    "avg_launch_us", "concurrency", "kernel") if key in r["roofline"]}
+                    "bound", "achieved", "peak", "nominal", "unit", "frac", "traffic",
+                    "launch_bytes", "avg_launch_us", "concurrency", "kernel", "hbm")
+                    if key in r["roofline"]}
                 extra[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"],
                                "steps": r["steps"], "ms_per_step": r["ms_per_step"],
                                "dtype": r["dtype"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],

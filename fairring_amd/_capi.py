@@ -20,7 +20,7 @@ EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_plan_launches", "frg_reduce_slice", "frg_reduce_slice_static",
     "frg_reduce_slice_compressed", "frg_allreduce_compressed",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
-    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
+    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
     "frg_set_tuning",
     "frg_last_error", "frg_version",
@@ -104,7 +104,8 @@ def lib():
         fn.argtypes = [vp]
     L.frg_work_block_stream.argtypes = [vp, vp]
     L.frg_set_wait_timeout.argtypes = [ctypes.c_double]
-    L.frg_get_progress.argtypes = [vp, ctypes.POINTER(ctypes.c_int64 * 6)]
+    L.frg_get_progress.argtypes = [vp, ctypes.POINTER(ctypes.c_int64 * 4)]
+    L.frg_get_progress2.argtypes = [vp, ctypes.POINTER(ctypes.c_int64 * 7), ctypes.c_uint64]
     L.frg_set_profiling.argtypes = [vp, i32]
     L.frg_kernel_times.argtypes = [vp, ctypes.POINTER(ctypes.c_float), i32, ctypes.POINTER(i32)]
     L.frg_launch_records.argtypes = [vp, ctypes.POINTER(LaunchRecord), i32, ctypes.POINTER(i32)]

@@ -3,6 +3,8 @@
 #include <string>
 
 #include "../../include/fairring_hip.h"
+#include <cstring>
+
 #include "ksum_kernels.h"
 #include "layout.h"
 #include "pipeline.h"
@@ -297,8 +299,24 @@ int frg_get_progress(frg_ctx* ctx, frg_progress* out) {
   out->started = p.started.load();
   out->enqueued = p.enqueued.load();
   out->launches = p.launches.load();
-  out->on_callers_stream = p.onCallersStream.load();
-  out->merged = p.merged.load();
+  return FRG_OK;
+}
+
+int frg_get_progress2(frg_ctx* ctx, frg_progress2* out, uint64_t size) {
+  if (ctx == nullptr || out == nullptr) return fail(FRG_ERR_INVALID, "null argument");
+  if (size < sizeof(frg_progress) || size % sizeof(int64_t) != 0) {
+    return fail(FRG_ERR_INVALID, "struct size must be a multiple of 8, at least 32");
+  }
+  const frg::Progress& p = asCtx(ctx)->progress();
+  frg_progress2 all = {};
+  all.submitted = p.submitted.load();
+  all.started = p.started.load();
+  all.enqueued = p.enqueued.load();
+  all.launches = p.launches.load();
+  all.on_callers_stream = p.onCallersStream.load();
+  all.merged = p.merged.load();
+  all.segmented_launches = p.segmentedLaunches.load();
+  std::memcpy(out, &all, size < sizeof(all) ? static_cast<size_t>(size) : sizeof(all));
   return FRG_OK;
 }
 
@@ -376,6 +394,6 @@ int frg_set_tuning(int blocks_per_cu) {
 
 const char* frg_last_error(void) { return frg::lastError(); }
 
-const char* frg_version(void) { return "0.2"; }
+const char* frg_version(void) { return "0.3"; }
 
 }  // extern "C"

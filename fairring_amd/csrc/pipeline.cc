@@ -214,45 +214,23 @@ StreamPool& streamPool() {
   return *pool;
 }
 
-// Events for a caller's stream to wait on an operation (frg_work_block_stream):
-// kept per device and never destroyed, since a work handle may outlive its
-// context and creating and destroying an event per wait costs more than the
-// record and the wait themselves. An event goes back as soon as the wait on it
-// is enqueued: the wait holds what it needs of the record.
-class WaitEventPool {
- public:
-  hipEvent_t take(int device) {
-    {
-      std::lock_guard<std::mutex> g(mu_);
-      for (size_t i = 0; i < idle_.size(); ++i) {
-        if (idle_[i].device != device) continue;
-        hipEvent_t e = idle_[i].event;
-        idle_[i] = idle_.back();
-        idle_.pop_back();
-        return e;
-      }
-    }
-    hipEvent_t e;
-    FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-    return e;
-  }
-  void give(int device, hipEvent_t e) {
-    std::lock_guard<std::mutex> g(mu_);
-    idle_.push_back(Entry{e, device});
-  }
+// An event for one record and the waits on it. Every record gets an event of
+// its own, which is destroyed as soon as the waits on it have been enqueued (a
+// wait that is pending keeps what it needs: the runtime releases the event's
+// resources when it has fired). That is what the reference does with its
+// at::cuda::CUDAEvent objects (fairring/device.cc:453-456), and it means that
+// no event is ever recorded a second time, so nothing here depends on how a
+// wait that has been enqueued but not yet executed treats a later record of
+// its event. (Events used to be pooled and recorded again at once; creating
+// and destroying one costs about a microsecond of host time.)
+hipEvent_t newEvent() {
+  hipEvent_t e;
+  FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  return e;
+}
 
- private:
-  struct Entry {
-    hipEvent_t event;
-    int device;
-  };
-  std::mutex mu_;
-  std::vector<Entry> idle_;
-};
-
-WaitEventPool& waitEventPool() {
-  static WaitEventPool* pool = new WaitEventPool();
-  return *pool;
+void retireEvent(hipEvent_t e) {
+  if (e != nullptr) (void)hipEventDestroy(e);
 }
 
 }  // namespace
@@ -338,7 +316,7 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
     // first used (copyStreams()): until then the context holds its reduce
     // streams only.
     c->numCopyStreams_ = o.num_copy_streams > 0 ? (o.num_copy_streams < 4 ? o.num_copy_streams : 4)
-                                                : 2;
+                                                : kDefaultStagingStreams;
     FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->stagingPool_),
                             static_cast<size_t>(c->numSlots_ * c->slotBytes_)));
     // The scratch of the launch chains, here rather than on first use: an
@@ -347,14 +325,6 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
     FRG_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&c->carryScratch_),
                             c->reduceStreams_.size() *
                                 static_cast<size_t>(c->carryScratchBytes_ + 16)));
-    for (int64_t i = 0; i < c->numSlots_; ++i) {
-      hipEvent_t a, b;
-      FRG_HIP_CHECK(hipEventCreateWithFlags(&a, hipEventDisableTiming));
-      FRG_HIP_CHECK(hipEventCreateWithFlags(&b, hipEventDisableTiming));
-      c->slotFreeEvents_.push_back(a);
-      c->slotFilledEvents_.push_back(b);
-    }
-    c->slotUsed_.assign(static_cast<size_t>(c->numSlots_), 0);
     prepareStaticScratch(device);  // for frg_reduce_slice_static; failures are left to that call
     c->streamLaunches_.assign(c->reduceStreams_.size(), 0);
     c->streamElems_.assign(c->reduceStreams_.size(), 0);
@@ -428,9 +398,6 @@ Context::~Context() {
   if (inlineEvent_ != nullptr) (void)hipEventDestroy(inlineEvent_);
   if (stagingPool_) (void)hipFree(stagingPool_);
   if (carryScratch_) (void)hipFree(carryScratch_);
-  for (hipEvent_t e : slotFreeEvents_) (void)hipEventDestroy(e);
-  for (hipEvent_t e : slotFilledEvents_) (void)hipEventDestroy(e);
-  for (hipEvent_t e : freeEvents_) (void)hipEventDestroy(e);
   for (auto& p : profEvents_) {
     (void)hipEventDestroy(p.begin);
     (void)hipEventDestroy(p.end);
@@ -462,23 +429,18 @@ std::vector<hipStream_t> Context::streams() {
   return v;
 }
 
-hipEvent_t Context::takeEvent() {
-  {
-    std::lock_guard<std::mutex> g(eventMu_);
-    if (!freeEvents_.empty()) {
-      hipEvent_t e = freeEvents_.back();
-      freeEvents_.pop_back();
-      return e;
-    }
-  }
-  hipEvent_t e;
-  FRG_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-  return e;
-}
+hipEvent_t Context::takeEvent() { return newEvent(); }
 
-void Context::giveEvent(hipEvent_t e) {
-  std::lock_guard<std::mutex> g(eventMu_);
-  freeEvents_.push_back(e);
+void Context::giveEvent(hipEvent_t e) { retireEvent(e); }
+
+// Retires the event `holder` names, if any, and puts a new one in its place:
+// for the places that keep "the last record" around (a staging slot's free
+// event, the event behind a launch on a caller's stream).
+hipEvent_t Context::freshEvent(hipEvent_t* holder) {
+  hipEvent_t e = newEvent();
+  retireEvent(*holder);
+  *holder = e;
+  return e;
 }
 
 void Context::releaseWork(Work* w) {
@@ -621,10 +583,10 @@ int Context::blockStream(Work* w, hipStream_t stream, std::string* err) {
         if (w->donePositions[i] <= p.nullStreamWaitsFor[idx]) continue;
         upTo = p.streamPosition[idx].load(std::memory_order_acquire);
       }
-      hipEvent_t e = waitEventPool().take(w->device);
+      hipEvent_t e = newEvent();
       hipError_t r = hipEventRecord(e, s);
       if (r == hipSuccess) r = hipStreamWaitEvent(stream, e, 0);
-      waitEventPool().give(w->device, e);
+      retireEvent(e);
       FRG_HIP_CHECK(r);
       if (remember && upTo > p.nullStreamWaitsFor[idx]) p.nullStreamWaitsFor[idx] = upTo;
     }
@@ -644,10 +606,7 @@ void Context::orderAfterInline(hipStream_t producer) {
   if (!inlineRecorded_) {
     // the null stream, which is always there to record on: behind whatever it
     // holds by now, the launch included
-    if (inlineEvent_ == nullptr) {
-      FRG_HIP_CHECK(hipEventCreateWithFlags(&inlineEvent_, hipEventDisableTiming));
-    }
-    FRG_HIP_CHECK(hipEventRecord(inlineEvent_, nullptr));
+    FRG_HIP_CHECK(hipEventRecord(freshEvent(&inlineEvent_), nullptr));
     inlineRecorded_ = true;
   }
   if (hipEventQuery(inlineEvent_) == hipSuccess) {
@@ -717,10 +676,8 @@ bool Context::tryInline(const Request& req, Work* work) {
       // recorded when another stream turns up.
       inlineRecorded_ = req.producerStream != nullptr;
       if (inlineRecorded_) {
-        if (inlineEvent_ == nullptr) {
-          FRG_HIP_CHECK(hipEventCreateWithFlags(&inlineEvent_, hipEventDisableTiming));
-        }
-        FRG_HIP_CHECK(hipEventRecord(inlineEvent_, req.producerStream));
+        // a new event every time: a stream may still be waiting for the last launch's
+        FRG_HIP_CHECK(hipEventRecord(freshEvent(&inlineEvent_), req.producerStream));
       }
       inlineStream_ = req.producerStream;
       inlinePending_ = true;
@@ -1079,7 +1036,7 @@ void Context::joinTail(size_t src, size_t target) {
   hipEvent_t e = takeEvent();
   hipError_t r = hipEventRecord(e, reduceStreams_[src]);
   if (r == hipSuccess) r = hipStreamWaitEvent(reduceStreams_[target], e, 0);
-  giveEvent(e);  // the wait holds what it needs of the record
+  giveEvent(e);
   FRG_HIP_CHECK(r);
   if (!history_[src].empty()) orderedAfter_[target][src] = history_[src].back().seq;
 }
@@ -1373,13 +1330,27 @@ std::vector<hipStream_t> Context::runResident(const Request& req,
   return used;
 }
 
-// Contributions in pinned host memory (server-side accumulation): contribution
-// 0 lands directly in `out`; each later one is copied into the next staging
-// slot on the copy stream as soon as the reduction that last read that slot
-// has finished, and folded into `out` on the reduce stream in index order
-// (slot rule of fairring/device.cc:543-545,587-589; cursor of :482). With four
-// or more slots, half the pool is folded per launch so that copies into the
-// other half overlap it.
+// Contributions in pinned host memory (server-side accumulation,
+// fairring/device.cc:543-589: collect into a staging slot, then reduce).
+// Contribution 0 lands directly in `out`; the later ones are copied into
+// staging slots and folded into `out` in index order.
+//
+// The pool's slots are dealt in groups of `batch` (half the pool from four slots
+// on, else one slot), and every group belongs to one of the staging streams:
+// that stream copies a batch of contributions into the group's slots and then
+// runs the fold that reads them, so a slot is never overwritten before its last
+// reader has finished (the slot rule of device.cc:543-545,587-589) by stream
+// order alone. What crosses streams is the order of the folds: each one waits
+// for an event recorded behind the fold before it, when that ran on another
+// stream. While one stream folds, the other's copies keep the host link busy.
+//
+// (The folds used to run on a reduce stream, with a "filled" event from the copy
+// stream to it and a "free" event back per slot. On MI355X / ROCm 7.2
+// hipMemcpyAsync then held the calling thread up for 0.2 to 0.45 ms per copy, up
+// to 11 ms, whenever the copy stream's last packet was such a wait, so the
+// command thread paced the copies one at a time: 64 contributions of 25 MiB
+// crossed the link at 46 to 50 GB/s. In this form the same call returns in 1.5
+// us and the link runs at what bare copies get, 56 GB/s on the same box.)
 std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   // A staged slice must fit a slot as well as the slice size.
@@ -1387,29 +1358,32 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
       layout_.sliceSizeInBytes < slotBytes_ ? layout_.sliceSizeInBytes : slotBytes_;
   const int K = static_cast<int>(req.contribs.size());
   hipStream_t s = reduceStreams_[0];
-  const std::vector<hipStream_t> copies = copyStreams();  // created on first use
-  // The copy streams write `out` and the slots and know nothing of earlier
+  const std::vector<hipStream_t> all = copyStreams();  // created on first use
+  // the pool is split evenly among the staging streams: each fills its share, then folds it
+  int64_t batch = numSlots_ / static_cast<int64_t>(all.size());
+  if (batch < 1) batch = 1;
+  if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
+  const int64_t groups = numSlots_ / batch;
+  const size_t nStaging = static_cast<int64_t>(all.size()) < groups ? all.size()
+                                                                    : static_cast<size_t>(groups);
+  const std::vector<hipStream_t> staging(all.begin(), all.begin() + static_cast<long>(nStaging));
+  // The staging streams write `out` and the slots and know nothing of earlier
   // operations: the whole operation is ordered after everything enqueued so far
-  // (it is bound by the host link; two event packets do not show).
+  // (it is bound by the host link; a few event packets do not show).
   for (size_t src = 1; src < reduceStreams_.size(); ++src) {
     if (!history_[src].empty()) joinTail(src, 0);
   }
   {
     hipEvent_t tail = takeEvent();
     hipError_t r = hipEventRecord(tail, s);
-    for (hipStream_t cs : copies) {
-      if (r == hipSuccess) r = hipStreamWaitEvent(cs, tail, 0);
+    for (hipStream_t st : staging) {
+      if (r == hipSuccess) r = hipStreamWaitEvent(st, tail, 0);
     }
     giveEvent(tail);
     FRG_HIP_CHECK(r);
   }
   bool initialFired = false;
-  waitInitial(s, initialEvent, &initialFired);
-  for (hipStream_t cs : copies) waitInitial(cs, initialEvent, &initialFired);
-  const size_t nCopy = copies.size();
-  int64_t batch = numSlots_ / 2;
-  if (batch < 1) batch = 1;
-  if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
+  for (hipStream_t st : staging) waitInitial(st, initialEvent, &initialFired);
   // bf16 / fp16 sums folded in more than one batch keep their partial sums in
   // fp32 between the launches (one rounding, like a single launch); the slices
   // are then as short as the scratch buffer that holds those partial sums.
@@ -1420,95 +1394,142 @@ std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t i
   }
   const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
 
-  for (int64_t i = 0; i < nSlices; ++i) {
-    int64_t off, len;
-    sliceBounds(req.numel, sliceBytes, elsize, i, &off, &len);
-    const size_t bytes = static_cast<size_t>(len * elsize);
-    char* outp = static_cast<char*>(req.out) + off * elsize;
-
-    int firstStaged = 0;
-    if (!req.carry) {
-      // contribution 0 needs no staging: it lands in `out` directly
-      FRG_HIP_CHECK(hipMemcpyAsync(outp,
-                                   static_cast<const char*>(req.contribs[0]) + off * elsize,
-                                   bytes, hipMemcpyHostToDevice, copies[0]));
-      hipEvent_t first = takeEvent();
-      FRG_HIP_CHECK(hipEventRecord(first, copies[0]));
-      FRG_HIP_CHECK(hipStreamWaitEvent(s, first, 0));
-      giveEvent(first);
-      firstStaged = 1;
+  // The fold enqueued last, anywhere: the stream it ran on and an event behind it.
+  size_t lastFoldStream = nStaging;  // none yet
+  hipEvent_t lastFold = nullptr;
+  auto orderAfterLastFold = [&](size_t si) {
+    if (lastFold != nullptr && lastFoldStream != si) {
+      FRG_HIP_CHECK(hipStreamWaitEvent(staging[si], lastFold, 0));
     }
+  };
+  auto foldEnqueued = [&](size_t si) {
+    giveEvent(lastFold);
+    lastFold = nullptr;
+    lastFold = takeEvent();
+    lastFoldStream = si;
+    FRG_HIP_CHECK(hipEventRecord(lastFold, staging[si]));
+  };
+  std::vector<char> took(nStaging, 0);
+  try {
+    for (int64_t i = 0; i < nSlices; ++i) {
+      int64_t off, len;
+      sliceBounds(req.numel, sliceBytes, elsize, i, &off, &len);
+      const size_t bytes = static_cast<size_t>(len * elsize);
+      char* outp = static_cast<char*>(req.out) + off * elsize;
 
-    if (K == firstStaged && req.scaleMode != FRG_SCALE_NONE) {
-      // nothing left to fold, but the post-scale is still owed
-      const void* self = outp;
-      ReduceArgs a;
-      a.out = outp;
-      a.contribs = &self;
-      a.K = 1;
-      a.n = len;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = req.scaleMode;
-      a.scale = req.scale;
-      launch(a, s);
-    }
-
-    std::vector<const void*> staged;
-    std::vector<int64_t> slots;
-    char* accBuf = accChain ? scratchFor(0, outp, /*acc=*/true, elsize) : nullptr;
-    bool inAcc = false;  // the partial sum sits in accBuf (fp32), not in `out`
-    for (int k = firstStaged; k < K;) {
-      staged.clear();
-      slots.clear();
-      for (; k < K && static_cast<int64_t>(staged.size()) < batch; ++k) {
-        const int64_t slot = (nextStagingSlot_++) % numSlots_;
-        hipStream_t cs = copies[static_cast<size_t>(slot) % nCopy];
-        if (slotUsed_[slot]) {
-          FRG_HIP_CHECK(hipStreamWaitEvent(cs, slotFreeEvents_[slot], 0));
+      int firstStaged = 0;
+      if (!req.carry) {
+        // Contribution 0 needs no staging: it lands in `out` directly, on the
+        // stream of the group that comes next, behind whatever fold wrote this
+        // part of `out` last (none within this operation: the slices are
+        // disjoint ranges; an earlier operation's is covered by the joins above).
+        const size_t si = static_cast<size_t>((nextStagingSlot_ / batch) % groups) % nStaging;
+        orderAfterLastFold(si);  // keeps the folds of all slices in one chain (they share the scratch)
+        FRG_HIP_CHECK(hipMemcpyAsync(outp,
+                                     static_cast<const char*>(req.contribs[0]) + off * elsize,
+                                     bytes, hipMemcpyHostToDevice, staging[si]));
+        took[si] = 1;
+        firstStaged = 1;
+        if (K == 1) {
+          if (req.scaleMode != FRG_SCALE_NONE) {
+            // nothing left to fold, but the post-scale is still owed
+            const void* self = outp;
+            ReduceArgs a;
+            a.out = outp;
+            a.contribs = &self;
+            a.K = 1;
+            a.n = len;
+            a.dtype = req.dtype;
+            a.op = req.op;
+            a.scale_mode = req.scaleMode;
+            a.scale = req.scale;
+            launch(a, staging[si]);
+          }
+          continue;
         }
-        char* dst = stagingPool_ + slot * slotBytes_;
-        FRG_HIP_CHECK(hipMemcpyAsync(dst,
-                                     static_cast<const char*>(req.contribs[k]) + off * elsize,
-                                     bytes, hipMemcpyHostToDevice, cs));
-        FRG_HIP_CHECK(hipEventRecord(slotFilledEvents_[slot], cs));
-        staged.push_back(dst);
-        slots.push_back(slot);
+        // the first fold of the slice reads what this copy wrote
+        giveEvent(lastFold);
+        lastFold = nullptr;
+        lastFold = takeEvent();
+        lastFoldStream = si;
+        FRG_HIP_CHECK(hipEventRecord(lastFold, staging[si]));
       }
-      // A copy stream is in order, so per copy stream the last slot's event
-      // covers the earlier ones of the batch.
-      for (size_t b = slots.size() > nCopy ? slots.size() - nCopy : 0; b < slots.size(); ++b) {
-        FRG_HIP_CHECK(hipStreamWaitEvent(s, slotFilledEvents_[slots[b]], 0));
-      }
-      ReduceArgs a;
-      a.out = outp;
-      a.contribs = staged.data();
-      a.K = static_cast<int>(staged.size());
-      a.n = len;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = k == K ? req.scaleMode : FRG_SCALE_NONE;
-      a.scale = req.scale;
-      a.carry = true;
-      if (accChain) {
-        a.carry_src = inAcc ? accBuf : outp;
-        a.carry_acc = inAcc;
-        if (k < K) {  // more batches follow
-          a.out = accBuf;
-          a.out_acc = true;
-          inAcc = true;
+
+      std::vector<const void*> staged;
+      char* accBuf = accChain ? scratchFor(0, outp, /*acc=*/true, elsize) : nullptr;
+      bool inAcc = false;  // the partial sum sits in accBuf (fp32), not in `out`
+      for (int k = firstStaged; k < K;) {
+        const int64_t group = (nextStagingSlot_ / batch) % groups;
+        nextStagingSlot_ += batch;  // the rotation of fairring/device.cc:482, a group at a time
+        const size_t si = static_cast<size_t>(group) % nStaging;
+        hipStream_t st = staging[si];
+        const int k0 = k;
+        const int kn = K - k < batch ? K - k : static_cast<int>(batch);
+        k += kn;
+        // Two streams that start their copies together share the link, finish
+        // together and then fold one after the other with the link idle (8 % of
+        // the time with 25 MiB slots). The first batch of every stream but the
+        // first therefore goes in two halves, copy and fold each: from then on
+        // that stream's copies end half a copy apart from its neighbour's, and
+        // one of them is always in flight.
+        int64_t cuts[3] = {0, len, len};
+        int parts = 1;
+        if (si > 0 && !took[si] && bytes >= (4u << 20)) {
+          cuts[1] = len / 2 / (kTileBytes / elsize) * (kTileBytes / elsize);
+          parts = 2;
         }
-      }
-      launch(a, s);
-      for (int64_t slot : slots) {
-        FRG_HIP_CHECK(hipEventRecord(slotFreeEvents_[slot], s));
-        slotUsed_[slot] = 1;
+        took[si] = 1;
+        for (int part = 0; part < parts; ++part) {
+          const int64_t lo = cuts[part], hi = cuts[part + 1];
+          staged.clear();
+          for (int j = 0; j < kn; ++j) {
+            char* dst = stagingPool_ + (group * batch + j) * slotBytes_;
+            FRG_HIP_CHECK(hipMemcpyAsync(
+                dst + lo * elsize,
+                static_cast<const char*>(req.contribs[k0 + j]) + (off + lo) * elsize,
+                static_cast<size_t>((hi - lo) * elsize), hipMemcpyHostToDevice, st));
+            staged.push_back(dst + lo * elsize);
+          }
+          orderAfterLastFold(si);
+          ReduceArgs a;
+          a.out = outp + lo * elsize;
+          a.contribs = staged.data();
+          a.K = kn;
+          a.n = hi - lo;
+          a.dtype = req.dtype;
+          a.op = req.op;
+          a.scale_mode = k == K ? req.scaleMode : FRG_SCALE_NONE;
+          a.scale = req.scale;
+          a.carry = true;
+          if (accChain) {
+            a.carry_src = inAcc ? accBuf + lo * 4 : outp + lo * elsize;
+            a.carry_acc = inAcc;
+            if (k < K) {  // more batches follow
+              a.out = accBuf + lo * 4;
+              a.out_acc = true;
+            }
+          }
+          launch(a, st);
+          foldEnqueued(si);
+        }
+        if (accChain && k < K) inAcc = true;
       }
     }
-    // The next slice's first copy overwrites nothing this slice still reads
-    // (it targets another range of `out`), so no extra wait is needed here.
+    // The operation ends on the first reduce stream, like any other: whatever
+    // comes later is ordered against that.
+    for (size_t si = 0; si < nStaging; ++si) {
+      if (!took[si]) continue;
+      hipEvent_t e = takeEvent();
+      hipError_t r = hipEventRecord(e, staging[si]);
+      if (r == hipSuccess) r = hipStreamWaitEvent(s, e, 0);
+      giveEvent(e);
+      FRG_HIP_CHECK(r);
+    }
+  } catch (...) {
+    giveEvent(lastFold);
+    throw;
   }
-  // every copy of the operation has been joined into the reduce stream
+  giveEvent(lastFold);
   if (req.numel > 0) remember(spansOf(req), {0});
   return {s};
 }
@@ -1616,9 +1637,10 @@ void Context::runGroup(const std::vector<std::shared_ptr<QueuedOp>>& group) {
       // marks the future under a guard of the last stream): join the others into it.
       for (size_t i = 0; i + 1 < used.size(); ++i) {
         hipEvent_t j = takeEvent();
-        FRG_HIP_CHECK(hipEventRecord(j, used[i]));
-        FRG_HIP_CHECK(hipStreamWaitEvent(lastStream, j, 0));
+        hipError_t r = hipEventRecord(j, used[i]);
+        if (r == hipSuccess) r = hipStreamWaitEvent(lastStream, j, 0);
         giveEvent(j);
+        FRG_HIP_CHECK(r);
       }
       used.assign(1, lastStream);
     }

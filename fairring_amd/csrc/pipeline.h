@@ -64,7 +64,8 @@ struct Progress {
   std::atomic<int64_t> enqueued{0};   // operations whose GPU work is all enqueued
   std::atomic<int64_t> launches{0};   // kernel launches issued
   std::atomic<int64_t> onCallersStream{0};  // operations launched by submit() on the producer stream
-  std::atomic<int64_t> merged{0};           // operations run together with a neighbour that was waiting
+  std::atomic<int64_t> merged{0};           // operations run together with others that were waiting
+  std::atomic<int64_t> segmentedLaunches{0};  // launches that covered pieces of several operations
   // Per reduce stream: how many operations it has been given, and up to which
   // of them the device's null stream already waits (the null stream is never
   // destroyed, so what it was once told to wait for stays waited for: a step's
@@ -181,6 +182,7 @@ class Context {
   char* scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize);
   hipEvent_t takeEvent();
   void giveEvent(hipEvent_t e);
+  hipEvent_t freshEvent(hipEvent_t* holder);
 
   // ---- order between operations ------------------------------------------
   // Operations are dealt to the reduce streams so that neighbours overlap, but
@@ -278,10 +280,11 @@ class Context {
   void orderAfterInline(hipStream_t producer);
 
   std::vector<hipStream_t> reduceStreams_;
-  // Slot s is filled on copy stream s % copyStreams_.size(): while one stream works through the
-  // event packets around its copy, the other's copy keeps the host link busy.
+  // The staging streams of the host-staged path: each owns groups of slots, copies into them
+  // and runs the folds that read them; while one folds, the other's copies keep the link busy.
   std::vector<hipStream_t> copyStreams_;
-  int numCopyStreams_ = 2;
+  static constexpr int kDefaultStagingStreams = 1;
+  int numCopyStreams_ = kDefaultStagingStreams;
   std::mutex copyMu_;  // guards the creation of copyStreams_
 
   char* stagingPool_ = nullptr;            // numSlots_ x slotBytes_ of device memory
@@ -295,15 +298,10 @@ class Context {
   static constexpr int64_t kDefaultCarryScratchBytes = 8 * 1024 * 1024;
   int64_t carryScratchBytes_ = kDefaultCarryScratchBytes;
   char* carryScratch_ = nullptr;
-  std::vector<hipEvent_t> slotFreeEvents_;    // recorded after a slot's last consumer
-  std::vector<hipEvent_t> slotFilledEvents_;  // recorded after the copy into a slot
-  std::vector<char> slotUsed_;
   std::atomic<int64_t> nextStagingSlot_{0};  // round-robin cursor (fairring/device.cc:482)
   int64_t nextSeq_ = 0;          // operation counter for log lines
   std::shared_ptr<Progress> progress_ = std::make_shared<Progress>();
 
-  std::mutex eventMu_;
-  std::vector<hipEvent_t> freeEvents_;
 
   std::atomic<bool> profiling_{false};  // per-launch dispatch timestamps
   std::mutex profMu_;

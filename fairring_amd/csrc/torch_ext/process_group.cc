@@ -463,7 +463,9 @@ void ProcessGroupFairring::setSimulatedPeerContributions(std::vector<at::Tensor>
     peersFromHost_ = fromHost;
     // The group holds its peers' tensors for as long as they are in use, so an
     // operation does not record them on the pipeline's streams; the ones that
-    // go now may still be read by operations in flight, and are recorded here.
+    // go now may still be read by launches in flight, and are recorded here.
+    // (Operations that have not been enqueued yet hold their peers themselves
+    // until they are: the allocator's events then land behind their launches.)
     if (peersUsed_) {
       for (const at::Tensor& t : old) {
         if (!t.is_cuda()) continue;
@@ -697,6 +699,12 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::reduceCommon(
     if (!seen) peersUsedFrom_.push_back(asStream);
   }
   keepAlive.push_back(own);
+  // The peers' tensors as well, until the command thread has enqueued the
+  // operation: the group may be handed new peers (and the caller may free the
+  // old ones) while this operation still waits in the queue, and what
+  // setSimulatedPeerContributions records on the streams at that moment only
+  // covers launches that are already enqueued.
+  keepAlive.insert(keepAlive.end(), peers.begin(), peers.end());
   auto state = std::make_shared<OpState>();
   state->tensor = out;
   state->inputs = std::move(keepAlive);
@@ -830,7 +838,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
   auto future = c10::make_intrusive<c10::ivalue::Future>(
       c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
-  auto* pending = new Pending{future, t, {}, device};
+  // the peers are held until the operation is enqueued (see reduceCommon)
+  auto* pending = new Pending{future, t, peers, device};
   // buffer.to(wire).div_(size): on the GPU a multiply by the reciprocal, in
   // the wire type's arithmetic
   const int rc = frg_allreduce_compressed(

@@ -360,12 +360,13 @@ class DeviceFairring:
     def progress(self):
         """Operations submitted / started / fully enqueued, kernel launches
         issued, operations launched by the call itself on the producer stream
-        (small ones, with nothing in flight) and operations run as one with
-        neighbours that were waiting in the queue, so far."""
-        out = (ctypes.c_int64 * 6)()
-        _capi.check(_capi.lib().frg_get_progress(self._h, ctypes.byref(out)))
+        (small ones, with nothing in flight), operations run as one with others
+        that were waiting in the queue, and launches that covered pieces of
+        several such operations, so far."""
+        out = (ctypes.c_int64 * 7)()
+        _capi.check(_capi.lib().frg_get_progress2(self._h, ctypes.byref(out), ctypes.sizeof(out)))
         return dict(submitted=out[0], started=out[1], enqueued=out[2], launches=out[3],
-                    on_callers_stream=out[4], merged=out[5])
+                    on_callers_stream=out[4], merged=out[5], segmented_launches=out[6])
 
     def synchronize(self):
         _capi.check(_capi.lib().frg_synchronize(self._h))

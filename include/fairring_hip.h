@@ -347,18 +347,34 @@ FRG_API int frg_work_wait(frg_work* work);
 FRG_API int frg_set_wait_timeout(double seconds);
 
 /* Where the pipeline stands, for such reports: operations accepted, begun by
- * the command thread and fully enqueued, and kernel launches issued so far;
- * and how many of the operations were small enough, with nothing in flight, to
- * be launched by the call itself on the producer stream (see frg_allreduce). */
+ * the command thread and fully enqueued, and kernel launches issued so far.
+ * This struct keeps the four fields it had in version 0.1 of the ABI. */
 typedef struct frg_progress {
   int64_t submitted;
   int64_t started;
   int64_t enqueued;
   int64_t launches;
-  int64_t on_callers_stream;
-  int64_t merged; /* operations run as one with neighbours that were waiting (see frg_allreduce) */
 } frg_progress;
 FRG_API int frg_get_progress(frg_ctx* ctx, frg_progress* out);
+
+/* The same with the counters added since, in a struct that may grow: `size` is
+ * sizeof(frg_progress2) as the caller was compiled, and no more than that many
+ * bytes are written (fields the library does not know of are left alone, so a
+ * caller zero-initialises). on_callers_stream: operations small enough, with
+ * nothing in flight, to be launched by the call itself on the producer stream;
+ * merged: operations run as one with others that were waiting in the queue;
+ * segmented_launches: launches that each covered pieces of several such
+ * operations (see frg_allreduce for all three). */
+typedef struct frg_progress2 {
+  int64_t submitted;
+  int64_t started;
+  int64_t enqueued;
+  int64_t launches;
+  int64_t on_callers_stream;
+  int64_t merged;
+  int64_t segmented_launches;
+} frg_progress2;
+FRG_API int frg_get_progress2(frg_ctx* ctx, frg_progress2* out, uint64_t size);
 
 /* WorkFairring::isCompleted (process_group.cc:43-45): FRG_OK once the command
  * thread has enqueued the whole operation, FRG_ERR_NOT_READY before. */
@@ -422,8 +438,11 @@ FRG_API int frg_set_tuning(int blocks_per_cu);
 /* Message of the last failure on the calling thread (or of the failed work). */
 FRG_API const char* frg_last_error(void);
 
-/* "major.minor" of this ABI. 0.2: frg_progress grew (on_callers_stream, merged);
- * frg_plan_launches, frg_get_copy_streams, frg_reduce_slice_static added. */
+/* "major.minor" of this ABI. 0.2: frg_plan_launches, frg_get_copy_streams,
+ * frg_reduce_slice_static added (and frg_progress grew in place, which 0.3
+ * takes back). 0.3: frg_progress has its four fields of 0.1 again and
+ * frg_get_progress2 carries the later counters with the caller's struct size;
+ * frg_allreduce_gathered added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus

@@ -193,6 +193,18 @@ void waitOn(FakeStream* s, std::shared_ptr<Record> r) {
   });
 }
 
+// How a stream wait binds to its event: to the record the event held when the
+// wait was enqueued (what the HIP runtime does, the default), or, as a probe,
+// to whatever record the event holds when the wait packet is executed.
+std::atomic<int> gLatestRecordWaits{0};
+std::mutex gGraveyardMu;
+std::vector<FakeEvent*> gGraveyard;  // destroyed events a late-binding wait may still read
+
+bool recordDone(const std::shared_ptr<Record>& r) {
+  std::lock_guard<std::mutex> g(r->mu);
+  return r->done;
+}
+
 // The legacy null stream: work submitted to it starts after everything
 // submitted so far to the blocking streams, and work submitted to a blocking
 // stream starts after everything submitted so far to the null stream. Streams
@@ -318,6 +330,22 @@ hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned int
   }
   if (!r) return hipSuccess;
   FakeStream* s = resolve(stream);
+  if (gLatestRecordWaits.load()) {
+    // a wait on a record that has fired is no packet at all, as in the runtime
+    if (recordDone(r)) return hipSuccess;
+    implicitSync(s);
+    s->push([event] {
+      std::shared_ptr<Record> latest;
+      {
+        std::lock_guard<std::mutex> g(event->mu);
+        latest = event->current;
+      }
+      if (!latest) return;
+      std::unique_lock<std::mutex> lock(latest->mu);
+      latest->cv.wait(lock, [&] { return latest->done; });
+    });
+    return hipSuccess;
+  }
   implicitSync(s);
   waitOn(s, r);
   return hipSuccess;
@@ -333,6 +361,12 @@ hipError_t hipEventCreate(hipEvent_t* event) { return hipEventCreateWithFlags(ev
 
 hipError_t hipEventDestroy(hipEvent_t event) {
   enter("hipEventDestroy");
+  if (gLatestRecordWaits.load()) {
+    // a wait that binds late still reads the event: it is kept, with its last record
+    std::lock_guard<std::mutex> g(gGraveyardMu);
+    gGraveyard.push_back(event);
+    return hipSuccess;
+  }
   delete event;  // pending waits hold their own reference to the record
   return hipSuccess;
 }
@@ -483,6 +517,8 @@ void fake_hip_set_hw_queues(int n) {
     s->queue = shared != nullptr ? shared : new HwQueue();
   }
 }
+
+void fake_hip_set_latest_record_waits(int on) { gLatestRecordWaits = on; }
 
 void fake_hip_fail_call(const char* api, int nth) {
   std::lock_guard<std::mutex> g(gCallMu);

@@ -87,6 +87,13 @@ void fake_hip_occupy(hipStream_t stream, int ms);
 // Every stream, existing or yet to be created, shares `n` in-order hardware
 // queues (0: a queue per stream, the default). Call it while no work is in flight.
 void fake_hip_set_hw_queues(int n);
+// A probe of how much the pipeline leans on the binding of a stream wait: with
+// 1, a wait on an event that has not fired binds to the record the event holds
+// when the wait packet is executed, not to the one it held when
+// hipStreamWaitEvent was called (0, the default, and what the HIP runtime
+// does). A caller that re-records an event while a wait on it is still pending
+// then sees that wait follow the new record. Call it while no work is in flight.
+void fake_hip_set_latest_record_waits(int on);
 // Makes hipStreamIsCapturing report a capture in progress on every stream (1) or none (0).
 void fake_hip_set_capturing(int on);
 // Makes the `nth` next call (1 = the very next) of the named API fail once.

@@ -504,8 +504,8 @@ void scenarioSmallOperationsOnTheCallersStream() {
     CHECK(note.thread == std::this_thread::get_id());
     CHECK(frg_work_is_completed(w) == FRG_OK);
     CHECK(fake_hip_calls("hipStreamWaitEvent") == waits);
-    frg_progress pr = {};
-    CHECK(frg_get_progress(ctx, &pr) == FRG_OK);
+    frg_progress2 pr = {};
+    CHECK(frg_get_progress2(ctx, &pr, sizeof(pr)) == FRG_OK);
     CHECK(pr.submitted == 1 && pr.started == 1 && pr.enqueued == 1 && pr.launches == 1);
     // frg_synchronize covers it, without the caller touching its stream
     CHECK(frg_synchronize(ctx) == FRG_OK);
@@ -603,8 +603,8 @@ void scenarioSmallOperationsOnTheCallersStream() {
     CHECK(note.thread == std::this_thread::get_id());
     CHECK(frg_work_wait(w) == FRG_ERR_UNSUPPORTED);
     frg_work_release(w);
-    frg_progress pr = {};
-    CHECK(frg_get_progress(ctx, &pr) == FRG_OK);
+    frg_progress2 pr = {};
+    CHECK(frg_get_progress2(ctx, &pr, sizeof(pr)) == FRG_OK);
     CHECK(pr.submitted == pr.enqueued && pr.submitted == pr.started);
   }
   CHECK(frg_destroy(ctx) == FRG_OK);
@@ -713,8 +713,8 @@ void scenarioNeighboursRunAsOne() {
       std::unique_lock<std::mutex> lock(gate.mu);
       gate.cv.wait(lock, [&] { return gate.reached; });
     }
-    frg_progress before = {};
-    CHECK(frg_get_progress(ctx, &before) == FRG_OK);
+    frg_progress2 before = {};
+    CHECK(frg_get_progress2(ctx, &before, sizeof(before)) == FRG_OK);
     Order order;
     std::vector<OrderNote> notes(pieces);
     std::vector<frg_work*> w(pieces, nullptr);
@@ -740,8 +740,8 @@ void scenarioNeighboursRunAsOne() {
     gate.cv.notify_all();
     for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
     CHECK(frg_synchronize(ctx) == FRG_OK);
-    frg_progress after = {};
-    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    frg_progress2 after = {};
+    CHECK(frg_get_progress2(ctx, &after, sizeof(after)) == FRG_OK);
     CHECK(after.enqueued - before.enqueued == pieces);
     if (variant <= 1) {
       CHECK(after.merged - before.merged == pieces);           // one run of eight
@@ -780,8 +780,8 @@ void scenarioNeighboursRunAsOne() {
       std::unique_lock<std::mutex> lock(gate.mu);
       gate.cv.wait(lock, [&] { return gate.reached; });
     }
-    frg_progress before = {};
-    CHECK(frg_get_progress(ctx, &before) == FRG_OK);
+    frg_progress2 before = {};
+    CHECK(frg_get_progress2(ctx, &before, sizeof(before)) == FRG_OK);
     // pieces of n/4 from the top of z[n, 2n) downwards, each written from the piece n below it
     // and added to itself: z[n + j] += z[j]; the four would join into z[n, 2n) += z[0, n),
     // fine; then the same one step further down, z[j] += z[j - ...] is what must not join:
@@ -803,8 +803,8 @@ void scenarioNeighboursRunAsOne() {
     }
     gate.cv.notify_all();
     for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
-    frg_progress after = {};
-    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    frg_progress2 after = {};
+    CHECK(frg_get_progress2(ctx, &after, sizeof(after)) == FRG_OK);
     CHECK(after.merged == before.merged);
     // sequentially: piece i adds the ORIGINAL piece below it (that one is updated only later)
     Vec want = z0;
@@ -850,8 +850,8 @@ void scenarioNeighboursRunAsOne() {
     }
     gate.cv.notify_all();
     for (frg_work* x : w) CHECK(frg_work_wait(x) == FRG_OK);
-    frg_progress after = {};
-    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    frg_progress2 after = {};
+    CHECK(frg_get_progress2(ctx, &after, sizeof(after)) == FRG_OK);
     CHECK(after.merged == count);
     Vec want = z0;
     for (int i = 0; i < count; ++i) {
@@ -894,7 +894,7 @@ void scenarioProducerOrdering() {
 
 void scenarioHostStaged() {
   std::puts("host-staged accumulation: slot rotation and reuse");
-  for (int slots : {1, 2, 3, 5, 8}) {
+  for (int slots : {1, 2, 3, 5, 7, 8, 9, 11}) {
     frg_ctx* ctx = makeCtx(4096 * slots, 4096, 0, 0);
     frg_layout l;
     CHECK(frg_get_layout(ctx, &l) == FRG_OK && l.num_staging_slots == slots);
@@ -918,6 +918,32 @@ void scenarioHostStaged() {
                                nullptr, &w) == FRG_OK);
       CHECK(frg_work_wait(w) == FRG_OK);
       CHECK(same(own, fold(c, FRG_SCALE_DIV, static_cast<float>(k))));
+      frg_work_release(w);
+    }
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+  // slices of 4 MiB and more: the second staging stream's first batch goes in two halves
+  for (int slots : {2, 4}) {
+    const int64_t n = (5ll << 20) / 4 + 12345;  // two slices: 4 MiB and a ragged rest
+    frg_ctx* ctx = makeCtx((4ll << 20) * slots, 4ll << 20, 0, 0);
+    for (int k : {2, 3, 6}) {
+      auto c = randomContribs(k, n, 90 + k + slots);
+      Vec own = c[0];
+      std::vector<Vec> rest(c.begin() + 1, c.end());
+      auto tr = table(rest);
+      frg_work* w = nullptr;
+      CHECK(frg_allreduce_host(ctx, own.data(), tr.data(), k - 1, n, FRG_F32, FRG_SUM,
+                               FRG_SCALE_MUL, 0.5f, /*carry=*/1, nullptr, nullptr, nullptr,
+                               &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(own, fold(c, FRG_SCALE_MUL, 0.5f)));
+      frg_work_release(w);
+      Vec out(n, -1.f);
+      auto t = table(c);
+      CHECK(frg_allreduce_host(ctx, out.data(), t.data(), k, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE,
+                               1.f, /*carry=*/0, nullptr, nullptr, nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(out, fold(c, FRG_SCALE_NONE, 1.f)));
       frg_work_release(w);
     }
     CHECK(frg_destroy(ctx) == FRG_OK);
@@ -974,6 +1000,7 @@ void scenarioOrderBetweenOperations() {
     tab[0] = own.data();
     frg_work* w[3] = {nullptr, nullptr, nullptr};
     fake_hip_occupy(s0, 60);
+    std::printf("  shared tensor, case %d\n", round);
     if (round == 0) {
       // three in-place reductions of the same tensor, none waited for (a scale
       // of its own each, so that their order shows in the result)
@@ -1027,6 +1054,7 @@ void scenarioOrderBetweenOperations() {
     auto ta = table(a), tb = table(b);
     frg_work *wa = nullptr, *wb = nullptr;
     fake_hip_occupy(s0, 300);
+    std::puts("  independent buckets");
     CHECK(frg_allreduce(ctx, outA.data(), ta.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
                         nullptr, nullptr, nullptr, &wa) == FRG_OK);
     CHECK(frg_allreduce(ctx, outB.data(), tb.data(), 3, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
@@ -1041,6 +1069,7 @@ void scenarioOrderBetweenOperations() {
     frg_work_release(wa);
     frg_work_release(wb);
     // many independent buckets: the bookkeeping stays bounded (a forced join now and then)
+    std::puts("  many independent buckets");
     std::vector<Vec> outs(200, Vec(256));
     auto small = randomContribs(2, 256, 52);
     auto ts = table(small);
@@ -1059,6 +1088,7 @@ void scenarioOrderBetweenOperations() {
     auto t = table(c);
     Vec out(n, -1.f);
     hipStream_t s1 = streamsOf(ctx)[1];
+    std::puts("  resident, host-staged, resident on one tensor");
     CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 16, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
                         nullptr, nullptr, nullptr, nullptr) == FRG_OK);  // takes stream 0
     fake_hip_occupy(s1, 60);
@@ -1073,7 +1103,7 @@ void scenarioOrderBetweenOperations() {
     CHECK(frg_allreduce(ctx, out2.data(), again, 2, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,
                         nullptr, nullptr, nullptr, &w) == FRG_OK);
     CHECK(frg_work_wait(w) == FRG_OK);
-    CHECK(streamsOf(ctx).size() == 4);  // the copy streams exist once something was staged
+    CHECK(streamsOf(ctx).size() == 3);  // the staging stream exists once something was staged
     const Vec first = fold(c, FRG_SCALE_NONE, 1.f);
     const Vec staged = fold(c, FRG_SCALE_NONE, 1.f, &first);
     CHECK(same(out, staged));
@@ -1341,7 +1371,7 @@ void scenarioErrors() {
   fake_hip_fail_call("hipMalloc", 1);
   CHECK(frg_create(0, &o, &bad) == FRG_ERR_HIP && bad == nullptr);
   // a failure after the staging pool exists: released once, nothing else left behind
-  fake_hip_fail_call("hipEventCreate", 1);
+  fake_hip_fail_call("hipMalloc", 2);  // the chain scratch
   CHECK(frg_create(0, &o, &bad) == FRG_ERR_HIP && bad == nullptr);
   CHECK(frg_create(7, &o, &bad) == FRG_ERR_INVALID);
 }
@@ -1437,6 +1467,8 @@ void concurrentSubmitters(frg_ctx* ctx) {
 std::atomic<long> gScenarioTicks{0};
 const char* volatile gScenarioName = "start-up";
 
+int gStallLimitSeconds = 150;
+
 void watchdog() {
   long seen = -1;
   int stale = 0;
@@ -1445,8 +1477,9 @@ void watchdog() {
     const long now = gScenarioTicks.load();
     stale = now == seen ? stale + 1 : 0;
     seen = now;
-    if (stale > 150) {
-      std::fprintf(stderr, "no progress for 150 s in scenario: %s\n", gScenarioName);
+    if (stale > gStallLimitSeconds) {
+      std::fprintf(stderr, "no progress for %d s in scenario: %s\n", gStallLimitSeconds,
+                   gScenarioName);
       std::abort();
     }
   }
@@ -1491,9 +1524,19 @@ void runAll() {
 
 }  // namespace
 
-int main() {
+// With the argument "latest-record-waits" every scenario runs on a runtime whose
+// stream waits bind to the record their event holds when the wait packet is
+// executed (not what HIP does): what the pipeline makes of that shows how much
+// it leans on re-recording an event while a wait on it is pending.
+int main(int argc, char** argv) {
+  std::setvbuf(stdout, nullptr, _IOLBF, 0);  // a run that is aborted still shows how far it got
   // every scenario but the one about them sends its small operations through the pipeline
   setenv("FAIRRING_INLINE_BYTES", "0", 1);
+  if (const char* limit = std::getenv("HOST_TEST_STALL_SECONDS")) gStallLimitSeconds = std::atoi(limit);
+  if (argc > 1 && std::string(argv[1]) == "latest-record-waits") {
+    std::puts("== stream waits bind to their event's latest record");
+    fake_hip_set_latest_record_waits(1);
+  }
   std::thread(watchdog).detach();
   std::puts("== every stream on a queue of its own");
   runAll();

@@ -128,8 +128,9 @@ def test_header_is_plain_c(tmp_path):
         pytest.skip("gcc not available")
     src = tmp_path / "use_header.c"
     src.write_text('#include "fairring_hip.h"\n'
-                   "int probe(void) { frg_options o = {0}; frg_progress p = {0};\n"
-                   "  return (int)(o.num_machines + p.launches) + FRG_SCALE_PRE_DIV + FRG_I8; }\n")
+                   "int probe(void) { frg_options o = {0}; frg_progress p = {0}; frg_progress2 q = {0};\n"
+                   "  return (int)(o.num_machines + p.launches + q.segmented_launches + sizeof(q))\n"
+                   "         + FRG_SCALE_PRE_DIV + FRG_I8; }\n")
     r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
                         "-I", os.path.join(ROOT, "include"), str(src)],
                        capture_output=True, text=True, timeout=120)
@@ -151,7 +152,7 @@ def test_c_client_builds_and_fails_cleanly_without_a_gpu(tmp_path):
     if torch.cuda.is_available():
         assert r.returncode == 0 and "abi client ok" in r.stdout, r.stderr
     else:
-        assert r.returncode == 2 and "abi 0.2" in r.stdout     # the HIP runtime finds no device
+        assert r.returncode == 2 and "abi 0.3" in r.stdout     # the HIP runtime finds no device
 
 
 def test_a_missing_library_is_a_loud_error_not_a_fallback(tmp_path):
