@@ -52,7 +52,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2",
-                    choices=["c2", "c3", "c4", "c5", "c5pg", "copy", "hook", "smallops"])
+                    choices=["c2", "c3", "c4", "c5", "c5pg", "c5sep", "gather", "copy", "hook",
+                             "smallops"])
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="default workload only: do not measure the other workloads afterwards")
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
@@ -621,6 +622,213 @@ def run_c5pg(args, np, torch, fa, oracle, shared=None):
     return value, elapsed, cfg, roof, checked, None, "f32"
 
 
+def run_c5sep(args, np, torch, fa, oracle):
+    """The bucket stream as DistributedDataParallel lays it out: every bucket an allocation of
+    its own, and so is every peer's copy of it (48 buckets of 25 MiB, 8 contributions), one
+    `_fairring.ProcessGroup.allreduce` per bucket, in place, divide fused, every work waited for
+    at the end of the step. Nothing here is contiguous with anything else, so no two buckets
+    can run as one operation."""
+    import datetime
+
+    import torch.distributed as dist
+
+    import fairring  # noqa: F401  (registers the backend, loads the extension)
+    from fairring_amd import _fairring
+
+    k = args.k or 8
+    buckets = 48
+    n = args.slice_bytes // 4
+    numel = args.numel or buckets * n
+    buckets = max(1, numel // n)
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(515)
+    fresh = [torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(buckets)]
+    owns = [t.clone() for t in fresh]
+    peers = [[torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(k - 1)]
+             for _ in range(buckets)]
+    torch.cuda.synchronize()
+    o = _fairring.ProcessGroup.Options(
+        max_memory_allocated_in_bytes=args.total_memory, max_padding_allocated_in_bytes=MiB,
+        min_parallelism=2, is_high_priority_stream=True,
+        timeout=datetime.timedelta(seconds=60), slice_size_in_bytes=args.slice_bytes)
+    pg = _fairring.ProcessGroup(dist.HashStore(), 0, k, o)
+    pg._set_fused_divide(True)
+    own_lists = [[t] for t in owns]
+
+    def step():
+        works = []
+        for ov, pv in zip(own_lists, peers):
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg.allreduce(ov))
+        return works
+
+    def finish(works):
+        for w in works:
+            w.wait()
+
+    for _ in range(max(args.warmup, 1)):
+        finish(step())
+    pg._synchronize()
+    torch.cuda.synchronize()
+    pg._launch_records()
+    steps = args.steps * 4          # a step is 11 GB: a few more of them for a steady figure
+    t0 = time.perf_counter()
+    pg._profile_mark()
+    pending = [step() for _ in range(steps)]
+    pg._profile_mark()
+    for works in pending:
+        finish(works)
+    pg._synchronize()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    recs = pg._launch_records()
+    value = (k + 1) * n * buckets * 4 * steps / elapsed / 1e9
+    roof = roofline_from_records(recs, (k + 1) * 4, launch_elems(args, n, n, 4, k), SPAN_HOW)
+    roof["kernel"] = "ksumKernel<F32Vec, SUM, K=%d>" % k
+    # parity on fresh buckets (the timed steps reduced in place), three of them against the oracle
+    for t, f in zip(owns, fresh):
+        t.copy_(f)
+    finish(step())
+    pg._synchronize()
+    torch.cuda.synchronize()
+    checked = []
+    for b in sorted({0, buckets // 2, buckets - 1}):
+        host = [fresh[b].cpu().numpy()] + [p.cpu().numpy() for p in peers[b]]
+        want = oracle.sum_f32(host, oracle.SCALE_MUL, 1.0 / k, threads=os.cpu_count() or 1)
+        if not (owns[b].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all():
+            raise SystemExit("parity FAILED on bucket %d (c5sep)" % b)
+        checked.append(b)
+    layout = pg._layout()
+    del pg
+    cfg = {
+        "workload": "DDP-shaped bucket stream: %d buckets of %d B, each bucket and each of its %d "
+                    "peer copies an allocation of its own, one _fairring.ProcessGroup.allreduce per "
+                    "bucket, in place, fused x1/%d, every work waited for at the end of the step "
+                    "(configs[4] with DistributedDataParallel's own bucket layout)" % (
+                        buckets, args.slice_bytes, k - 1, k),
+        "k": k, "numel": n * buckets, "buckets": buckets, "staging_total_bytes": args.total_memory,
+        "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
+                   "staging_slots": layout[3]},
+    }
+    return value, elapsed / 4, cfg, roof, checked, None, "f32"
+
+
+# One 25 MiB bucket of a transformer layer's gradients: two matrices, three vectors, a rest.
+GATHER_SEGMENTS = [4194304, 2048, 2048, 2097152, 2048, 256000]
+
+
+def run_gather(args, np, torch, fa, oracle, shared=None):
+    """The bucket stream with this rank's contribution read from the gradient tensors
+    themselves (frg_allreduce_gathered): per 25 MiB bucket six tensors of their own, the
+    bucket written once; beside it the same stream the way DistributedDataParallel does it by
+    default, every gradient copied into its bucket first and the bucket reduced in place."""
+    k, numel = args.k or 8, args.numel or 1_370_000_000
+    slice_elems = args.slice_bytes // 4
+    spans = ddp_buckets(numel, slice_elems, MiB // 4)
+    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
+                            slice_size_in_bytes=args.slice_bytes,
+                            num_reduce_streams=args.streams, max_launch_bytes=args.launch_bytes)
+    if shared is not None:
+        xs, out = shared
+    else:
+        xs = synth(torch, numel, k, "f32", 20240)
+        out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    torch.cuda.synchronize()
+    # this rank's gradients: tensors of their own holding what xs[0] holds
+    grads = []
+    for lo, hi in spans:
+        segs, at = [], lo
+        for ln in GATHER_SEGMENTS:
+            ln = min(ln, hi - at)
+            if ln > 0:
+                segs.append(xs[0][at:at + ln].clone())
+                at += ln
+        if at < hi:
+            segs.append(xs[0][at:hi].clone())
+        grads.append(segs)
+    torch.cuda.synchronize()
+    views = [(out[lo:hi], [x[lo:hi] for x in xs]) for lo, hi in spans]
+    prepared = {}
+
+    class Last:
+        def __init__(self, works):
+            self.works = works
+
+        def wait(self):
+            for w in self.works:
+                w.wait()
+
+    def step(d):
+        if id(d) not in prepared:
+            prepared[id(d)] = [d.prepare(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k,
+                                         gathered=(0, segs))
+                               for (o, cs), segs in zip(views, grads)]
+        return Last([submit() for submit in prepared[id(d)]])
+
+    elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
+    step_bytes = (k + 1) * numel * 4
+    value = step_bytes * args.steps / elapsed / 1e9
+    roof = roofline_from_records(recs, (k + 1) * 4,
+                                 launch_elems(args, slice_elems, slice_elems, 4, k), SPAN_HOW)
+    roof["kernel"] = "ksumSegmentedKernel<F32Vec, K=%d, x1/%d>" % (k, k)
+    segmented = dev.progress()["segmented_launches"]
+    step(dev).wait()
+    checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)
+    # the default way: copy every gradient to its place in the bucket (one copy kernel per
+    # tensor, as the reducer issues them), then reduce the bucket in place
+    bucket = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    bviews = [(bucket[lo:hi], [bucket[lo:hi]] + [x[lo:hi] for x in xs[1:]]) for lo, hi in spans]
+    targets = []
+    for (lo, hi), segs in zip(spans, grads):
+        at, row = lo, []
+        for sg in segs:
+            row.append(bucket[at:at + sg.numel()])
+            at += sg.numel()
+        targets.append(row)
+    plain = [dev.prepare(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k) for o, cs in bviews]
+
+    def two_pass():
+        works = []
+        for submit, row, segs in zip(plain, targets, grads):
+            for dst, src in zip(row, segs):
+                dst.copy_(src)
+            works.append(submit())
+        return Last(works)
+
+    two_pass().wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    w = None
+    for _ in range(args.steps):
+        w = two_pass()
+    w.wait()
+    dev.synchronize()
+    torch.cuda.synchronize()
+    two = step_bytes * args.steps / (time.perf_counter() - t0) / 1e9
+    same = torch.equal(bucket.view(torch.int32), out.view(torch.int32))
+    if not same:
+        raise SystemExit("parity FAILED: gathered differs from copy + allreduce")
+    layout = dev.layout
+    dev.close()
+    cfg = {
+        "workload": "DDP bucket stream with this rank's contribution read from its gradient "
+                    "tensors: %d fp32 elements as %d buckets of %d B, %d tensors of their own per "
+                    "bucket (%s elements), K=%d, fused x1/%d; the copy of every gradient into its "
+                    "bucket (8 bytes per element) is not made" % (
+                        numel, len(spans), args.slice_bytes, len(GATHER_SEGMENTS),
+                        "/".join(str(v) for v in GATHER_SEGMENTS), k, k),
+        "k": k, "numel": numel, "buckets": len(spans), "tensors": sum(len(sg) for sg in grads),
+        "segmented_launches": segmented,
+        "copy_then_allreduce_GBps": round(two, 1),
+        "copy_then_allreduce_note": "same algorithmic bytes over the time of copying every "
+                                    "gradient into its bucket and reducing the bucket in place; "
+                                    "results equal bit for bit",
+        "layout": layout,
+    }
+    return value, elapsed, cfg, roof, checked, None, "f32"
+
+
 def run_hook(args, np, torch, fa, oracle):
     """The reduction with torch's bf16 compression hook folded in: this rank's
     fp32 gradient is compressed in registers, K - 1 peers' bf16 tensors are read,
@@ -834,16 +1042,16 @@ def main():
         # they are run on their own, fewer steps, no CPU baseline.
         shared = tuple(keep) if keep else None
         extra = {}
-        for name in ("c5", "c5pg", "c4", "hook", "c3"):
+        for name in ("c5", "c5pg", "gather", "c5sep", "c4", "hook", "c3"):
             sub = argparse.Namespace(**vars(args))
             sub.workload, sub.no_cpu_baseline = name, True
             sub.steps, sub.warmup = min(args.steps, 3 if name == "c3" else 10), 3
-            if name == "c4":
+            if name in ("c5sep", "c4"):
                 shared = None
-                keep.clear()       # the fp32 inputs go before the bf16 ones are made
+                keep.clear()       # the fp32 inputs go before other ones are made
             try:
                 r = measure(sub, name, np, torch, fa, oracle,
-                            shared=shared if name in ("c5", "c5pg") else None)
+                            shared=shared if name in ("c5", "c5pg", "gather") else None)
                 # compact: the whole record stays one line of a few KB
                 roof = {key: r["roofline"][key] for key in (
                     "bound", "achieved", "peak", "nominal", "unit", "frac", "traffic",
@@ -853,8 +1061,9 @@ def main():
                                "steps": r["steps"], "ms_per_step": r["ms_per_step"],
                                "dtype": r["dtype"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
                                "parity": r["parity"].split(";")[0], "roofline": roof}
-                if "host_link_GBps" in r["config"]:
-                    extra[name]["host_link_GBps"] = r["config"]["host_link_GBps"]
+                for key in ("host_link_GBps", "copy_then_allreduce_GBps"):
+                    if key in r["config"]:
+                        extra[name][key] = r["config"][key]
             except (SystemExit, Exception) as e:  # noqa: BLE001  (reported, and the run fails)
                 extra[name] = {"error": "%s: %s" % (type(e).__name__, e)}
                 failed.append(name)
@@ -882,6 +1091,11 @@ def measure(args, workload, np, torch, fa, oracle, keep=None, shared=None):
     elif workload == "c5pg":
         value, elapsed, cfg, roof, checked, base, dtype = run_c5pg(args, np, torch, fa, oracle,
                                                                    shared=shared)
+    elif workload == "c5sep":
+        value, elapsed, cfg, roof, checked, base, dtype = run_c5sep(args, np, torch, fa, oracle)
+    elif workload == "gather":
+        value, elapsed, cfg, roof, checked, base, dtype = run_gather(args, np, torch, fa, oracle,
+                                                                     shared=shared)
     else:
         value, elapsed, cfg, roof, checked, base, dtype = run_c5(args, np, torch, fa, oracle,
                                                                  shared=shared)
@@ -910,6 +1124,10 @@ def measure(args, workload, np, torch, fa, oracle, keep=None, shared=None):
         "c5": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream",
         "c5pg": "reduce GB/s (bytes read+written), 8-way fp32 DDP bucket stream through "
                 "ProcessGroup.allreduce",
+        "c5sep": "reduce GB/s (bytes read+written), 8-way fp32 bucket stream, every bucket and "
+                 "contribution its own allocation, through ProcessGroup.allreduce",
+        "gather": "reduce GB/s (bytes read+written), 8-way fp32 bucket stream, own contribution "
+                  "read from the gradient tensors",
         "copy": "copy GB/s (bytes read+written), 25 MiB slices",
         "hook": "reduce GB/s (bytes read+written), 8-way with the bf16 compression hook folded in",
     }[workload]

@@ -20,7 +20,7 @@ EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_plan_launches", "frg_reduce_slice", "frg_reduce_slice_static",
     "frg_reduce_slice_compressed", "frg_allreduce_compressed",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
-    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
+    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_allreduce_gathered", "frg_reduce_pieces", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
     "frg_set_tuning",
     "frg_last_error", "frg_version",
@@ -49,6 +49,15 @@ class Options(ctypes.Structure):
                 ("num_reduce_streams", ctypes.c_int32),
                 ("num_copy_streams", ctypes.c_int32),
                 ("max_launch_bytes", ctypes.c_int64)]
+
+
+class Segment(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("numel", ctypes.c_int64)]
+
+
+class Piece(ctypes.Structure):
+    _fields_ = [("out", ctypes.c_void_p), ("contribs", ctypes.POINTER(ctypes.c_void_p)),
+                ("numel", ctypes.c_int64)]
 
 
 class LaunchRecord(ctypes.Structure):
@@ -97,6 +106,9 @@ def lib():
     L.frg_reduce_slice_compressed.argtypes = [vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp]
     L.frg_allreduce_compressed.argtypes = [vp, vp, i32, pvp, i32, i32, i64, i32, i32, f32, vp,
                                            DONE_FN, vp, pvp]
+    L.frg_allreduce_gathered.argtypes = [vp, vp, pvp, i32, i32, ctypes.POINTER(Segment), i32, i64,
+                                         i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    L.frg_reduce_pieces.argtypes = [ctypes.POINTER(Piece), i32, i32, i32, i32, i32, f32, vp]
     L.frg_allreduce_host.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp,
                                      DONE_FN, vp, pvp]
     for fn in (L.frg_work_wait, L.frg_work_is_completed, L.frg_work_release, L.frg_synchronize,

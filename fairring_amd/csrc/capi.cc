@@ -1,6 +1,7 @@
 // The C ABI declared in include/fairring_hip.h: argument checks, error strings
 // and nothing else; the work is in pipeline.cc and ksum_kernels.hip.
 #include <string>
+#include <vector>
 
 #include "../../include/fairring_hip.h"
 #include <cstring>
@@ -154,6 +155,70 @@ int frg_reduce_slice(void* out, const void* const* contribs, int K, int64_t n, i
   return FRG_OK;
 }
 
+int frg_reduce_pieces(const frg_piece* pieces, int num_pieces, int K, int dtype, int op,
+                      int scale_mode, float scale, void* stream) {
+  if (num_pieces < 0 || (num_pieces > 0 && pieces == nullptr)) {
+    return fail(FRG_ERR_INVALID, "bad piece list");
+  }
+  if (K < 1 || K > frg::kMaxContribsPerLaunch) {
+    return fail(FRG_ERR_INVALID, "K must be in [1, 64], got " + std::to_string(K));
+  }
+  const int64_t elsize = frg::elementSize(dtype);
+  if (elsize == 0) return fail(FRG_ERR_UNSUPPORTED, "unsupported dtype " + std::to_string(dtype));
+  return guarded([&] {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const bool kindOk = frg::segmentedKind(K, dtype, op, false);
+    const int cap = frg::maxSegmentsPerLaunch(K);
+    std::vector<frg::SegPiece> batch;
+    std::string err;
+    auto flush = [&]() -> int {
+      if (batch.empty()) return FRG_OK;
+      frg::SegmentedArgs a;
+      a.pieces = batch.data();
+      a.numPieces = static_cast<int>(batch.size());
+      a.K = K;
+      a.dtype = dtype;
+      a.scale_mode = scale_mode;
+      a.scale = scale;
+      const int rc = frg::launchSegmented(a, s, &err);
+      batch.clear();
+      return rc;
+    };
+    for (int i = 0; i < num_pieces; ++i) {
+      const frg_piece& pc = pieces[i];
+      if (pc.numel < 0) return fail(FRG_ERR_INVALID, "negative element count");
+      if (pc.numel == 0) continue;
+      if (pc.out == nullptr || pc.contribs == nullptr) return fail(FRG_ERR_INVALID, "null piece");
+      for (int k = 0; k < K; ++k) {
+        if (pc.contribs[k] == nullptr) return fail(FRG_ERR_INVALID, "null contribution");
+      }
+      if (kindOk && frg::segmentable(pc.out, pc.contribs, K, elsize)) {
+        batch.push_back(frg::SegPiece{pc.out, pc.contribs, pc.numel});
+        if (static_cast<int>(batch.size()) == cap) {
+          const int rc = flush();
+          if (rc != FRG_OK) return fail(rc, err);
+        }
+        continue;
+      }
+      // not one for the segmented kernel: a launch of its own
+      frg::ReduceArgs a;
+      a.out = pc.out;
+      a.contribs = pc.contribs;
+      a.K = K;
+      a.n = pc.numel;
+      a.dtype = dtype;
+      a.op = op;
+      a.scale_mode = scale_mode;
+      a.scale = scale;
+      const int rc = frg::launchReduce(a, s, &err);
+      if (rc != FRG_OK) return fail(rc, err);
+    }
+    const int rc = flush();
+    if (rc != FRG_OK) return fail(rc, err);
+    return static_cast<int>(FRG_OK);
+  });
+}
+
 int frg_reduce_slice_compressed(void* out, int out_dtype, const void* const* contribs, int K,
                                 int raw_index, int64_t n, int wire_dtype, int scale_mode,
                                 float scale, void* stream) {
@@ -235,6 +300,47 @@ int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs, int K, i
                   frg_done_fn done, void* user, frg_work** work) {
   return submitCommon(ctx, out, contribs, K, numel, dtype, op, scale_mode, scale,
                       producer_stream, done, user, work, /*fromHost=*/false, /*carry=*/false);
+}
+
+int frg_allreduce_gathered(frg_ctx* ctx, void* out, const void* const* contribs, int K,
+                           int gathered_index, const frg_segment* segments, int num_segments,
+                           int64_t numel, int dtype, int op, int scale_mode, float scale,
+                           void* producer_stream, frg_done_fn done, void* user, frg_work** work) {
+  if (work) *work = nullptr;
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  if (K < 1 || contribs == nullptr) {
+    return fail(FRG_ERR_INVALID, "at least one contribution is required");
+  }
+  if (num_segments < 0 || (num_segments > 0 && segments == nullptr)) {
+    return fail(FRG_ERR_INVALID, "bad segment list");
+  }
+  if (gathered_index < 0 || gathered_index >= K) {
+    return fail(FRG_ERR_INVALID, "gathered_index out of range");
+  }
+  return guarded([&] {
+    Context::Request r;
+    r.out = out;
+    r.contribs.assign(contribs, contribs + K);
+    r.numel = numel;
+    r.dtype = dtype;
+    r.op = op;
+    r.scaleMode = scale_mode;
+    r.scale = scale;
+    r.gatheredIndex = gathered_index;
+    r.gathered.reserve(static_cast<size_t>(num_segments));
+    for (int i = 0; i < num_segments; ++i) {
+      r.gathered.push_back(Context::Request::Segment{segments[i].ptr, segments[i].numel});
+    }
+    r.producerStream = static_cast<hipStream_t>(producer_stream);
+    r.done = done;
+    r.user = user;
+    std::string err;
+    Work* w = nullptr;
+    const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    if (work) *work = reinterpret_cast<frg_work*>(w);
+    return static_cast<int>(FRG_OK);
+  });
 }
 
 int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype, const void* const* contribs,

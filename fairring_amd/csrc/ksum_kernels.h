@@ -62,6 +62,101 @@ inline char* placeInScratch(char* base, const void* like, bool acc, int64_t elsi
 // status; on failure `err` says why. Never synchronises.
 int launchReduce(const ReduceArgs& args, hipStream_t stream, std::string* err);
 
+// ---- one launch over several pieces ------------------------------------------
+//
+// A piece is an elementwise reduction of its own: an output, K contributions
+// and a length, anywhere in memory. A segmented launch runs up to
+// maxSegmentsPerLaunch(K) pieces with the same K, element type and scale as one
+// kernel launch: the tiles of all pieces are dealt to one persistent grid, so a
+// bucket whose own contribution lies scattered over many gradient tensors (one
+// piece per tensor), or the odds and ends of several operations, cost one
+// launch instead of one per piece. SUM of fp32, bf16 or fp16, up to
+// kMaxSegmentContribs contributions, nothing carried in; every pointer of a
+// piece must sit at the same position within 16 bytes (segmentable() says
+// whether a piece qualifies; what does not goes through launchReduce).
+struct SegPiece {
+  void* out = nullptr;
+  const void* const* contribs = nullptr;  // host array of K device pointers
+  int64_t n = 0;                          // elements
+};
+
+constexpr int kMaxSegmentContribs = 16;
+inline constexpr int maxSegmentsPerLaunch(int K) { return K <= 8 ? 24 : 12; }
+
+struct SegmentedArgs {
+  const SegPiece* pieces = nullptr;
+  int numPieces = 0;
+  int K = 0;
+  int dtype = 0;
+  int scale_mode = 0;
+  float scale = 1.0f;
+  int blocks_per_cu = 0;  // 0 = 4 per CU
+  hipEvent_t startEvent = nullptr;
+  hipEvent_t stopEvent = nullptr;
+};
+
+// The kernel's tile: 256 vectors of 16 bytes of every contribution.
+constexpr int64_t kSegmentTileVectors = 256;
+constexpr int64_t kSegmentTileBytes = kSegmentTileVectors * 16;
+
+// Whether a reduction of this kind can be part of a segmented launch at all.
+inline bool segmentedKind(int K, int dtype, int op, bool carry) {
+  // FRG_F32 = 0, FRG_BF16 = 1, FRG_F16 = 2; FRG_SUM = 0
+  return K >= 1 && K <= kMaxSegmentContribs && op == 0 && !carry && dtype >= 0 && dtype <= 2;
+}
+
+// Whether a piece can: its pointers sit at one position within 16 bytes.
+inline bool segmentable(const void* out, const void* const* contribs, int K, int64_t elsize) {
+  const uintptr_t o = reinterpret_cast<uintptr_t>(out);
+  if (o % static_cast<uintptr_t>(elsize) != 0) return false;
+  for (int k = 0; k < K; ++k) {
+    if ((reinterpret_cast<uintptr_t>(contribs[k]) & 15) != (o & 15)) return false;
+  }
+  return true;
+}
+
+// How the kernel walks such a piece: [head scalars][nvec vectors][tail
+// scalars], the first `lead` vectors (those ahead of the first 4 KiB boundary of
+// the output) as a tile of their own, whole tiles behind it, the last one
+// possibly partial.
+struct PieceSplit {
+  int64_t head = 0, nvec = 0, tail = 0, lead = 0, tiles = 0;
+};
+
+inline PieceSplit splitPiece(const void* out, int64_t n, int64_t elsize) {
+  const int64_t lanes = 16 / elsize;
+  const uintptr_t o = reinterpret_cast<uintptr_t>(out);
+  PieceSplit p;
+  p.head = static_cast<int64_t>(((16 - (o & 15)) & 15) / static_cast<uintptr_t>(elsize));
+  if (p.head > n) p.head = n;
+  p.nvec = (n - p.head) / lanes;
+  p.tail = n - p.head - p.nvec * lanes;
+  const uintptr_t first = o + static_cast<uintptr_t>(p.head * elsize);
+  const uintptr_t mask = static_cast<uintptr_t>(kSegmentTileBytes) - 1;
+  p.lead = static_cast<int64_t>(((static_cast<uintptr_t>(kSegmentTileBytes) - (first & mask)) & mask) / 16);
+  if (p.lead > p.nvec) p.lead = p.nvec;
+  p.tiles = (p.lead > 0 ? 1 : 0) + (p.nvec - p.lead + kSegmentTileVectors - 1) / kSegmentTileVectors;
+  if (p.tiles == 0 && n > 0) p.tiles = 1;  // scalars only: still a piece of the launch
+  return p;
+}
+
+// Tiles the kernel deals for a piece, and the elements of the piece ahead of
+// its tile `tile` (0 for the first): where a piece may be cut in two.
+inline int64_t segmentTiles(const void* out, int64_t n, int64_t elsize) {
+  return n > 0 ? splitPiece(out, n, elsize).tiles : 0;
+}
+
+inline int64_t segmentTileStart(const void* out, int64_t n, int64_t elsize, int64_t tile) {
+  if (tile <= 0) return 0;
+  const PieceSplit sp = splitPiece(out, n, elsize);
+  const int64_t vec = sp.lead > 0 ? sp.lead + (tile - 1) * kSegmentTileVectors
+                                  : tile * kSegmentTileVectors;
+  const int64_t start = sp.head + vec * (16 / elsize);
+  return start < n ? start : n;
+}
+
+int launchSegmented(const SegmentedArgs& args, hipStream_t stream, std::string* err);
+
 // Launch-shape knobs (process-wide); 0 keeps the default.
 void setTuning(int blocksPerCu);
 

@@ -92,9 +92,9 @@ constexpr int kOutIsAcc = 2;
 // variants then hold nothing but loads, adds, one multiply and the store (a
 // third of the code, which matters when a launch lasts 10 us and every CU
 // starts it with a cold instruction cache).
-template <typename TR, int OP, int KT, int SC>
+template <typename TR, int OP, int KT, int SC, typename PT>
 __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
-                                          const Ptrs<KT>& in, int K,
+                                          const PT& in, int K,
                                           const typename TR::elem_t* carrySrc,
                                           int scaleMode, float scale, int accFlags,
                                           int64_t elemBase, unsigned int lane) {
@@ -333,6 +333,162 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
   return hipGetLastError();
 }
 
+// ---- one launch over several pieces -------------------------------------------
+
+// The pieces of a segmented launch, by value in the kernel arguments (2.4 KiB):
+// per piece the output, the contributions, the split of its length into [head
+// scalars][lead vectors][tiles][tail scalars] and where its tiles start in the
+// launch's tile count. `lead` vectors bring the tiles of a piece to a 4 KiB
+// boundary of its output.
+template <int KC, int S>
+struct SegTable {
+  void* out[S];
+  const void* in[S][KC];
+  long long tileBegin[S + 1];
+  long long nvec[S];
+  int lead[S];
+  short head[S];
+  short tail[S];
+  int nseg;
+};
+
+// A row of the table, indexed like Ptrs.
+struct SegRow {
+  const void* const* p;
+};
+
+// Every block walks the launch's tiles blockIdx, blockIdx + grid, ...: the
+// piece a tile belongs to is found by walking the prefix sums (tiles ascend,
+// so the walk never restarts; all of it uniform, in scalar registers), the
+// piece's pointers are read from the kernel arguments, and the tile is reduced
+// exactly as ksumKernel does it. A piece's first tile (its lead) and its last
+// may be partial. The scalars at the ends of piece e are done by block e.
+template <typename TRV, typename TRS, int KT, int SC, int KC, int S>
+__global__ void __launch_bounds__(kBlock)
+    ksumSegmentedKernel(const SegTable<KC, S> tab, int K, int scaleMode, float scale) {
+  using elem_t = typename TRV::elem_t;
+  constexpr long long kTile = static_cast<long long>(kBlock) * kUnroll;
+  const long long total = tab.tileBegin[tab.nseg];
+  int s = 0;
+  for (long long t = blockIdx.x; t < total; t += gridDim.x) {
+    while (t >= tab.tileBegin[s + 1]) ++s;
+    const long long lt = t - tab.tileBegin[s];
+    const long long lead = tab.lead[s];
+    const long long nvec = tab.nvec[s];
+    long long v0, count;
+    if (lead > 0) {
+      v0 = lt == 0 ? 0 : lead + (lt - 1) * kTile;
+      count = lt == 0 ? lead : nvec - v0;
+    } else {
+      v0 = lt * kTile;
+      count = nvec - v0;
+    }
+    const int64_t elemBase = tab.head[s] + v0 * TRV::kLanes;
+    const SegRow row{tab.in[s]};
+    elem_t* out = static_cast<elem_t*>(tab.out[s]);
+    if (count >= kTile) {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        reduceOne<TRV, FRG_SUM, KT, SC>(out, row, K, static_cast<const elem_t*>(nullptr), scaleMode,
+                                        scale, 0, elemBase, threadIdx.x + u * kBlock);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const unsigned int lane = threadIdx.x + u * kBlock;
+        if (lane < count) {
+          reduceOne<TRV, FRG_SUM, KT, SC>(out, row, K, static_cast<const elem_t*>(nullptr),
+                                          scaleMode, scale, 0, elemBase, lane);
+        }
+      }
+    }
+  }
+  for (int e = blockIdx.x; e < tab.nseg; e += gridDim.x) {
+    const int head = tab.head[e], tail = tab.tail[e];
+    if (static_cast<int>(threadIdx.x) < head + tail) {
+      const int64_t i = static_cast<int>(threadIdx.x) < head
+                            ? static_cast<int64_t>(threadIdx.x)
+                            : head + tab.nvec[e] * TRV::kLanes + (threadIdx.x - head);
+      const SegRow row{tab.in[e]};
+      reduceOne<TRS, FRG_SUM, KT, SC>(static_cast<elem_t*>(tab.out[e]), row, K,
+                                      static_cast<const elem_t*>(nullptr), scaleMode, scale, 0, i, 0u);
+    }
+  }
+}
+
+static_assert(static_cast<int64_t>(kBlock) * kUnroll == kSegmentTileVectors, "the tile of the kernels");
+
+template <typename TRV, typename TRS, int KT, int SC>
+hipError_t launchSegmentedVariant(const SegmentedArgs& a, int numCus, hipStream_t stream) {
+  constexpr int KC = KT > 0 ? KT : kMaxSegmentContribs;
+  constexpr int S = maxSegmentsPerLaunch(KC);
+  using Table = SegTable<KC, S>;
+  static_assert(sizeof(Table) <= 3072, "the table travels in the kernel arguments");
+  Table tab = {};
+  const int64_t elsize = static_cast<int64_t>(sizeof(typename TRV::elem_t));
+  long long tiles = 0;
+  int nseg = 0;
+  for (int i = 0; i < a.numPieces; ++i) {
+    const SegPiece& pc = a.pieces[i];
+    if (pc.n <= 0) continue;
+    const PieceSplit sp = splitPiece(pc.out, pc.n, elsize);
+    tab.out[nseg] = pc.out;
+    for (int k = 0; k < KC; ++k) tab.in[nseg][k] = pc.contribs[k < a.K ? k : 0];
+    tab.tileBegin[nseg] = tiles;
+    tab.nvec[nseg] = sp.nvec;
+    tab.lead[nseg] = static_cast<int>(sp.lead);
+    tab.head[nseg] = static_cast<short>(sp.head);
+    tab.tail[nseg] = static_cast<short>(sp.tail);
+    tiles += sp.tiles;
+    ++nseg;
+  }
+  if (nseg == 0) return hipSuccess;
+  for (int i = nseg; i <= S; ++i) tab.tileBegin[i] = tiles;
+  tab.nseg = nseg;
+  const int blocksPerCu = a.blocks_per_cu > 0 ? a.blocks_per_cu : 4;
+  long long grid = static_cast<long long>(numCus) * blocksPerCu;
+  if (grid > tiles) grid = tiles;
+  if (grid < nseg) grid = nseg;  // a block per piece for the scalars at its ends
+  if (a.startEvent != nullptr || a.stopEvent != nullptr) {
+    hipExtLaunchKernelGGL((ksumSegmentedKernel<TRV, TRS, KT, SC, KC, S>),
+                          dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, stream, a.startEvent,
+                          a.stopEvent, 0, tab, a.K, a.scale_mode, a.scale);
+  } else {
+    hipLaunchKernelGGL((ksumSegmentedKernel<TRV, TRS, KT, SC, KC, S>),
+                       dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, stream, tab, a.K,
+                       a.scale_mode, a.scale);
+  }
+  return hipGetLastError();
+}
+
+// The gradient shapes (2, 4 or 8 contributions; no scale, the multiply by 1/K
+// on the store, or every term times 1/K) as compile-time variants, like the
+// plain kernel's; everything else through the runtime-K body.
+template <typename TRV, typename TRS>
+hipError_t dispatchSegmented(const SegmentedArgs& a, int numCus, hipStream_t stream) {
+#define FRG_SEG_CASE(KK, MODE, SCV)                                                    \
+  if (a.K == KK && a.scale_mode == MODE) {                                             \
+    return launchSegmentedVariant<TRV, TRS, KK, SCV>(a, numCus, stream);               \
+  }
+  FRG_SEG_CASE(8, FRG_SCALE_NONE, FRG_SCALE_NONE)
+  FRG_SEG_CASE(8, FRG_SCALE_MUL, FRG_SCALE_MUL)
+  FRG_SEG_CASE(8, FRG_SCALE_PRE_MUL, kPreMul)
+  FRG_SEG_CASE(4, FRG_SCALE_NONE, FRG_SCALE_NONE)
+  FRG_SEG_CASE(4, FRG_SCALE_MUL, FRG_SCALE_MUL)
+  FRG_SEG_CASE(4, FRG_SCALE_PRE_MUL, kPreMul)
+  FRG_SEG_CASE(2, FRG_SCALE_NONE, FRG_SCALE_NONE)
+  FRG_SEG_CASE(2, FRG_SCALE_MUL, FRG_SCALE_MUL)
+  FRG_SEG_CASE(2, FRG_SCALE_PRE_MUL, kPreMul)
+#undef FRG_SEG_CASE
+  if (a.scale_mode == FRG_SCALE_PRE_MUL) {
+    return launchSegmentedVariant<TRV, TRS, 0, kPreMul>(a, numCus, stream);
+  }
+  if (a.scale_mode == FRG_SCALE_PRE_DIV) {
+    return launchSegmentedVariant<TRV, TRS, 0, kPreDiv>(a, numCus, stream);
+  }
+  return launchSegmentedVariant<TRV, TRS, 0, -1>(a, numCus, stream);
+}
+
 // FAST: also instantiate the compile-time-K variants (the gradient types);
 // the other types run the runtime-K variant for every K.
 template <typename TRV, typename TRS, bool FAST>
@@ -473,6 +629,66 @@ bool isFloating(int dtype) {
 }
 
 void setTuning(int blocksPerCu) { gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0; }
+
+int launchSegmented(const SegmentedArgs& a, hipStream_t stream, std::string* err) {
+  auto fail = [&](int code, const std::string& msg) {
+    if (err) *err = msg;
+    return code;
+  };
+  const int64_t elsize = elementSize(a.dtype);
+  if (!segmentedKind(a.K, a.dtype, FRG_SUM, false)) {
+    return fail(FRG_ERR_UNSUPPORTED, "a segmented launch takes a SUM of fp32, bf16 or fp16 with "
+                                     "up to 16 contributions");
+  }
+  if (a.scale_mode < FRG_SCALE_NONE || a.scale_mode > FRG_SCALE_PRE_DIV) {
+    return fail(FRG_ERR_INVALID, "bad scale mode");
+  }
+  if (a.numPieces < 0 || a.numPieces > maxSegmentsPerLaunch(a.K) ||
+      (a.numPieces > 0 && a.pieces == nullptr)) {
+    return fail(FRG_ERR_INVALID, "a segmented launch takes up to " +
+                                     std::to_string(maxSegmentsPerLaunch(a.K)) + " pieces");
+  }
+  for (int i = 0; i < a.numPieces; ++i) {
+    const SegPiece& pc = a.pieces[i];
+    if (pc.n < 0) return fail(FRG_ERR_INVALID, "negative element count");
+    if (pc.n == 0) continue;
+    if (pc.out == nullptr || pc.contribs == nullptr) return fail(FRG_ERR_INVALID, "null piece");
+    const uintptr_t o = reinterpret_cast<uintptr_t>(pc.out);
+    const uintptr_t bytes = static_cast<uintptr_t>(pc.n) * static_cast<uintptr_t>(elsize);
+    for (int k = 0; k < a.K; ++k) {
+      const uintptr_t p = reinterpret_cast<uintptr_t>(pc.contribs[k]);
+      if (p == 0) return fail(FRG_ERR_INVALID, "null contribution " + std::to_string(k));
+      if (p != o && p < o + bytes && o < p + bytes) {
+        return fail(FRG_ERR_INVALID, "output partially overlaps contribution " + std::to_string(k));
+      }
+    }
+    if (!segmentable(pc.out, pc.contribs, a.K, elsize)) {
+      return fail(FRG_ERR_INVALID, "the pointers of a piece of a segmented launch must agree "
+                                   "modulo 16 bytes");
+    }
+  }
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return fail(FRG_ERR_HIP, "hipGetDevice failed");
+  const int numCus = computeUnits(device);
+  hipError_t e = hipErrorInvalidValue;
+  switch (a.dtype) {
+    case FRG_F32:
+      e = dispatchSegmented<F32Vec, F32Scalar>(a, numCus, stream);
+      break;
+    case FRG_BF16:
+      e = dispatchSegmented<Bf16Vec, Bf16Scalar>(a, numCus, stream);
+      break;
+    case FRG_F16:
+      e = dispatchSegmented<F16Vec, F16Scalar>(a, numCus, stream);
+      break;
+    default:
+      break;
+  }
+  if (e != hipSuccess) {
+    return fail(FRG_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString(e));
+  }
+  return FRG_OK;
+}
 
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   auto fail = [&](int code, const std::string& msg) {

@@ -622,7 +622,8 @@ void Context::orderAfterInline(hipStream_t producer) {
 // the completion callback (on this, the caller's, thread). Returns false when
 // the operation is to go through the pipeline instead.
 bool Context::tryInline(const Request& req, Work* work) {
-  if (inlineTrafficBytes_ <= 0 || req.fromHost || req.compressed || !launchBytesByContribs_) {
+  if (inlineTrafficBytes_ <= 0 || req.fromHost || req.compressed || !launchBytesByContribs_ ||
+      !req.gathered.empty()) {
     return false;
   }
   const int total = static_cast<int>(req.contribs.size());
@@ -767,6 +768,44 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     }
     if (req.rawIndex < -1 || req.rawIndex >= K) {
       *err = "raw_index out of range";
+      return FRG_ERR_INVALID;
+    }
+  }
+  if (!req.gathered.empty() || req.gatheredIndex >= 0) {
+    const int K = static_cast<int>(req.contribs.size());
+    if (req.fromHost || req.compressed) {
+      *err = "a piecewise contribution goes with device-resident, uncompressed contributions";
+      return FRG_ERR_UNSUPPORTED;
+    }
+    if (req.gatheredIndex < 0 || req.gatheredIndex >= K) {
+      *err = "gathered_index out of range";
+      return FRG_ERR_INVALID;
+    }
+    int64_t sum = 0;
+    for (const Request::Segment& g : req.gathered) {
+      if (g.numel < 0 || (g.numel > 0 && g.ptr == nullptr)) {
+        *err = "bad segment (negative length or null pointer)";
+        return FRG_ERR_INVALID;
+      }
+      sum += g.numel;
+    }
+    if (sum != req.numel) {
+      *err = "the segments hold " + std::to_string(sum) + " elements, the operation " +
+             std::to_string(req.numel);
+      return FRG_ERR_INVALID;
+    }
+    for (int k = 0; k < K; ++k) {
+      if (k != req.gatheredIndex && req.contribs[static_cast<size_t>(k)] == req.out &&
+          req.numel > 0) {
+        *err = "the output of an operation with a piecewise contribution must not be another "
+               "of its contributions";
+        return FRG_ERR_INVALID;
+      }
+    }
+    // the slot it leaves in the table is never read; give it a value that passes the checks
+    req.contribs[static_cast<size_t>(req.gatheredIndex)] = req.out;
+    if (req.numel > 0 && req.gathered.empty()) {
+      *err = "no segments";
       return FRG_ERR_INVALID;
     }
   }
@@ -928,6 +967,42 @@ void Context::launchCompressed(const CompressedArgs& args, hipStream_t stream) {
   launchAndCount<CompressedArgs>(args, stream, &launchCompressedReduce);
 }
 
+// One launch over several pieces; the books count its elements like any launch's.
+void Context::launchSegments(const SegmentedArgs& args, hipStream_t stream) {
+  SegmentedArgs a = args;
+  int64_t elems = 0;
+  for (int i = 0; i < args.numPieces; ++i) elems += args.pieces[i].n;
+  const bool prof = profiling_.load(std::memory_order_relaxed) && elems > 0;
+  if (prof) {
+    FRG_HIP_CHECK(hipEventCreate(&a.startEvent));
+    FRG_HIP_CHECK(hipEventCreate(&a.stopEvent));
+  }
+  std::string err;
+  const int rc = launchSegmented(a, stream, &err);
+  if (rc == FRG_OK && elems > 0) {
+    for (size_t i = 0; i < reduceStreams_.size(); ++i) {
+      if (reduceStreams_[i] == stream) {
+        streamLaunches_[i] += 1;
+        streamElems_[i] += elems;
+      }
+    }
+    lastContribs_ = args.K;
+    progress_->launches.fetch_add(1);
+    progress_->segmentedLaunches.fetch_add(1);
+  }
+  if (prof) {
+    if (rc == FRG_OK) {
+      std::lock_guard<std::mutex> g(profMu_);
+      profEvents_.push_back(ProfRecord{a.startEvent, a.stopEvent, elems, a.K, stream, 1});
+    } else {
+      (void)hipEventDestroy(a.startEvent);
+      (void)hipEventDestroy(a.stopEvent);
+    }
+  }
+  if (rc == FRG_ERR_HIP) throw HipFailure(err);
+  if (rc != FRG_OK) throw ContractFailure(rc, err);
+}
+
 // The scratch region of a reduce stream (reused in stream order), placed so that the vector variant of the kernel still runs:
 // at the same position within 16 bytes as `like` for a buffer of the storage
 // type, or, for fp32 accumulators of a 2-byte type, such that it reaches a
@@ -1012,8 +1087,13 @@ Context::OpSpans Context::spansOf(const Request& req) {
     for (size_t k = 0; k < req.contribs.size(); ++k) {
       const uintptr_t p = reinterpret_cast<uintptr_t>(req.contribs[k]);
       if (p == o) continue;  // in place: covered by the write
+      if (static_cast<int>(k) == req.gatheredIndex) continue;  // given piecewise, below
       const uintptr_t es = (req.compressed && static_cast<int>(k) == req.rawIndex) ? 4 : wireSize;
       op.reads.push_back(Span{p, p + n * es});
+    }
+    for (const Request::Segment& g : req.gathered) {
+      const uintptr_t p = reinterpret_cast<uintptr_t>(g.ptr);
+      if (g.numel > 0) op.reads.push_back(Span{p, p + static_cast<uintptr_t>(g.numel) * wireSize});
     }
   }
   return op;
@@ -1330,6 +1410,203 @@ std::vector<hipStream_t> Context::runResident(const Request& req,
   return used;
 }
 
+// One contribution given piecewise (a bucket's own gradients, each still in its
+// own tensor): the output is cut where the pieces end, every piece is an
+// elementwise reduction of its own (the output and the other contributions at
+// the piece's offset, the piece itself in the gathered contribution's place),
+// and the pieces are packed into segmented launches, cut on 4 KiB tiles of the
+// output, of about the size a plain operation's launches have. The copy of
+// every gradient into the bucket that DDP makes ahead of the allreduce
+// (torch:csrc/distributed/c10d/reducer.cpp, copy_grad_to_bucket) is thereby
+// part of the reduction: 8 bytes per element of HBM traffic less. A piece whose
+// pointers disagree modulo 16 (an odd-sized tensor ahead of it in the bucket),
+// and any reduction the segmented kernel does not cover (MAX, more than 16
+// contributions, other element types), runs as a plain launch of its own.
+std::vector<hipStream_t> Context::runGathered(const Request& req,
+                                              const std::vector<hipEvent_t>& initialEvents) {
+  const int64_t elsize = elementSize(req.dtype);
+  const int total = static_cast<int>(req.contribs.size());
+  const int g = req.gatheredIndex;
+  nextStagingSlot_ += numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
+  const bool kindOk = segmentedKind(total, req.dtype, req.op, false);
+  const int maxSegs = maxSegmentsPerLaunch(total);
+  int64_t targetTiles = defaultLaunchShape(total, req.numel * elsize).bytes / kTileBytes;
+  if (targetTiles < 1) targetTiles = 1;
+  const bool accChain = total > kMaxContribsPerLaunch && req.op == FRG_SUM &&
+                        (req.dtype == FRG_BF16 || req.dtype == FRG_F16);
+
+  // A unit is one launch: several pieces through the segmented kernel, or one
+  // piece through the plain one.
+  struct Unit {
+    bool segmented = true;
+    std::vector<SegPiece> pieces;
+    int64_t off = 0;  // plain: offset of the piece in the output
+  };
+  std::vector<Unit> units;
+  std::deque<std::vector<const void*>> tables;  // the pieces' pointer tables stay put
+  auto tableOf = [&](const Request::Segment& seg, int64_t off) {
+    std::vector<const void*> tab(static_cast<size_t>(total));
+    for (int k = 0; k < total; ++k) {
+      tab[static_cast<size_t>(k)] =
+          k == g ? seg.ptr
+                 : static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + off * elsize;
+    }
+    return tab;
+  };
+  // Launches of `targetTiles` each, the last one with what is left over when
+  // that is less than half a launch's worth: a bucket of 25 MiB is 8 + 8 + 9
+  // MiB like a plain operation's, not three launches and a sliver.
+  int64_t segmentedTiles = 0;
+  {
+    int64_t off = 0;
+    for (const Request::Segment& seg : req.gathered) {
+      if (seg.numel <= 0) continue;
+      char* outp = static_cast<char*>(req.out) + off * elsize;
+      const std::vector<const void*> tab = tableOf(seg, off);
+      if (kindOk && segmentable(outp, tab.data(), total, elsize)) {
+        segmentedTiles += segmentTiles(outp, seg.numel, elsize);
+      }
+      off += seg.numel;
+    }
+  }
+  int64_t tilesLeft = segmentedTiles;  // not yet given to a launch
+  Unit cur;
+  int64_t curTiles = 0;
+  auto flush = [&] {
+    if (!cur.pieces.empty()) units.push_back(std::move(cur));
+    cur = Unit();
+    curTiles = 0;
+  };
+  int64_t off = 0;
+  for (const Request::Segment& seg : req.gathered) {
+    const int64_t len = seg.numel;
+    if (len <= 0) continue;
+    char* outp = static_cast<char*>(req.out) + off * elsize;
+    std::vector<const void*> tab = tableOf(seg, off);
+    if (!kindOk || !segmentable(outp, tab.data(), total, elsize)) {
+      flush();
+      tables.push_back(std::move(tab));
+      Unit plain;
+      plain.segmented = false;
+      plain.off = off;
+      plain.pieces.push_back(SegPiece{outp, tables.back().data(), len});
+      units.push_back(std::move(plain));
+      off += len;
+      continue;
+    }
+    const int64_t tiles = segmentTiles(outp, len, elsize);
+    for (int64_t t = 0; t < tiles;) {
+      int64_t take = tiles - t;
+      // a launch holds targetTiles, unless what would be left behind it is less
+      // than half a launch's worth: then it takes that too
+      const int64_t room = targetTiles - curTiles;
+      const bool openEnded = tilesLeft - room < targetTiles / 2;
+      if (!openEnded && take > room) take = room;
+      const int64_t e0 = segmentTileStart(outp, len, elsize, t);
+      const int64_t e1 = t + take == tiles ? len : segmentTileStart(outp, len, elsize, t + take);
+      std::vector<const void*> part(static_cast<size_t>(total));
+      for (int k = 0; k < total; ++k) {
+        part[static_cast<size_t>(k)] = static_cast<const char*>(tab[static_cast<size_t>(k)]) + e0 * elsize;
+      }
+      tables.push_back(std::move(part));
+      cur.pieces.push_back(SegPiece{outp + e0 * elsize, tables.back().data(), e1 - e0});
+      curTiles += take;
+      tilesLeft -= take;
+      t += take;
+      if ((!openEnded && curTiles >= targetTiles) ||
+          static_cast<int>(cur.pieces.size()) == maxSegs) {
+        flush();
+      }
+    }
+    off += len;
+  }
+  flush();
+
+  const size_t nStreams = reduceStreams_.size();
+  std::vector<char> initialsFired(initialEvents.size(), 0);
+  auto waitInitials = [&](hipStream_t stream) {
+    for (size_t i = 0; i < initialEvents.size(); ++i) {
+      bool fired = initialsFired[i] != 0;
+      waitInitial(stream, initialEvents[i], &fired);
+      initialsFired[i] = fired ? 1 : 0;
+    }
+  };
+  std::vector<char> waited(nStreams, 0);
+  const bool oneStream = units.size() <= static_cast<size_t>(oneStreamLaunches_);
+  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
+  size_t lastIdx = opStream;
+  if (oneStream && !units.empty()) ++nextLaunch_;
+  const OpSpans spans = spansOf(req);
+  if (!units.empty()) {
+    std::vector<size_t> targets;
+    if (oneStream) {
+      targets.push_back(opStream);
+    } else {
+      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
+    }
+    orderAfterConflicts(spans, targets);
+  }
+  for (const Unit& u : units) {
+    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
+    hipStream_t s = reduceStreams_[si];
+    if (!waited[si]) {
+      waitInitials(s);
+      waited[si] = 1;
+    }
+    lastIdx = si;
+    if (u.segmented) {
+      SegmentedArgs a;
+      a.pieces = u.pieces.data();
+      a.numPieces = static_cast<int>(u.pieces.size());
+      a.K = total;
+      a.dtype = req.dtype;
+      a.scale_mode = req.scaleMode;
+      a.scale = req.scale;
+      launchSegments(a, s);
+      continue;
+    }
+    const SegPiece& pc = u.pieces[0];
+    if (accChain) {
+      std::vector<const void*> ptrs(pc.contribs, pc.contribs + total);
+      chainThroughScratch(req, ptrs, u.off, pc.n, si, true);
+      continue;
+    }
+    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
+      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
+      const bool lastLaunch = k0 + kn == total;
+      ReduceArgs a;
+      a.out = pc.out;
+      a.contribs = pc.contribs + k0;
+      a.K = kn;
+      a.n = pc.n;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
+                                                                        : FRG_SCALE_NONE;
+      a.scale = req.scale;
+      a.carry = k0 > 0;
+      launch(a, s);
+    }
+  }
+  if (!units.empty()) {
+    std::vector<size_t> ran;
+    for (size_t si = 0; si < nStreams; ++si) {
+      if (waited[si]) ran.push_back(si);
+    }
+    remember(spans, ran);
+  }
+  if (!waited[lastIdx]) {
+    waitInitials(reduceStreams_[lastIdx]);
+    waited[lastIdx] = 1;
+  }
+  std::vector<hipStream_t> used;
+  for (size_t si = 0; si < nStreams; ++si) {
+    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
+  }
+  used.push_back(reduceStreams_[lastIdx]);
+  return used;
+}
+
 // Contributions in pinned host memory (server-side accumulation,
 // fairring/device.cc:543-589: collect into a staging slot, then reduce).
 // Contribution 0 lands directly in `out`; the later ones are copied into
@@ -1544,7 +1821,8 @@ bool Context::adjoins(const QueuedOp& last, const QueuedOp& next, int64_t bytesS
                       int* direction) {
   const Request& a = last.req;
   const Request& b = next.req;
-  if (!launchBytesByContribs_ || a.fromHost || b.fromHost || a.compressed || b.compressed) {
+  if (!launchBytesByContribs_ || a.fromHost || b.fromHost || a.compressed || b.compressed ||
+      !a.gathered.empty() || !b.gathered.empty()) {
     return false;
   }
   if (a.dtype != b.dtype || a.op != b.op || a.scaleMode != b.scaleMode || a.scale != b.scale ||
@@ -1630,7 +1908,8 @@ void Context::runGroup(const std::vector<std::shared_ptr<QueuedOp>>& group) {
       }
     }
     used = req->fromHost ? runHostStaged(*req, initials.empty() ? nullptr : initials[0])
-                         : runResident(*req, initials, slices);
+                         : (!req->gathered.empty() ? runGathered(*req, initials)
+                                                   : runResident(*req, initials, slices));
     lastStream = used.back();
     if (anyCallback && used.size() > 1) {
       // The callback orders consumers after ONE stream (fairring/device.cc:337-340

@@ -134,6 +134,15 @@ class Context {
     bool compressed = false;
     int outDtype = FRG_F32;
     int rawIndex = -1;
+    // Contribution `gatheredIndex` is not one buffer but these pieces, in the
+    // order they lie in the output (a bucket's own gradients, still in the
+    // tensors autograd left them in); contribs[gatheredIndex] is ignored.
+    struct Segment {
+      const void* ptr = nullptr;
+      int64_t numel = 0;
+    };
+    std::vector<Segment> gathered;
+    int gatheredIndex = -1;
     hipStream_t producerStream = nullptr;
     frg_done_fn done = nullptr;
     void* user = nullptr;
@@ -170,6 +179,9 @@ class Context {
                                        const std::vector<hipEvent_t>& initialEvents,
                                        int64_t slices);
   std::vector<hipStream_t> runHostStaged(const Request& req, hipEvent_t initialEvent);
+  std::vector<hipStream_t> runGathered(const Request& req,
+                                       const std::vector<hipEvent_t>& initialEvents);
+  void launchSegments(const struct SegmentedArgs& args, hipStream_t stream);
   // Makes `stream` wait for `initialEvent` unless that event has already fired.
   void waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fired);
   template <typename Args>

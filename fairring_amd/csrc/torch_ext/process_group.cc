@@ -799,6 +799,94 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreducePreDivided(at::Ten
                       /*chunkOffset=*/0, /*peerNumel=*/t.numel(), {}, /*preDivide=*/true);
 }
 
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceFromGrads(
+    at::Tensor bucket, std::vector<at::Tensor> grads, bool preDivide) {
+  FRG_CHECK(bucket.layout() == at::kStrided);
+  FRG_CHECK(bucket.is_cuda());
+  FRG_CHECK(bucket.is_non_overlapping_and_dense());
+  at::Tensor out = viewAsFlat(bucket);
+  const int dtype = dtypeCode(out);
+  TORCH_CHECK(dtype >= 0, "fairring: unsupported dtype ", out.scalar_type());
+  FRG_CHECK(8 % out.element_size() == 0);
+  int64_t total = 0;
+  std::vector<frg_segment> segments;
+  segments.reserve(grads.size());
+  for (at::Tensor& gr : grads) {
+    TORCH_CHECK(gr.is_cuda() && gr.device() == out.device() && gr.scalar_type() == out.scalar_type(),
+                "fairring: a gradient must be a tensor of the bucket's type on the bucket's device");
+    TORCH_CHECK(gr.layout() == at::kStrided && gr.is_non_overlapping_and_dense(),
+                "fairring: a gradient must be dense");
+    gr = viewAsFlat(gr);
+    segments.push_back(frg_segment{gr.data_ptr(), gr.numel()});
+    total += gr.numel();
+  }
+  TORCH_CHECK(total == out.numel(), "fairring: the gradients hold ", total,
+              " elements, the bucket ", out.numel());
+  TORCH_CHECK(!preDivide || at::isFloatingType(out.scalar_type()),
+              "fairring: a pre-divided allreduce takes a floating-point bucket");
+
+  std::lock_guard<std::mutex> g(mutex_);
+  const c10::DeviceIndex device = out.device().index();
+  frg_ctx* ctx = contextFor(device);
+  const int size = getSize();
+  const int rank = getRank();
+  const int64_t n = out.numel();
+  const std::vector<at::Tensor>& peers = peers_;
+  TORCH_CHECK(static_cast<int>(peers.size()) == size - 1,
+              "fairring: this build runs on one GPU without a transport; a group of size ",
+              size, " needs ", size - 1, " simulated peer contributions, got ", peers.size());
+  TORCH_CHECK(peers.empty() || !peersFromHost_,
+              "fairring: an allreduce from gradients takes GPU-resident peers");
+  for (const at::Tensor& p : peers) {
+    TORCH_CHECK(p.scalar_type() == out.scalar_type() && p.numel() == n &&
+                    p.device() == out.device(),
+                "fairring: peer contribution must match the bucket's dtype, size and device");
+  }
+  peersUsed_ = true;
+  std::vector<const void*> table;
+  table.reserve(size);
+  for (int r = 0, pi = 0; r < size; ++r) {
+    table.push_back(r == rank ? nullptr : peers[pi].data_ptr());
+    if (r != rank) ++pi;
+  }
+  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&out}, &grads);
+
+  const bool divide = !preDivide && fusedDivide_ && size > 1;
+  const bool pow2 = (size & (size - 1)) == 0;
+  int scaleMode = !divide ? FRG_SCALE_NONE : (pow2 ? FRG_SCALE_MUL : FRG_SCALE_DIV);
+  float scale = !divide ? 1.0f : (pow2 ? 1.0f / static_cast<float>(size)
+                                        : static_cast<float>(size));
+  if (preDivide) {
+    scaleMode = FRG_SCALE_PRE_MUL;
+    scale = 1.0f / static_cast<float>(size);
+  }
+  const auto currentStream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device);
+  {
+    const c10::Stream asStream = currentStream.unwrap();
+    bool seen = false;
+    for (const c10::Stream& st : peersUsedFrom_) seen = seen || st == asStream;
+    if (!seen) peersUsedFrom_.push_back(asStream);
+  }
+  auto state = std::make_shared<OpState>();
+  state->tensor = out;
+  state->inputs = std::move(grads);
+  state->inputs.insert(state->inputs.end(), peers.begin(), peers.end());
+  state->device = device;
+  auto* holder = new std::shared_ptr<OpState>(state);
+  frg_work* handle = nullptr;
+  const int rc = frg_allreduce_gathered(ctx, out.data_ptr(), table.data(), size, rank,
+                                        segments.data(), static_cast<int>(segments.size()), n,
+                                        dtype, FRG_SUM, scaleMode, scale, currentStream.stream(),
+                                        &onEnqueued, holder, &handle);
+  if (rc != FRG_OK) {
+    delete holder;
+    TORCH_CHECK(false, "fairring: ", frg_last_error());
+  }
+  return c10::make_intrusive<WorkFairring>(
+      c10d::OpType::ALLREDUCE, std::move(state), handle,
+      c10::intrusive_ptr<c10d::Backend>::unsafe_reclaim_from_nonowning(this), ctx);
+}
+
 c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Tensor bucket,
                                                                          at::ScalarType wire) {
   FRG_CHECK(bucket.layout() == at::kStrided);

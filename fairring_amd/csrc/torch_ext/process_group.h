@@ -157,6 +157,19 @@ class ProcessGroupFairring : public c10d::Backend {
   // this rank's bucket is compressed in registers, the sum is rounded to
   // `wire` once and written back widened into `bucket`.
   c10::intrusive_ptr<c10d::Work> allreduceCompressed(at::Tensor bucket, at::ScalarType wire);
+  // allreduceFromGrads: the allreduce of a bucket together with the copy that
+  // fills it. With DDP's default (gradient_as_bucket_view=False) the reducer
+  // copies every gradient to its place in the bucket just before the allreduce
+  // (torch:csrc/distributed/c10d/reducer.cpp, copy_grad_to_bucket; with no hook
+  // registered that copy multiplies by 1/size as well). Here this rank's
+  // contribution is read from `grads`, the gradient tensors in the order they
+  // lie in `bucket` (dense, their sizes adding up to the bucket's), and the
+  // reduced bucket is written once: the bucket is never read. With `preDivide`
+  // every contribution is scaled by 1/size before the sum (the peers hand in
+  // unscaled buckets), as in allreducePreDivided.
+  c10::intrusive_ptr<c10d::Work> allreduceFromGrads(at::Tensor bucket,
+                                                    std::vector<at::Tensor> grads,
+                                                    bool preDivide);
 
   // {slot size, slice size, padding slots, staging slots} once initialised.
   std::vector<int64_t> layout();
@@ -192,7 +205,7 @@ class ProcessGroupFairring : public c10d::Backend {
   std::map<c10::DeviceIndex, std::vector<c10::Stream>> copyStreams_;
   const std::vector<c10::Stream>& copyStreamsFor(c10::DeviceIndex device, frg_ctx* ctx);
   static constexpr int kNumReduceStreams = 2;
-  static constexpr int kNumCopyStreams = 2;
+  static constexpr int kNumCopyStreams = 0;  // the library's default
   void recordOnPipelineStreams(c10::DeviceIndex device, bool copyStreamsToo,
                                std::initializer_list<const at::Tensor*> tensors,
                                const std::vector<at::Tensor>* more);

@@ -14,7 +14,8 @@ the bucket crosses HBM once on the way in and once on the way out.
 import torch
 import torch.distributed as dist
 
-__all__ = ["allreduce_hook", "fp16_compress_hook", "bf16_compress_hook"]
+__all__ = ["allreduce_hook", "allreduce_from_grads_hook", "fp16_compress_hook",
+           "bf16_compress_hook"]
 
 
 def _backend(process_group, device):
@@ -35,6 +36,30 @@ def allreduce_hook(process_group, bucket):
     rank's bucket divided by the group size before the sum."""
     buf = bucket.buffer()
     return _backend(process_group, buf.device)._allreduce_pre_divided(buf).get_future().then(_first)
+
+
+def allreduce_from_grads_hook(process_group, bucket):
+    """allreduce_hook for a model wrapped with DDP's default
+    gradient_as_bucket_view=False: this rank's contribution is read from the
+    parameters' .grad tensors, where autograd left them, instead of from the
+    bucket the reducer has copied them into, and the reduced mean is written to
+    the bucket once. Same result as allreduce_hook, bit for bit. (The reducer
+    still makes its copy before it calls any hook; what this hook shows is the
+    reduction that makes that copy unnecessary, for a reducer that skips it.)
+    Falls back to allreduce_hook when a gradient is missing, is a view into the
+    bucket already, or is not laid out like its place in the bucket."""
+    buf = bucket.buffer()
+    backend = _backend(process_group, buf.device)
+    views = bucket.gradients()
+    grads = [p.grad for p in bucket.parameters()]
+    usable = len(grads) == len(views) and all(
+        g is not None and g.dtype == buf.dtype and g.device == buf.device
+        and g.shape == v.shape and g.stride() == v.stride()
+        and g.untyped_storage().data_ptr() != buf.untyped_storage().data_ptr()
+        for g, v in zip(grads, views))
+    if not usable or sum(g.numel() for g in grads) != buf.numel():
+        return backend._allreduce_pre_divided(buf).get_future().then(_first)
+    return backend._allreduce_from_grads(buf, grads, True).get_future().then(_first)
 
 
 def _compress_hook(dtype, process_group, bucket):

@@ -131,6 +131,33 @@ def reduce_slice_static(out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0,
         stream.cuda_stream))
 
 
+def reduce_pieces(pieces, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+    """Several reductions of one kind as one call (frg_reduce_pieces): `pieces`
+    is a list of (out, [contributions]) with the same number of contributions
+    and dtype throughout; small tensors share launches."""
+    import torch
+    if not pieces:
+        return
+    out0, c0 = pieces[0]
+    stream = torch.cuda.current_stream(out0.device) if stream is None else stream
+    k = len(c0)
+    arr = (_capi.Piece * len(pieces))()
+    keep = []
+    for i, (out, contribs) in enumerate(pieces):
+        if len(contribs) != k or out.dtype != out0.dtype:
+            raise FairringError(_capi.ERR_INVALID, "pieces differ in kind")
+        for c in contribs:
+            if c.numel() != out.numel() or c.dtype != out.dtype:
+                raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        keep.append(tab)
+        arr[i].out = out.data_ptr()
+        arr[i].contribs = ctypes.cast(tab, ctypes.POINTER(ctypes.c_void_p))
+        arr[i].numel = out.numel()
+    _capi.check(_capi.lib().frg_reduce_pieces(arr, len(pieces), k, _dtype_code(out0), op,
+                                              scale_mode, scale, stream.cuda_stream))
+
+
 def _check_compressed(out, contribs, raw_index):
     """Shapes and types of the reduction with compression folded in; returns
     the wire dtype code."""
@@ -314,6 +341,48 @@ class DeviceFairring:
             ctypes.byref(wh)))
         return Work(wh, (out, list(contribs)))
 
+    def allreduce_gathered(self, out, contribs, gathered_index, segments, op=SUM,
+                           scale_mode=SCALE_NONE, scale=1.0, stream=None, done=None):
+        """allreduce with contribution `gathered_index` given as the list of
+        tensors `segments`, in the order they lie in `out` (a bucket's own
+        gradients where autograd left them); contribs[gathered_index] is ignored
+        and may be None (frg_allreduce_gathered). Returns at once."""
+        import torch
+        _check_dense(out, "output")
+        total = 0
+        for t in segments:
+            _check_dense(t, "segment")
+            if t.dtype != out.dtype:
+                raise FairringError(_capi.ERR_INVALID, "segment dtype mismatch")
+            total += t.numel()
+        if total != out.numel():
+            raise FairringError(_capi.ERR_INVALID, "the segments hold %d elements, the output %d"
+                                % (total, out.numel()))
+        ptrs = []
+        for k, c in enumerate(contribs):
+            if k == gathered_index:
+                ptrs.append(out.data_ptr())
+                continue
+            _check_dense(c, "contribution")
+            if c.numel() != out.numel() or c.dtype != out.dtype:
+                raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+            ptrs.append(c.data_ptr())
+        stream = torch.cuda.current_stream(out.device) if stream is None else stream
+        tab = _capi.ptr_table(ptrs)
+        segs = (_capi.Segment * max(len(segments), 1))()
+        for i, t in enumerate(segments):
+            segs[i].ptr = t.data_ptr()
+            segs[i].numel = t.numel()
+        wh = ctypes.c_void_p()
+        others = [c for k, c in enumerate(contribs) if k != gathered_index]
+        self._record_on_streams([out] + others + list(segments))
+        cb = _capi.DONE_FN(done) if done is not None else _capi.DONE_FN()
+        _capi.check(_capi.lib().frg_allreduce_gathered(
+            self._h, out.data_ptr(), tab, len(contribs), gathered_index, segs, len(segments),
+            out.numel(), _dtype_code(out), op, scale_mode, scale, stream.cuda_stream, cb, None,
+            ctypes.byref(wh)))
+        return Work(wh, (out, others, list(segments), cb))
+
     def allreduce_host(self, out, host_contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0,
                        carry=False, stream=None):
         """Server-side accumulation of contributions held in pinned host memory;
@@ -326,27 +395,54 @@ class DeviceFairring:
         return self._submit(out, host_contribs, op, scale_mode, scale, stream, host=True,
                             carry=carry)
 
-    def prepare(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+    def prepare(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None,
+                gathered=None):
         """Validate and marshal an allreduce once; the returned callable submits
         it with a single foreign call (for callers that repeat the same
         operation, e.g. one per DDP bucket per step). The callable returns a
         Work; the tensors stay referenced by the callable and are recorded on
-        the pipeline's streams once, here."""
+        the pipeline's streams once, here. `gathered` = (index, [tensors]) gives
+        that contribution piecewise (allreduce_gathered)."""
         import torch
         _check_dense(out, "output")
-        for c in contribs:
+        g_index, g_tensors = gathered if gathered is not None else (-1, [])
+        ptrs = []
+        for k, c in enumerate(contribs):
+            if k == g_index:
+                ptrs.append(out.data_ptr())
+                continue
             _check_dense(c, "contribution")
             if c.numel() != out.numel() or c.dtype != out.dtype:
                 raise FairringError(_capi.ERR_INVALID, "contribution shape/dtype mismatch")
+            ptrs.append(c.data_ptr())
         stream = torch.cuda.current_stream(out.device) if stream is None else stream
-        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        tab = _capi.ptr_table(ptrs)
         L = _capi.lib()
-        fn = L.frg_allreduce
-        args = (self._h, ctypes.c_void_p(out.data_ptr()), tab, len(contribs),
-                ctypes.c_int64(out.numel()), _dtype_code(out), op, scale_mode,
-                ctypes.c_float(scale), ctypes.c_void_p(stream.cuda_stream), _capi.DONE_FN(), None)
-        keep = (out, list(contribs), tab)
-        self._record_on_streams([out] + list(contribs))
+        others = [c for k, c in enumerate(contribs) if k != g_index]
+        if gathered is None:
+            fn = L.frg_allreduce
+            args = (self._h, ctypes.c_void_p(out.data_ptr()), tab, len(contribs),
+                    ctypes.c_int64(out.numel()), _dtype_code(out), op, scale_mode,
+                    ctypes.c_float(scale), ctypes.c_void_p(stream.cuda_stream), _capi.DONE_FN(),
+                    None)
+            keep = (out, others, tab)
+        else:
+            if sum(t.numel() for t in g_tensors) != out.numel():
+                raise FairringError(_capi.ERR_INVALID, "the segments do not add up to the output")
+            segs = (_capi.Segment * max(len(g_tensors), 1))()
+            for i, t in enumerate(g_tensors):
+                _check_dense(t, "segment")
+                if t.dtype != out.dtype:
+                    raise FairringError(_capi.ERR_INVALID, "segment dtype mismatch")
+                segs[i].ptr = t.data_ptr()
+                segs[i].numel = t.numel()
+            fn = L.frg_allreduce_gathered
+            args = (self._h, ctypes.c_void_p(out.data_ptr()), tab, len(contribs), g_index, segs,
+                    len(g_tensors), ctypes.c_int64(out.numel()), _dtype_code(out), op, scale_mode,
+                    ctypes.c_float(scale), ctypes.c_void_p(stream.cuda_stream), _capi.DONE_FN(),
+                    None)
+            keep = (out, others, tab, segs, list(g_tensors))
+        self._record_on_streams([out] + others + list(g_tensors))
 
         def submit():
             wh = ctypes.c_void_p()

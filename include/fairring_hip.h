@@ -148,6 +148,27 @@ FRG_API int frg_reduce_slice(void* out, const void* const* contribs, int K,
                              int64_t n, int dtype, int op, int scale_mode,
                              float scale, int carry, void* stream);
 
+/* Not in the reference, which reduces one contiguous shard per library call:
+ * several reductions of the same kind (K, element type, operator, scale) as one
+ * call on `stream`. Each piece is an elementwise reduction of its own, with an
+ * output, K contributions and a length, anywhere in device memory; an output
+ * may be one of its piece's contributions, pieces must not overlap each other.
+ * Sums of fp32, bf16 or fp16 with up to 16 contributions whose pointers agree
+ * modulo 16 bytes within a piece are packed up to 24 at a time (12 beyond 8
+ * contributions) into launches of one kernel that deals the 4 KiB tiles of all
+ * of them to one grid: many small tensors cost one launch, not one each.
+ * Whatever does not fit that (MAX, other types, more contributions, a piece
+ * with misaligned pointers) is launched on its own, as frg_reduce_slice would.
+ * Results are those of frg_reduce_slice piece by piece, bit for bit. Allocates
+ * nothing and records no event: fit for a stream under graph capture. */
+typedef struct frg_piece {
+  void* out;
+  const void* const* contribs; /* K device pointers */
+  int64_t numel;
+} frg_piece;
+FRG_API int frg_reduce_pieces(const frg_piece* pieces, int num_pieces, int K, int dtype, int op,
+                              int scale_mode, float scale, void* stream);
+
 /* No counterpart in the reference. frg_reduce_slice for any number of
  * contributions, for callers that cannot allocate: a stream that is being
  * captured into a HIP graph, a tight serving loop, a harness that forbids
@@ -308,6 +329,34 @@ FRG_API int frg_allreduce(frg_ctx* ctx, void* out, const void* const* contribs,
                           int scale_mode, float scale, void* producer_stream,
                           frg_done_fn done, void* user, frg_work** work);
 
+/* frg_allreduce with one contribution given piecewise: the caller at
+ * fairring/process_group.cc:131-155 is DDP's per-bucket allreduce, and with
+ * DDP's default (gradient_as_bucket_view=False) every gradient has been copied
+ * into the bucket just before (torch:csrc/distributed/c10d/reducer.cpp,
+ * mark_variable_ready_dense -> copy_grad_to_bucket; with no hook registered the
+ * copy also multiplies by 1/world). Here contribution `gathered_index` is read
+ * from where autograd left it: `segments` lists the gradient tensors in the
+ * order they lie in the bucket (their lengths add up to `numel`), `out` is the
+ * bucket, contribs[gathered_index] is ignored and the other contributions are
+ * whole buckets as in frg_allreduce. The result is that of frg_allreduce on the
+ * bucket with the segments copied into it, bit for bit (with a pre-scale, as
+ * everywhere, every term is scaled and rounded before the fold, which is what
+ * the fused copy-and-divide leaves); the copy itself, 8 bytes per element of
+ * HBM traffic, is not made. `out` must not be one of the other contributions.
+ * Segments whose position in the bucket is a multiple of 16 bytes away from
+ * their own address modulo 16 run through the kernel of frg_reduce_pieces,
+ * packed into launches of a plain operation's size; the others, and reductions
+ * that kernel does not cover, as launches of their own. */
+typedef struct frg_segment {
+  const void* ptr;
+  int64_t numel;
+} frg_segment;
+FRG_API int frg_allreduce_gathered(frg_ctx* ctx, void* out, const void* const* contribs, int K,
+                                   int gathered_index, const frg_segment* segments,
+                                   int num_segments, int64_t numel, int dtype, int op,
+                                   int scale_mode, float scale, void* producer_stream,
+                                   frg_done_fn done, void* user, frg_work** work);
+
 /* frg_reduce_slice_compressed through the pipeline: sliced by the wire type's
  * element size (the tensor the reference would be handed is the compressed
  * one), launches dealt to the reduce streams like frg_allreduce's. */
@@ -442,7 +491,7 @@ FRG_API const char* frg_last_error(void);
  * frg_reduce_slice_static added (and frg_progress grew in place, which 0.3
  * takes back). 0.3: frg_progress has its four fields of 0.1 again and
  * frg_get_progress2 carries the later counters with the caller's struct size;
- * frg_allreduce_gathered added. */
+ * frg_allreduce_gathered and frg_reduce_pieces added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus

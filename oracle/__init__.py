@@ -141,6 +141,23 @@ def reduce(kind, contribs, op="sum", scale_mode=SCALE_NONE, scale=1.0):
     return out
 
 
+def gathered_reduce(kind, contribs, gathered_index, segments, op="sum", scale_mode=SCALE_NONE,
+                    scale=1.0):
+    """The allreduce of a bucket whose own contribution still lies in separate
+    gradient tensors: what the per-bucket allreduce of
+    fairring/process_group.cc:131-155 returns after DDP has copied every gradient
+    to its place in the bucket (torch:csrc/distributed/c10d/reducer.cpp,
+    copy_grad_to_bucket: bucket_view.copy_(grad), views laid end to end in the
+    flat bucket). `segments` are those tensors in bucket order; their
+    concatenation takes the place of contribs[gathered_index] (ignored, may be
+    None); the rest is `reduce`."""
+    npdt, _ = TYPES[kind]
+    own = (np.concatenate([np.ascontiguousarray(s, dtype=npdt).reshape(-1) for s in segments])
+           if segments else np.empty(0, npdt))
+    full = [own if k == gathered_index else c for k, c in enumerate(contribs)]
+    return reduce(kind, full, op, scale_mode, scale)
+
+
 def compressed_sum(contribs, raw_index, wire="bf16", scale_mode=SCALE_NONE, scale=1.0,
                    out_f32=True, threads=1):
     """torch's compress hook + allreduce + decompress for one rank's bucket.

@@ -147,6 +147,39 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
   return FRG_OK;
 }
 
+int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err);
+
+// The segmented launch: every piece as a unit of work of its own, in order (the
+// packing into launches and the cuts on tiles are the pipeline's and are what is
+// under test; the real kernel's limits are checked here as it checks them).
+int launchSegmented(const SegmentedArgs& a, hipStream_t stream, std::string* err) {
+  auto fail = [&](int code, const char* msg) {
+    if (err) *err = msg;
+    return code;
+  };
+  if (!segmentedKind(a.K, a.dtype, FRG_SUM, false)) return fail(FRG_ERR_UNSUPPORTED, "not a segmented kind");
+  if (a.numPieces < 0 || a.numPieces > maxSegmentsPerLaunch(a.K)) return fail(FRG_ERR_INVALID, "too many pieces");
+  for (int i = 0; i < a.numPieces; ++i) {
+    const SegPiece& pc = a.pieces[i];
+    if (pc.n == 0) continue;
+    if (!segmentable(pc.out, pc.contribs, a.K, elementSize(a.dtype))) {
+      return fail(FRG_ERR_INVALID, "piece not congruent modulo 16");
+    }
+    ReduceArgs r;
+    r.out = pc.out;
+    r.contribs = pc.contribs;
+    r.K = a.K;
+    r.n = pc.n;
+    r.dtype = a.dtype;
+    r.op = FRG_SUM;
+    r.scale_mode = a.scale_mode;
+    r.scale = a.scale;
+    const int rc = launchReduce(r, stream, err);
+    if (rc != FRG_OK) return rc;
+  }
+  return FRG_OK;
+}
+
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
   auto fail = [&](int code, const char* msg) {
     if (err) *err = msg;

@@ -950,6 +950,99 @@ void scenarioHostStaged() {
   }
 }
 
+void scenarioGathered() {
+  std::puts("one contribution given piecewise: cut on tiles, packed into segmented launches");
+  std::mt19937 rng(321);
+  for (int round = 0; round < 6; ++round) {
+    const int k = round % 2 == 0 ? 8 : 3;
+    const int g = static_cast<int>(rng() % k);
+    // segment lengths: big ones (one crosses a launch's 8 MiB), tiny ones, odd ones
+    std::vector<int64_t> lens;
+    if (round < 2) {
+      lens = {2500000, 2048, 2048, 700000, 0, 4096, 1, 3};
+    } else if (round == 2) {
+      lens = {5000000, 16, 2048, 1200000};  // 23.7 MiB: launches of 8 + 8 + the rest
+    } else {
+      const int count = 1 + static_cast<int>(rng() % 40);
+      for (int i = 0; i < count; ++i) {
+        const int kind = static_cast<int>(rng() % 4);
+        lens.push_back(kind == 0 ? static_cast<int64_t>(rng() % 9)
+                                 : (kind == 1 ? 4 * static_cast<int64_t>(rng() % 3000)
+                                              : static_cast<int64_t>(rng() % 50000)));
+      }
+    }
+    int64_t n = 0;
+    for (int64_t l : lens) n += l;
+    auto c = randomContribs(k, n, 600 + round);
+    // the gathered contribution lives in tensors of its own (some start off a 16-byte boundary)
+    std::vector<Vec> pieces;
+    std::vector<frg_segment> segs;
+    int64_t off = 0;
+    for (size_t i = 0; i < lens.size(); ++i) {
+      const int64_t skew = (round >= 4 && i % 3 == 1) ? 1 : 0;
+      Vec v(static_cast<size_t>(lens[i] + skew + 4));
+      for (int64_t j = 0; j < lens[i]; ++j) v[static_cast<size_t>(j + skew)] = c[g][static_cast<size_t>(off + j)];
+      pieces.push_back(std::move(v));
+      off += lens[i];
+    }
+    for (size_t i = 0; i < lens.size(); ++i) {
+      const int64_t skew = (round >= 4 && i % 3 == 1) ? 1 : 0;
+      segs.push_back(frg_segment{pieces[i].data() + skew, lens[i]});
+    }
+    auto t = table(c);
+    t[static_cast<size_t>(g)] = nullptr;  // ignored
+    frg_ctx* ctx = makeCtx(8192, 4096, 2, 0);
+    Vec out(static_cast<size_t>(n), -1.f);
+    frg_work* w = nullptr;
+    const int mode = round % 3 == 0 ? FRG_SCALE_MUL : (round % 3 == 1 ? FRG_SCALE_PRE_MUL : FRG_SCALE_NONE);
+    CHECK(frg_allreduce_gathered(ctx, out.data(), t.data(), k, g, segs.data(),
+                                 static_cast<int>(segs.size()), n, FRG_F32, FRG_SUM, mode, 0.125f,
+                                 nullptr, nullptr, nullptr, &w) == FRG_OK);
+    CHECK(frg_work_wait(w) == FRG_OK);
+    CHECK(same(out, fold(c, mode, 0.125f)));
+    frg_work_release(w);
+    frg_progress2 pr = {};
+    CHECK(frg_get_progress2(ctx, &pr, sizeof(pr)) == FRG_OK);
+    CHECK(pr.segmented_launches >= 1);
+    if (round == 2) {
+      CHECK(pr.segmented_launches == 3 && pr.launches == 3);  // 2048 + 2048 + 1974 tiles
+    }
+    if (round == 0) {
+      // 3.2 M elements of 8 contributions, 12.2 MiB each: a launch of 8 MiB and one with the
+      // rest (more than half a launch's worth); the last piece sits 4 bytes off its tensor's
+      // position within 16 bytes (a one-element piece lies ahead of it): a plain launch of its own
+      CHECK(pr.segmented_launches == 2 && pr.launches == 3);
+    }
+    // MAX is not the segmented kernel's: every piece as a plain launch, same result as the fold
+    Vec mx(static_cast<size_t>(n), -1.f);
+    CHECK(frg_allreduce_gathered(ctx, mx.data(), t.data(), k, g, segs.data(),
+                                 static_cast<int>(segs.size()), n, FRG_F32, FRG_MAX, FRG_SCALE_NONE,
+                                 1.f, nullptr, nullptr, nullptr, &w) == FRG_OK);
+    CHECK(frg_work_wait(w) == FRG_OK);
+    for (int64_t i = 0; i < n; ++i) {
+      float m = c[0][static_cast<size_t>(i)];
+      for (int kk = 1; kk < k; ++kk) m = m > c[kk][static_cast<size_t>(i)] ? m : c[kk][static_cast<size_t>(i)];
+      CHECK(mx[static_cast<size_t>(i)] == m);
+    }
+    frg_work_release(w);
+    // contract: lengths must add up, the index must be in range, the output no other contribution
+    CHECK(frg_allreduce_gathered(ctx, out.data(), t.data(), k, g, segs.data(),
+                                 static_cast<int>(segs.size()), n + 1, FRG_F32, FRG_SUM, 0, 1.f,
+                                 nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+    CHECK(frg_allreduce_gathered(ctx, out.data(), t.data(), k, k, segs.data(),
+                                 static_cast<int>(segs.size()), n, FRG_F32, FRG_SUM, 0, 1.f,
+                                 nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+    if (n > 0) {
+      auto alias = t;
+      alias[static_cast<size_t>((g + 1) % k)] = out.data();
+      CHECK(frg_allreduce_gathered(ctx, out.data(), alias.data(), k, g, segs.data(),
+                                   static_cast<int>(segs.size()), n, FRG_F32, FRG_SUM, 0, 1.f,
+                                   nullptr, nullptr, nullptr, nullptr) == FRG_ERR_INVALID);
+    }
+    CHECK(frg_destroy(ctx) == FRG_OK);
+  }
+}
+
 bool gSharedHwQueues = false;
 
 // Streams of a context as the ABI hands them out (reduce streams first).
@@ -1507,6 +1600,7 @@ void runAll() {
       {"order between operations", scenarioOrderBetweenOperations},
       {"random dependent operations", scenarioRandomDependentOperations},
       {"host staged", scenarioHostStaged},
+      {"gathered contribution", scenarioGathered},
       {"callback", scenarioCallback},
       {"process-group-shaped", scenarioProcessGroupShaped},
       {"errors", scenarioErrors},

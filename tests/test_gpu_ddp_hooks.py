@@ -89,6 +89,75 @@ def test_compressed_allreduce(wire, tdt, rank, size):
                       oracle.compressed_sum(contribs, rank, wire, oracle.SCALE_MUL, s))
 
 
+class GradBucket(Bucket):
+    """A bucket with the parameters it was assembled from."""
+
+    def __init__(self, t, params):
+        super().__init__(t)
+        self._params = params
+
+    def parameters(self):
+        return self._params
+
+    def gradients(self):
+        views, off = [], 0
+        for p in self._params:
+            views.append(self._t[off:off + p.numel()].view_as(p))
+            off += p.numel()
+        return views
+
+
+@pytest.mark.parametrize("kind,tdt", [("f32", torch.float32), ("bf16", torch.bfloat16)])
+@pytest.mark.parametrize("rank,size", [(0, 2), (5, 8), (2, 3)])
+def test_allreduce_from_grads(kind, tdt, rank, size):
+    # the bucket's own contribution is read from the gradient tensors; the bucket itself holds
+    # garbage on the way in
+    print("[case] pg from grads", kind, rank, size, flush=True)
+    shapes = [(1024, 512), (512,), (1,), (300, 7), (64, 64, 3), (5,)]
+    n = sum(int(np.prod(sh)) for sh in shapes)
+    rng = np.random.default_rng(40 * size + rank)
+    x = (rng.standard_normal((size, n)) * 0.01).astype(np.float32)
+    if kind == "bf16":
+        bits = oracle.np_f32_to_bf16_rne(x)
+        host = list(bits)
+        dev_of = lambda a: torch.from_numpy(a.view(np.int16).copy()).to(DEV).view(tdt)  # noqa: E731
+    else:
+        host = list(x)
+        dev_of = lambda a: torch.from_numpy(a.copy()).to(DEV)  # noqa: E731
+    pg = make_pg(rank, size)
+    pg._set_simulated_peer_contributions([dev_of(host[r]) for r in range(size) if r != rank])
+    grads, off = [], 0
+    for sh in shapes:
+        ln = int(np.prod(sh))
+        grads.append(dev_of(host[rank][off:off + ln]).view(sh))
+        off += ln
+    s = float(np.float32(1) / np.float32(size))
+    for pre in (True, False):
+        bucket = torch.full((n,), float("nan"), dtype=tdt, device=DEV)
+        work = pg._allreduce_from_grads(bucket, grads, pre)
+        work.wait()
+        torch.cuda.synchronize()
+        want = oracle.reduce(kind, host, "sum", oracle.SCALE_PRE_MUL if pre else oracle.SCALE_NONE, s)
+        got = bucket.cpu().numpy() if kind == "f32" else bits16(bucket)
+        assert_bits_equal(got, want, "%s pre=%s" % (kind, pre))
+    # the hook: same bits as allreduce_hook on a bucket the gradients were copied into
+    params = []
+    for gr in grads:
+        p = torch.nn.Parameter(torch.zeros_like(gr))
+        p.grad = gr
+        params.append(p)
+    bucket = torch.cat([gr.reshape(-1) for gr in grads])
+    via_hook = ddp_comm_hooks.allreduce_from_grads_hook(pg, GradBucket(bucket.clone().fill_(7), params))
+    got = via_hook.wait()
+    torch.cuda.synchronize()
+    want = ddp_comm_hooks.allreduce_hook(pg, Bucket(bucket)).wait()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16 if kind == "bf16" else torch.int32),
+                       want.view(torch.int16 if kind == "bf16" else torch.int32))
+    with pytest.raises(RuntimeError, match="gradients hold"):
+        pg._allreduce_from_grads(bucket, grads[:-1], True)
+
+
 def test_hook_contract_errors():
     print("[case] pg hook errors", flush=True)
     pg = make_pg(0, 2)
@@ -141,6 +210,11 @@ for name in ("allreduce_hook", "bf16_compress_hook", "fp16_compress_hook"):
     print(name, "ok", flush=True)
 for a, b in zip(plain, grads(ours.allreduce_hook)):
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+# gradient_as_bucket_view=False is DDP's default, used above: the hook that reads the gradients
+# where autograd left them gives the bits of torch's allreduce_hook
+for a, b in zip(grads(torch_hooks.allreduce_hook), grads(ours.allreduce_from_grads_hook)):
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+print("allreduce_from_grads_hook ok", flush=True)
 print("ddp hooks ok")
 dist.destroy_process_group()
 """

@@ -1,0 +1,208 @@
+"""GPU parity of the launches over several pieces (frg_reduce_pieces) and of the allreduce
+with one contribution given piecewise (frg_allreduce_gathered: a bucket's own gradients read
+from where autograd left them), through the C ABI, against the CPU oracle. Bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+
+fa = pytest.importorskip("fairring_amd")
+
+DEV = "cuda:0"
+MiB = 1024 * 1024
+KINDS = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def _print_case(*a):
+    print("[case]", *a, flush=True)
+
+
+def host_values(kind, rng, shape):
+    """Random values of the kind as the oracle takes them (fp32, or uint16 bit patterns)."""
+    x = (rng.standard_normal(shape) * 0.01).astype(np.float32)
+    if kind == "f32":
+        return x
+    if kind == "bf16":
+        return oracle.np_f32_to_bf16_rne(x)
+    return x.astype(np.float16).view(np.uint16)
+
+
+def to_gpu(kind, a, skew=0):
+    """A GPU tensor holding `a`, starting `skew` elements past a 16-byte boundary."""
+    a = np.ascontiguousarray(a)
+    if kind == "f32":
+        t = torch.from_numpy(a)
+    else:
+        t = torch.from_numpy(a.view(np.int16)).view(KINDS[kind])
+    buf = torch.empty(a.size + skew + 8, dtype=t.dtype, device=DEV)
+    buf[skew:skew + a.size].copy_(t)
+    return buf[skew:skew + a.size]
+
+
+def from_gpu(kind, t):
+    if kind == "f32":
+        return t.cpu().numpy()
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+SCALES = [("none", fa.SCALE_NONE, oracle.SCALE_NONE, lambda k: 1.0),
+          ("mul", fa.SCALE_MUL, oracle.SCALE_MUL, lambda k: 1.0 / k),
+          ("div", fa.SCALE_DIV, oracle.SCALE_DIV, lambda k: float(k)),
+          ("pre_mul", fa.SCALE_PRE_MUL, oracle.SCALE_PRE_MUL, lambda k: float(np.float32(1) / np.float32(k))),
+          ("pre_div", fa.SCALE_PRE_DIV, oracle.SCALE_PRE_DIV, lambda k: float(k))]
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("k", [1, 2, 3, 4, 8, 9, 16, 17])
+def test_reduce_pieces_vs_oracle(kind, k):
+    rng = np.random.default_rng(77 * k + len(kind))
+    sizes = [1, 3, 4, 5, 0, 255, 1024, 4099, 262147, 7, 1_500_003, 8, 16, 2048, 33]
+    for name, mode, omode, scale_of in SCALES:
+        _print_case("pieces", kind, k, name)
+        host, pieces, outs = [], [], []
+        for i, n in enumerate(sizes):
+            x = host_values(kind, rng, (k, n))
+            # every third piece has one contribution off the others' position within 16 bytes
+            # (a launch of its own); every fourth is reduced in place
+            skews = [(1 if (i % 3 == 2 and j == k - 1) else 0) for j in range(k)]
+            cs = [to_gpu(kind, x[j], skews[j]) for j in range(k)]
+            out = cs[0] if i % 4 == 3 else torch.empty(n + 8, dtype=KINDS[kind], device=DEV)[:n]
+            host.append(x)
+            pieces.append((out, cs))
+            outs.append(out)
+        fa.reduce_pieces(pieces, scale_mode=mode, scale=scale_of(k))
+        torch.cuda.synchronize()
+        for i, x in enumerate(host):
+            want = oracle.reduce(kind, list(x), "sum", omode, scale_of(k))
+            assert_bits_equal(from_gpu(kind, outs[i]), want, "%s k=%d piece %d (%d el) %s" % (
+                kind, k, i, sizes[i], name), half=kind == "f16")
+
+
+def test_reduce_pieces_many_small_tensors_and_other_kinds():
+    # more pieces than one launch takes; MAX and int32 go piece by piece through the plain kernel
+    _print_case("pieces many")
+    rng = np.random.default_rng(5)
+    k = 8
+    host = [(rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+            for n in rng.integers(1, 3000, size=100)]
+    pieces = [(torch.empty(x.shape[1], device=DEV), [to_gpu("f32", r) for r in x]) for x in host]
+    fa.reduce_pieces(pieces, scale_mode=fa.SCALE_MUL, scale=0.125)
+    torch.cuda.synchronize()
+    for (out, _), x in zip(pieces, host):
+        assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_MUL, 0.125))
+    fa.reduce_pieces(pieces, op=fa.MAX)
+    torch.cuda.synchronize()
+    for (out, _), x in zip(pieces, host):
+        assert_bits_equal(out.cpu().numpy(), oracle.max_f32(list(x)))
+    ih = [rng.integers(-2**31, 2**31, size=(3, n), dtype=np.int64).astype(np.int32) for n in (5, 4099)]
+    ip = [(torch.empty(x.shape[1], dtype=torch.int32, device=DEV),
+           [torch.from_numpy(r.copy()).to(DEV) for r in x]) for x in ih]
+    fa.reduce_pieces(ip)
+    torch.cuda.synchronize()
+    for (out, _), x in zip(ip, ih):
+        assert (out.cpu().numpy() == oracle.reduce("i32", list(x))).all()
+
+
+def bucket_case(kind, rng, k, g, lens, skew_every=0):
+    """Peers' buckets, this rank's gradients as tensors of their own, and the host copies."""
+    n = int(sum(lens))
+    x = host_values(kind, rng, (k, n))
+    peers = [None if j == g else to_gpu(kind, x[j]) for j in range(k)]
+    segs, off = [], 0
+    for i, ln in enumerate(lens):
+        skew = 1 if skew_every and i % skew_every == 1 else 0
+        segs.append(to_gpu(kind, x[g, off:off + ln], skew))
+        off += ln
+    return x, peers, segs, n
+
+
+LAYER = [2048 * 2048, 2048, 2048, 2048 * 512, 2048, 1, 3, 4096, 0, 2048 * 64 + 5, 16]
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+@pytest.mark.parametrize("k,g", [(8, 0), (8, 5), (2, 1), (3, 2), (16, 7)])
+def test_allreduce_gathered_vs_oracle(kind, k, g):
+    rng = np.random.default_rng(31 * k + g)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    for name, mode, omode, scale_of in SCALES[:4]:
+        _print_case("gathered", kind, k, g, name)
+        x, peers, segs, n = bucket_case(kind, rng, k, g, LAYER)
+        out = torch.empty(n, dtype=KINDS[kind], device=DEV)
+        dev.allreduce_gathered(out, peers, g, segs, scale_mode=mode, scale=scale_of(k)).wait()
+        want = oracle.reduce(kind, list(x), "sum", omode, scale_of(k))
+        assert_bits_equal(from_gpu(kind, out), want, "%s k=%d g=%d %s" % (kind, k, g, name))
+    assert dev.progress()["segmented_launches"] > 0
+    dev.close()
+
+
+def test_allreduce_gathered_misaligned_segments_other_reductions_and_the_copy_it_replaces():
+    rng = np.random.default_rng(12)
+    dev = fa.DeviceFairring(0)
+    # gradients that start off a 16-byte boundary, odd lengths ahead of big tensors
+    lens = [5, 300001, 1, 1 << 20, 7, 2048, 2048, 33, 1 << 18]
+    for kind, k, g in (("f32", 8, 3), ("f16", 4, 0), ("bf16", 8, 7)):
+        _print_case("gathered misaligned", kind, k)
+        x, peers, segs, n = bucket_case(kind, rng, k, g, lens, skew_every=2)
+        out = torch.empty(n, dtype=KINDS[kind], device=DEV)
+        dev.allreduce_gathered(out, peers, g, segs, scale_mode=fa.SCALE_MUL, scale=1.0 / k).wait()
+        want = oracle.reduce(kind, list(x), "sum", oracle.SCALE_MUL, 1.0 / k)
+        assert_bits_equal(from_gpu(kind, out), want, kind, half=kind == "f16")
+        # the same bits as copying every gradient into the bucket and reducing that in place
+        bucket = torch.cat(segs)
+        full = [bucket if j == g else peers[j] for j in range(k)]
+        dev.allreduce(bucket, full, scale_mode=fa.SCALE_MUL, scale=1.0 / k).wait()
+        assert torch.equal(bucket.view(torch.int16 if kind != "f32" else torch.int32),
+                           out.view(torch.int16 if kind != "f32" else torch.int32))
+    # more contributions than the segmented kernel takes, and MAX: plain launches per segment
+    _print_case("gathered k=20, max")
+    x, peers, segs, n = bucket_case("f32", rng, 20, 4, [4099, 1, 70000, 2048])
+    out = torch.empty(n, device=DEV)
+    dev.allreduce_gathered(out, peers, 4, segs, scale_mode=fa.SCALE_DIV, scale=20.0).wait()
+    assert_bits_equal(out.cpu().numpy(), oracle.sum_f32(list(x), oracle.SCALE_DIV, 20.0))
+    dev.allreduce_gathered(out, peers, 4, segs, op=fa.MAX).wait()
+    assert_bits_equal(out.cpu().numpy(), oracle.max_f32(list(x)))
+    # 70 bf16 contributions: a chain of launches per segment, one rounding
+    _print_case("gathered k=70 bf16")
+    x, peers, segs, n = bucket_case("bf16", rng, 70, 69, [4099, 3, 30000])
+    out = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    dev.allreduce_gathered(out, peers, 69, segs).wait()
+    assert_bits_equal(from_gpu("bf16", out), oracle.sum_bf16(list(x)))
+    # contract
+    with pytest.raises(fa.FairringError):
+        dev.allreduce_gathered(out, peers, 69, segs[:-1])
+    dev.close()
+
+
+def test_allreduce_gathered_waits_for_the_gradients_and_orders_what_follows():
+    # the gradients are still being written on the caller's stream when the operation is
+    # submitted; and an operation that overwrites a gradient afterwards runs behind it
+    _print_case("gathered ordering")
+    k, g = 8, 2
+    n_big = 8 * MiB
+    dev = fa.DeviceFairring(0)
+    peers = [None if j == g else torch.full((2 * n_big,), float(j), device=DEV) for j in range(k)]
+    for _ in range(3):
+        grads = [torch.zeros(n_big, device=DEV), torch.zeros(n_big, device=DEV)]
+        out = torch.empty(2 * n_big, device=DEV)
+        busy = torch.empty(64 * MiB, device=DEV)
+        for _ in range(6):
+            busy.normal_()                      # keeps the stream busy for a few milliseconds
+        grads[0].fill_(100.0)
+        grads[1].fill_(200.0)
+        w = dev.allreduce_gathered(out, peers, g, grads)
+        # overwrites the first gradient: must run after the operation above has read it
+        ones = [torch.ones(n_big, device=DEV) for _ in range(2)]
+        w2 = dev.allreduce(grads[0], ones)
+        w.wait()
+        w2.wait()
+        torch.cuda.synchronize()
+        rest = float(sum(j for j in range(k) if j != g))
+        assert float(out[:n_big].min()) == rest + 100.0 == float(out[:n_big].max())
+        assert float(out[n_big:].min()) == rest + 200.0 == float(out[n_big:].max())
+        assert float(grads[0].min()) == 2.0 == float(grads[0].max())
+    dev.close()

@@ -339,6 +339,40 @@ def test_allreduce_from_two_threads_and_futures_with_callbacks():
     assert sorted(seen) == [(t, i) for t in range(2) for i in range(30)]
 
 
+def test_peers_replaced_while_operations_wait_in_the_queue_stay_alive():
+    # The command thread is held inside a completion callback (a Python `then` that waits on a
+    # flag) while more operations queue up behind it; the group is then handed new peers, the
+    # old ones are dropped and tensors of the same size, full of other values, are allocated at
+    # once (the caching allocator hands a freed block straight back). The queued operations must
+    # still see the peers they were submitted with.
+    print("[case] pg peers replaced under queued operations", flush=True)
+    import threading
+    n = 1 << 23           # large enough to go through the command thread, not the caller's stream
+    pg = make_pg(0, 2)
+    warm = torch.ones(n, device=DEV)
+    pg._set_simulated_peer_contributions([torch.ones(n, device=DEV)])
+    pg.allreduce([warm]).wait()
+    torch.cuda.synchronize()
+    gate = threading.Event()
+    first = torch.zeros(n, device=DEV)
+    pg._set_simulated_peer_contributions([torch.full((n,), 10.0, device=DEV)])
+    held = pg.allreduce([first]).get_future().then(lambda f: gate.wait(30))
+    owns = [torch.full((n,), float(i), device=DEV) for i in range(1, 5)]
+    works = [pg.allreduce([o]) for o in owns]            # queued behind the held thread
+    pg._set_simulated_peer_contributions([torch.full((n,), -1.0, device=DEV)])
+    junk = [torch.full((n,), 12345.0, device=DEV) for _ in range(4)]   # lands where the old peer was
+    torch.cuda.synchronize()
+    gate.set()
+    held.wait()
+    for w in works:
+        w.wait()
+    torch.cuda.synchronize()
+    assert float(first[0]) == 10.0
+    for i, o in enumerate(owns, start=1):
+        assert float(o.min()) == float(o.max()) == i + 10.0, (i, float(o.min()), float(o.max()))
+    del junk
+
+
 def test_missing_peers_is_a_loud_error():
     print("[case] pg missing peers", flush=True)
     pg = make_pg(0, 2)

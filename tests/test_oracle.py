@@ -352,6 +352,45 @@ def test_pre_scale_matches_torch_allreduce_hook(world):
                       "f64 pre-div")
 
 
+@pytest.mark.parametrize("world,rank", [(2, 1), (8, 3), (5, 0)])
+def test_gathered_reduce_matches_torch_bucket_assembly(world, rank):
+    # What DDP's reducer does ahead of the allreduce, run by the installed torch: every gradient
+    # is copied to its place in the flat bucket (torch.cat lays them end to end like the bucket
+    # views), multiplied by 1/world where no hook is registered (mul_out into the view), and the
+    # buckets are summed in rank order.
+    rng = np.random.default_rng(900 + world)
+    lens = [4099, 1, 0, 2048, 3, 70001]
+    n = sum(lens)
+    x = _wide_f32(rng, (world, n))
+    grads = [torch.from_numpy(x[rank, sum(lens[:i]):sum(lens[:i + 1])].copy()) for i in range(len(lens))]
+    s = np.float32(1) / np.float32(world)
+    for pre in (False, True):
+        buckets = [torch.from_numpy(r.copy()) for r in x]
+        buckets[rank] = torch.cat(grads)
+        if pre:
+            buckets = [b.mul(torch.tensor(s)) for b in buckets]
+        acc = buckets[0].clone()
+        for b in buckets[1:]:
+            acc = torch.add(acc, b)
+        contribs = [None if k == rank else x[k] for k in range(world)]
+        got = oracle.gathered_reduce("f32", contribs, rank, [g.numpy() for g in grads], "sum",
+                                     oracle.SCALE_PRE_MUL if pre else oracle.SCALE_NONE, float(s))
+        assert_bits_equal(got, acc.numpy(), "gathered, pre-scale %s" % pre)
+    # bf16 gradients: one rounding at the end of an fp32 fold, like the plain sum
+    h = [torch.from_numpy(r.copy()).to(torch.bfloat16) for r in x]
+    hg = [g.to(torch.bfloat16) for g in grads]
+    hb = list(h)
+    hb[rank] = torch.cat(hg)
+    acc = hb[0].float()
+    for b in hb[1:]:
+        acc = acc + b.float()
+    want = acc.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    bits = [None if k == rank else t.view(torch.int16).numpy().view(np.uint16) for k, t in enumerate(h)]
+    got = oracle.gathered_reduce("bf16", bits, rank,
+                                 [g.view(torch.int16).numpy().view(np.uint16) for g in hg])
+    assert_bits_equal(got, want, "gathered bf16")
+
+
 @pytest.mark.parametrize("wire,dt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
 @pytest.mark.parametrize("world", [1, 2, 3, 8, 64])
 def test_compressed_sum_matches_torch_compress_hook(wire, dt, world):
