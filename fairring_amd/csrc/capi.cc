@@ -498,6 +498,12 @@ int frg_set_tuning(int blocks_per_cu) {
   return FRG_OK;
 }
 
+int frg_set_tile_runs(int log2_tiles) {
+  if (log2_tiles < 0 || log2_tiles > 12) return fail(FRG_ERR_INVALID, "log2_tiles must be in [0, 12]");
+  frg::setXcdChunkShift(log2_tiles);
+  return FRG_OK;
+}
+
 const char* frg_last_error(void) { return frg::lastError(); }
 
 const char* frg_version(void) { return "0.3"; }

@@ -159,6 +159,9 @@ int launchSegmented(const SegmentedArgs& args, hipStream_t stream, std::string* 
 
 // Launch-shape knobs (process-wide); 0 keeps the default.
 void setTuning(int blocksPerCu);
+// log2 of the consecutive 4 KiB tiles the blocks of one XCD take in a row (6 by
+// default: 256 KiB; 0: tile = block index). For measurements.
+void setXcdChunkShift(int shift);
 
 // Compute units of a device (cached).
 int computeUnits(int device);

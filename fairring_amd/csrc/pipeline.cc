@@ -287,9 +287,6 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   c->maxLaunchBytes_ = o.max_launch_bytes == 0 ? kDefaultMaxLaunchBytes
                                                : (o.max_launch_bytes < 0 ? 0 : o.max_launch_bytes);
   c->maxLaunchBytes_ -= c->maxLaunchBytes_ % 16;  // keep every launch 16-byte congruent
-  if (const char* v = std::getenv("FAIRRING_IDLE_PRODUCER_CHECK")) {
-    c->idleProducerCheck_ = std::atoi(v) != 0;
-  }
   if (const char* v = std::getenv("FAIRRING_MERGE_OPERATIONS")) {
     const long long m = std::atoll(v);
     if (m >= 1 && m <= 1024) c->mergeOperations_ = static_cast<int>(m);
@@ -297,10 +294,6 @@ int Context::create(int device, const frg_options& o, Context** out, std::string
   if (const char* v = std::getenv("FAIRRING_INLINE_BYTES")) {
     const long long b = std::atoll(v);
     if (b >= 0) c->inlineTrafficBytes_ = b;
-  }
-  if (const char* v = std::getenv("FAIRRING_ONE_STREAM_LAUNCHES")) {
-    const long long m = std::atoll(v);
-    if (m >= 0 && m <= 1 << 20) c->oneStreamLaunches_ = static_cast<int>(m);
   }
   if (const char* v = std::getenv("FAIRRING_CHAIN_SCRATCH_BYTES")) {
     const long long b = std::atoll(v);
@@ -867,7 +860,7 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
     // runtime flushes its queue to find out) against 1 for the record: after a
     // "busy" the next operations from that stream record without asking.
     bool producerIdle = false;
-    if (idleProducerCheck_) {
+    {
       if (busyProducer_.load(std::memory_order_relaxed) == req.producerStream &&
           busyProducerSkips_.load(std::memory_order_relaxed) > 0) {
         busyProducerSkips_.fetch_sub(1, std::memory_order_relaxed);

@@ -293,7 +293,7 @@ class DeviceFairring:
                     padding_slots=out.num_padding_slots,
                     staging_slots=out.num_staging_slots)
 
-    def _submit(self, out, contribs, op, scale_mode, scale, stream, host, carry=False):
+    def _submit(self, out, contribs, op, scale_mode, scale, stream, host, carry=False, done=None):
         import torch
         _check_dense(out, "output")
         for c in contribs:
@@ -305,20 +305,26 @@ class DeviceFairring:
         L = _capi.lib()
         head = (self._h, out.data_ptr(), tab, len(contribs), out.numel(), _dtype_code(out), op,
                 scale_mode, scale)
-        tail = (stream.cuda_stream, _capi.DONE_FN(), None, ctypes.byref(wh))
+        cb = _capi.DONE_FN(done) if done is not None else _capi.DONE_FN()
+        tail = (stream.cuda_stream, cb, None, ctypes.byref(wh))
         self._record_on_streams([out] if host else [out] + list(contribs), host=host)
         if host:
             _capi.check(L.frg_allreduce_host(*head, 1 if carry else 0, *tail))
         else:
             _capi.check(L.frg_allreduce(*head, *tail))
-        return Work(wh, (out, list(contribs)))
+        return Work(wh, (out, list(contribs), cb))
 
-    def allreduce(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None):
+    def allreduce(self, out, contribs, op=SUM, scale_mode=SCALE_NONE, scale=1.0, stream=None,
+                  done=None):
         """DeviceFairring::allReduce (fairring/device.cc:291-353) with the peers'
-        contributions given as GPU tensors. Returns at once."""
+        contributions given as GPU tensors. Returns at once. `done(user, status,
+        last_stream)`, if given, is the completion callback of frg_allreduce: it
+        runs on the pipeline's command thread once the operation is enqueued (or
+        on this thread, before the call returns, for a small operation launched
+        on the caller's stream)."""
         for c in contribs:
             _check_dense(c, "contribution")
-        return self._submit(out, contribs, op, scale_mode, scale, stream, host=False)
+        return self._submit(out, contribs, op, scale_mode, scale, stream, host=False, done=done)
 
     def allreduce_compressed(self, out, contribs, raw_index=-1, scale_mode=SCALE_NONE, scale=1.0,
                              wire_dtype=None, stream=None):

@@ -484,6 +484,14 @@ FRG_API int frg_launch_records(frg_ctx* ctx, frg_launch_record* records, int cap
  * CU (0 keeps the built-in default, which depends on the loads per lane). */
 FRG_API int frg_set_tuning(int blocks_per_cu);
 
+/* Launch-shape knob of the reduction kernel: log2 of the number of consecutive
+ * 4 KiB tiles that the blocks running on one XCD take in a row within a round
+ * of the grid (the hardware deals the blocks of a launch to the 8 XCDs in
+ * turn). 6, the default, gives every XCD runs of 256 KiB; 0 gives every block
+ * the tile of its own index, so that an XCD reads every eighth tile. Results do
+ * not depend on it. For measurements. */
+FRG_API int frg_set_tile_runs(int log2_tiles);
+
 /* Message of the last failure on the calling thread (or of the failed work). */
 FRG_API const char* frg_last_error(void);
 
@@ -491,7 +499,7 @@ FRG_API const char* frg_last_error(void);
  * frg_reduce_slice_static added (and frg_progress grew in place, which 0.3
  * takes back). 0.3: frg_progress has its four fields of 0.1 again and
  * frg_get_progress2 carries the later counters with the caller's struct size;
- * frg_allreduce_gathered and frg_reduce_pieces added. */
+ * frg_allreduce_gathered, frg_reduce_pieces and frg_set_tile_runs added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus

@@ -39,6 +39,8 @@ bool isFloating(int dtype) {
 
 void setTuning(int) {}
 
+void setXcdChunkShift(int) {}
+
 int computeUnits(int) { return 4; }  // what the stand-in runtime reports
 
 void prepareStaticScratch(int) {}  // device code: not part of the host build

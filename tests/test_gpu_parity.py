@@ -929,6 +929,30 @@ def test_random_sequences_of_dependent_operations_match_sequential_execution(see
         dev.close()
 
 
+class HeldCommandThread:
+    """Keeps the pipeline's command thread inside the completion callback of an operation
+    (24 MiB moved: it goes through the command thread, not the caller's stream) until
+    release() is called, so that whatever is submitted meanwhile is waiting in the queue when
+    the thread takes up work again: what the command thread finds there does not depend on
+    how fast this thread is today."""
+
+    def __init__(self, dev):
+        import threading
+        self.entered, self.gate = threading.Event(), threading.Event()
+        self.buf = torch.zeros(2 * MiB, device=DEV)
+
+        def held(user, status, stream):
+            self.entered.set()
+            self.gate.wait(60)
+
+        self.work = dev.allreduce(self.buf, [self.buf, self.buf], done=held)
+        assert self.entered.wait(60), "the completion callback never ran"
+
+    def release(self):
+        self.gate.set()
+        self.work.wait()
+
+
 def _hold(stream, ballast, times=30):
     """Keeps `stream` busy for a few milliseconds (elementwise passes over 256 MiB)."""
     with torch.cuda.stream(stream):
@@ -1068,9 +1092,13 @@ def test_random_mix_of_small_and_large_operations_from_two_streams(seed, monkeyp
         return w
 
     try:
+        import time
         for episode in range(30):
             dev.synchronize()                              # the pipeline runs empty
             torch.cuda.synchronize()
+            # and stays so for longer than the rule stays off after a reduce stream was found
+            # busy (200 us), so that the episode's first operation is one it applies to for sure
+            time.sleep(0.002)
             first = int(rng.integers(2))
             _hold(producers[first], ballast[first], times=20)
             works = [submit(True, first)]
@@ -1119,20 +1147,17 @@ def test_neighbouring_buckets_waiting_in_the_queue_run_as_one(order):
                  for lo, hi in spans]
         warm = torch.zeros(bucket, device=DEV)
         dev.allreduce(warm, [warm, warm]).wait()
-        # something for the command thread to do meanwhile (some hundred launches), so that the
-        # buckets are waiting when it gets to them however slow this thread is today
-        busy = torch.zeros(256 * MiB, device=DEV)
-        occupy = dev.prepare(busy, [busy, busy])
         torch.cuda.synchronize()
         before = dev.progress()
-        occupied = occupy()
+        # the command thread is held until every bucket is waiting in its queue
+        held = HeldCommandThread(dev)
         works = [call() for call in calls]
+        held.release()
         for w in works:
             assert w.wait() is True
-        occupied.wait()
         after = dev.progress()
         assert after["enqueued"] - before["enqueued"] == len(spans) + 1
-        assert after["merged"] - before["merged"] >= 8       # nearly all of them, in practice
+        assert after["merged"] - before["merged"] == len(spans)   # runs of 16, 16 and 9
         assert bool(torch.equal(out.view(torch.int32), want.view(torch.int32)))
         lo, hi = n - 100_000, n
         assert_bits_equal(out[lo:hi].cpu().numpy(),
@@ -1164,10 +1189,14 @@ def test_neighbouring_operations_that_read_each_others_output_stay_apart():
         warm = torch.zeros(q, device=DEV)
         dev.allreduce(warm, [warm, warm]).wait()
         torch.cuda.synchronize()
+        before = dev.progress()["merged"]
+        held = HeldCommandThread(dev)                      # all 24 are waiting when it lets go
         works = [call() for call in calls]
+        held.release()
         for w in works:
             w.wait()
         assert bool(torch.equal(z.view(torch.int32), want.view(torch.int32)))
+        assert dev.progress()["merged"] - before == count  # six runs of four
     finally:
         dev.close()
 
@@ -1200,17 +1229,15 @@ def test_joined_neighbours_give_the_bits_of_separate_operations(dtype, op, scale
             calls = [dev.prepare(out[lo:hi], [x[lo:hi] for x in xs], **kwargs) for lo, hi in spans]
             dev.allreduce(out[:bucket], [x[:bucket] for x in xs], **kwargs).wait()
             out.zero_()
-            busy = torch.zeros(256 * MiB, device=DEV)      # keeps the command thread at work
-            occupy = dev.prepare(busy, [busy, busy])       # while the buckets queue up
             torch.cuda.synchronize()
             before = dev.progress()["merged"]
-            occupied = occupy()
+            held = HeldCommandThread(dev)                  # until all the buckets are queued
             works = [call() for call in calls]
+            held.release()
             for w in works:
                 w.wait()
-            occupied.wait()
             joined = dev.progress()["merged"] - before
-            assert (joined >= 4) if limit == "16" else (joined == 0)
+            assert joined == (count if limit == "16" else 0)   # runs of 16 and 8, or none
             outs.append(out)
         finally:
             dev.close()
@@ -1222,3 +1249,102 @@ def test_joined_neighbours_give_the_bits_of_separate_operations(dtype, op, scale
     if dtype == torch.int32:
         want = torch.stack(host).amax(dim=0)
         assert bool(torch.equal(outs[0][lo:hi].cpu(), want))
+
+
+KNOBS = [{}, {"FAIRRING_INLINE_BYTES": "0"}, {"FAIRRING_MERGE_OPERATIONS": "1"},
+         {"FAIRRING_SPIN_US": "0"}, {"FAIRRING_CHAIN_SCRATCH_BYTES": "65536"},
+         {"FAIRRING_INLINE_BYTES": "0", "FAIRRING_MERGE_OPERATIONS": "1", "FAIRRING_SPIN_US": "0"}]
+
+
+@pytest.mark.parametrize("knobs", KNOBS, ids=lambda kv: ",".join("%s=%s" % (k[9:], v) for k, v in kv.items()) or "defaults")
+def test_results_do_not_depend_on_the_pipelines_knobs(knobs, monkeypatch):
+    # One fixed mix of operations (small ones, a gradient's buckets in place, a whole gradient
+    # into a separate output, a gathered bucket; from two producer streams that are kept busy;
+    # the command thread held once so that buckets queue up) under every host-side knob's other
+    # setting: the knobs choose streams, launch shapes and who launches, never the bits.
+    _print_case("knob independence", knobs)
+    for key, value in knobs.items():
+        monkeypatch.setenv(key, value)
+    k = 4
+    g = torch.Generator(device=DEV)
+    g.manual_seed(4242)
+    bucket, count = 6_553_600, 6
+    grad = [torch.empty(bucket * count + 777, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    whole = [torch.empty(20_000_003, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    small = [torch.empty(300_000, device=DEV).normal_(0, 0.01, generator=g) for _ in range(k)]
+    host = {name: [t.cpu().numpy() for t in ts] for name, ts in (("grad", grad), ("whole", whole), ("small", small))}
+    ballast = torch.zeros(64 * MiB, device=DEV)
+    producers = [torch.cuda.Stream(), torch.cuda.Stream()]
+    small_out = torch.zeros(300_000, device=DEV)
+    whole_out = torch.empty_like(whole[0])
+    pieces = [whole[2][:1_000_000].clone(), whole[2][1_000_000:1_000_003].clone(),
+              whole[2][1_000_003:3_000_000].clone()]
+    gathered_out = torch.empty(3_000_000, device=DEV)
+    torch.cuda.synchronize()      # everything above was made on the default stream
+    dev = fa.DeviceFairring(0)
+    try:
+        works = []
+        # small operations from a busy producer, in place and not
+        _hold(producers[0], ballast, times=5)
+        cuts = [(0, 1000), (1000, 5_096), (5_096, 70_001), (70_001, 300_000)]
+        for i, (lo, hi) in enumerate(cuts):
+            works.append(dev.allreduce(small_out[lo:hi], [t[lo:hi] for t in small],
+                                       scale_mode=fa.SCALE_MUL, scale=0.25, stream=producers[i % 2]))
+        # a gradient's buckets, in place into contribution 0, from the other busy producer,
+        # queued behind a held command thread
+        _hold(producers[1], ballast, times=5)
+        held = HeldCommandThread(dev)
+        n = grad[0].numel()
+        spans = [(n - 777, n)] + [(n - 777 - (i + 1) * bucket, n - 777 - i * bucket) for i in range(count)]
+        for lo, hi in spans:
+            works.append(dev.allreduce(grad[0][lo:hi], [t[lo:hi] for t in grad],
+                                       scale_mode=fa.SCALE_MUL, scale=0.25, stream=producers[1]))
+        held.release()
+        # a whole gradient into a separate output
+        works.append(dev.allreduce(whole_out, whole, scale_mode=fa.SCALE_DIV, scale=4.0,
+                                   stream=producers[0]))
+        # a bucket whose own contribution is read from three tensors of its own
+        works.append(dev.allreduce_gathered(gathered_out, [t[:3_000_000] for t in whole], 2, pieces,
+                                            scale_mode=fa.SCALE_MUL, scale=0.25, stream=producers[0]))
+        for w in works:
+            w.wait()
+        dev.synchronize()
+        torch.cuda.synchronize()
+        assert_bits_equal(small_out.cpu().numpy(), oracle.sum_f32(host["small"], oracle.SCALE_MUL, 0.25), "small")
+        assert_bits_equal(grad[0].cpu().numpy(), oracle.sum_f32(host["grad"], oracle.SCALE_MUL, 0.25, threads=16), "buckets")
+        assert_bits_equal(whole_out.cpu().numpy(), oracle.sum_f32(host["whole"], oracle.SCALE_DIV, 4.0, threads=16), "whole")
+        assert_bits_equal(gathered_out.cpu().numpy(),
+                          oracle.sum_f32([h[:3_000_000] for h in host["whole"]], oracle.SCALE_MUL, 0.25, threads=16),
+                          "gathered")
+    finally:
+        dev.close()
+
+
+def test_results_do_not_depend_on_the_tile_runs():
+    # The blocks of one XCD take runs of 2^r consecutive tiles per round (r = 6 by default):
+    # a permutation of which block reduces which tile, nothing else. Sizes around the groups
+    # of 512 tiles the permutation works in, off-boundary starts, fp32 and bf16.
+    _print_case("tile runs")
+    from fairring_amd import _capi
+    rng = np.random.default_rng(66)
+    k = 8
+    try:
+        for n, skew in ((2 * 1024 * 1024 + 5, 0), (3 * 1024 * 1024 + 77, 3), (25 * MiB // 4, 0), (8 * MiB // 4 * 3, 1)):
+            x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+            want = oracle.sum_f32(list(x), oracle.SCALE_MUL, 0.125, threads=16)
+            bits = oracle.np_f32_to_bf16_rne(x)
+            wantb = oracle.sum_bf16(list(bits), oracle.SCALE_MUL, 0.125, threads=16)
+            for runs in (6, 0, 3, 9):
+                _capi.check(_capi.lib().frg_set_tile_runs(runs))
+                xs = [torch.empty(n + 8, device=DEV)[skew:skew + n].copy_(torch.from_numpy(r)) for r in x]
+                out = torch.empty(n + 8, device=DEV)[skew:skew + n]
+                fa.reduce_slice(out, xs, scale_mode=fa.SCALE_MUL, scale=0.125)
+                torch.cuda.synchronize()
+                assert_bits_equal(out.cpu().numpy(), want, "fp32 n=%d runs=%d" % (n, runs))
+                xb = to_gpu_bf16(bits)
+                ob = torch.empty_like(xb[0])
+                fa.reduce_slice(ob, xb, scale_mode=fa.SCALE_MUL, scale=0.125)
+                torch.cuda.synchronize()
+                assert_bits_equal(bf16_bits(ob), wantb, "bf16 n=%d runs=%d" % (n, runs))
+    finally:
+        _capi.lib().frg_set_tile_runs(6)
