@@ -21,6 +21,13 @@ Other workloads (the remaining configurations of the benchmark definition, for t
         _fairring.ProcessGroup.allreduce per bucket (group of 8, 7 simulated
         peers resident on the GPU, in place, completion through the future,
         every work waited for at the end of the step)
+  c5sep the bucket stream as DistributedDataParallel lays it out: 48 buckets of
+        25 MiB, every bucket and every peer's copy of it an allocation of its
+        own, one _fairring.ProcessGroup.allreduce per bucket
+  gather the c5 bucket stream with the bucket's own contribution still in six
+        gradient tensors of its own (ProcessGroup._allreduce_from_grads'
+        path): the copy into the bucket is part of the reduction; the record
+        also holds the rate of copy-then-allreduce on the same data
   copy  K = 1 (a plain copy of known size), the calibration for HBM counters
   hook  torch's bf16 compression hook folded into the reduction: own fp32
         gradient compressed in registers + 7 peers' bf16 tensors, result
@@ -31,6 +38,12 @@ kernel (algorithmic bytes per launch / average launch duration from HIP events
 on the kernel's own stream) and a CPU baseline timed on this host's cores. The
 default run (c2) then measures the other workloads as well, briefly, and adds
 them to the same line under "configs" (--no-extra-configs leaves them out).
+
+The default warm-up is 120 steps (0.9 s of sustained load), the default timed
+region 100 steps: under sustained load the device's rate steps up by about 2 %
+some 0.6 to 0.7 s in (6,565 -> 6,712 GB/s in one process, measured in chunks
+of 40 steps), and a timed region that starts earlier straddles that step and
+reports something between the two.
 """
 import argparse
 import json
@@ -49,8 +62,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=120)
     ap.add_argument("--workload", default="c2",
                     choices=["c2", "c3", "c4", "c5", "c5pg", "c5sep", "gather", "copy", "hook",
                              "smallops"])
@@ -1045,7 +1058,10 @@ def main():
         for name in ("c5", "c5pg", "gather", "c5sep", "c4", "hook", "c3"):
             sub = argparse.Namespace(**vars(args))
             sub.workload, sub.no_cpu_baseline = name, True
-            sub.steps, sub.warmup = min(args.steps, 3 if name == "c3" else 10), 3
+            # (the device has been under load for seconds by now; c3 moves 1.7 GB
+            # over the host link per step, the others 11 to 49 GB within HBM)
+            sub.steps = min(args.steps, 3 if name == "c3" else 30)
+            sub.warmup = min(args.warmup, 2 if name == "c3" else 20)
             if name in ("c5sep", "c4"):
                 shared = None
                 keep.clear()       # the fp32 inputs go before other ones are made
@@ -1110,12 +1126,15 @@ def measure(args, workload, np, torch, fa, oracle, keep=None, shared=None):
         tpath = os.path.join(ROOT, "profiles", traffic_file)
         if os.path.exists(tpath):
             import re
-            m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", open(tpath).read())
+            text = open(tpath).read()
+            m = re.search(r"traffic = [\d,]+ KiB = ([\d,]+) B per launch", text)
+            at = re.search(r"[Mm]easured at commit ([0-9a-f]{7,40})", text)
             if m:
                 roof["traffic"] = int(m.group(1).replace(",", ""))
                 roof["traffic_source"] = ("profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
-                                          "of an earlier run of this command; not measured in "
-                                          "this run)" % traffic_file)
+                                          "of an earlier run of this command%s; not measured in "
+                                          "this run)" % (traffic_file,
+                                                         ", at commit %s" % at.group(1) if at else ""))
 
     metric = {
         "c2": "reduce GB/s (bytes read+written), 8-way fp32, 25 MiB slices",

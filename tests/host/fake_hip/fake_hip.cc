@@ -454,8 +454,9 @@ static std::map<uintptr_t, size_t> gAllocs;  // what hipMalloc handed out
 
 hipError_t hipMalloc(void** ptr, size_t size) {
   if (enter("hipMalloc")) return ret(hipErrorOutOfMemory);
-  *ptr = std::malloc(size ? size : 1);
-  if (*ptr == nullptr) return ret(hipErrorOutOfMemory);
+  // device allocations start on a page boundary
+  *ptr = nullptr;
+  if (posix_memalign(ptr, 4096, size ? size : 1) != 0) return ret(hipErrorOutOfMemory);
   std::lock_guard<std::mutex> g(gAllocMu);
   gAllocs[reinterpret_cast<uintptr_t>(*ptr)] = size ? size : 1;
   return hipSuccess;
