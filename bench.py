@@ -29,6 +29,8 @@ Other workloads (the remaining configurations of the benchmark definition, for t
         path): the copy into the bucket is part of the reduction; the record
         also holds the rate of copy-then-allreduce on the same data
   copy  K = 1 (a plain copy of known size), the calibration for HBM counters
+  placement  the c2 reduction on 400 M elements at six placements of its buffers
+        in one process (diagnostic, prints its own line)
   hook  torch's bf16 compression hook folded into the reduction: own fp32
         gradient compressed in registers + 7 peers' bf16 tensors, result
         decompressed in place (22 algorithmic bytes per element)
@@ -66,7 +68,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=120)
     ap.add_argument("--workload", default="c2",
                     choices=["c2", "c3", "c4", "c5", "c5pg", "c5sep", "gather", "copy", "hook",
-                             "smallops"])
+                             "smallops", "placement"])
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="default workload only: do not measure the other workloads afterwards")
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
@@ -909,6 +911,49 @@ def run_hook(args, np, torch, fa, oracle):
     return value, elapsed, cfg, roof, checked, None, "bf16"
 
 
+def run_placement(args, torch, fa):
+    """The 8-way fp32 reduction of a 400 M-element gradient at several placements of its nine
+    buffers in one process: before each placement something else takes memory first, of
+    another size each time, so the buffers land elsewhere in HBM. Prints its own JSON line
+    with the rate at each placement (host clock over `--steps` passes after one warm-up
+    pass). Under `rocprofv3 --pmc` (dispatches serialised) the per-dispatch counter records
+    of each placement are what shows whether placements differ in how they load the memory
+    channels."""
+    import time
+    k, n = args.k or 8, args.numel or 400_000_000
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=args.slice_bytes,
+                            max_memory_allocated_in_bytes=args.total_memory)
+    g = torch.Generator(device="cuda:0")
+    spacers, report = [], []
+    for r in range(6):
+        g.manual_seed(100 + r)
+        spacers.append(torch.empty((r * 777 + 300) << 20, dtype=torch.uint8, device="cuda:0"))
+        xs = [torch.empty(n, device="cuda:0").normal_(0, 0.01, generator=g) for _ in range(k)]
+        out = torch.empty(n, device="cuda:0")
+        torch.cuda.synchronize()
+        dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k).wait()
+        dev.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        w = None
+        for _ in range(args.steps):
+            w = dev.allreduce(out, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+        w.wait()
+        dev.synchronize()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        report.append({"out": "%#x" % out.data_ptr(), "first_contribution": "%#x" % xs[0].data_ptr(),
+                       "GBps": round((k + 1) * 4 * n * args.steps / dt / 1e9, 1)})
+        del xs, out
+        torch.cuda.empty_cache()
+    dev.close()
+    rates = sorted(p["GBps"] for p in report)
+    print(json.dumps({"metric": "reduce GB/s (bytes read+written), 8-way fp32, by placement of the "
+                                "buffers", "unit": "GB/s", "value": rates[len(rates) // 2],
+                      "min": rates[0], "max": rates[-1], "n_gpus": 1, "steps": args.steps,
+                      "k": k, "numel": n, "placements": report}))
+
+
 def run_small_ops(args, torch, fa):
     """Per-operation cost at bucket sizes where the kernel is short (a DDP step's
     first 1 MiB bucket and its small ones): what the caller's thread pays per
@@ -1044,6 +1089,9 @@ def main():
 
     if args.workload == "smallops":
         run_small_ops(args, torch, fa)
+        return
+    if args.workload == "placement":
+        run_placement(args, torch, fa)
         return
 
     keep = []
