@@ -92,3 +92,92 @@ def test_static_scratch_rejects_what_it_cannot_hold():
     with pytest.raises(fa.FairringError) as e:
         fa.reduce_slice_static(out[:16], [x[:16]] * 4097)
     assert e.value.code == _capi.ERR_INVALID and "4096" in str(e.value)
+
+
+@pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+def test_static_scratch_chain_off_16_byte_boundaries(dtype, kind):
+    # The output and the contributions 2, 6 and 10 bytes past a 16-byte boundary (the vector
+    # variant with a scalar head, the fp32 accumulators in the scratch moved along with them),
+    # and the output at another offset than the contributions (the scalar variant): the bits of
+    # the pipeline's chain, and of the oracle's single fold with one rounding at the end.
+    print("[case] no-alloc entry point, offsets of 2 / 6 / 10 bytes,", kind, flush=True)
+    k, n = 70, 200_003
+    g = torch.Generator(device=DEV)
+    g.manual_seed(73)
+    base = [torch.empty(n + 16, device=DEV).normal_(0, 0.05, generator=g).to(dtype) for _ in range(k)]
+    dev = fa.DeviceFairring(0)
+    try:
+        for off, out_off in ((1, 1), (3, 3), (5, 5), (3, 0), (0, 5)):
+            xs = [b[off:off + n] for b in base]
+            want = torch.empty(n, dtype=dtype, device=DEV)
+            dev.allreduce(want, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k).wait()
+            room = torch.full((n + 16,), 3.0, dtype=dtype, device=DEV)
+            got = room[out_off:out_off + n]
+            fa.reduce_slice_static(got, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+            torch.cuda.synchronize()
+            assert_bits_equal(bits16(got), bits16(want), "offsets %d / %d" % (off, out_off))
+            assert_bits_equal(bits16(got), oracle.reduce(kind, [bits16(x) for x in xs], "sum",
+                                                         oracle.SCALE_MUL, 1.0 / k),
+                              "oracle, offsets %d / %d" % (off, out_off))
+            # nothing outside the output was written
+            assert bool((room[:out_off] == 3.0).all()) and bool((room[out_off + n:] == 3.0).all())
+    finally:
+        dev.close()
+
+
+def test_static_scratch_max_in_place_into_a_late_contribution():
+    # MAX carries its exact partial result; reduced in place into contribution 80, which only
+    # the second launch of the chain reads, it must not land there before that launch has run.
+    print("[case] no-alloc entry point, MAX in place at rank 80 (fp32 and int32)", flush=True)
+    k, n = 100, 150_001
+    g = torch.Generator(device=DEV)
+    g.manual_seed(74)
+    for dtype in (torch.float32, torch.int32):
+        if dtype == torch.int32:
+            xs = [torch.randint(-2**30, 2**30, (n,), device=DEV, dtype=dtype, generator=g)
+                  for _ in range(k)]
+        else:
+            xs = [torch.empty(n, device=DEV).normal_(0, 1.0, generator=g) for _ in range(k)]
+        want = torch.stack(xs).amax(dim=0)
+        host = [x[:50_000].cpu().numpy() for x in xs]
+        fa.reduce_slice_static(xs[80], xs, op=fa.MAX)
+        torch.cuda.synchronize()
+        assert bool(torch.equal(xs[80], want)), str(dtype)
+        assert_bits_equal(xs[80][:50_000].cpu().numpy(),
+                          oracle.reduce("f32" if dtype == torch.float32 else "i32", host, "max"), "oracle")
+
+
+def test_static_scratch_chain_captured_into_a_graph_and_replayed():
+    # What the entry point is for: a stream under capture. The context is created first (it
+    # looks the array up, so the capture meets no set-up); the captured chain is replayed with
+    # other inputs each time, with eager work and synchronisations in between, and every replay
+    # is compared with the eager call on the same inputs.
+    print("[case] no-alloc entry point under graph capture, three replays", flush=True)
+    k, n = 70, 120_001
+    g = torch.Generator(device=DEV)
+    g.manual_seed(75)
+    dev = fa.DeviceFairring(0)
+    try:
+        xs = [torch.empty(n, device=DEV).normal_(0, 0.05, generator=g).to(torch.bfloat16)
+              for _ in range(k)]
+        got = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+        eager = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+        fa.reduce_slice_static(eager, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)   # warm
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fa.reduce_slice_static(got, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+        for replay in range(3):
+            for x in xs[::7]:                  # eager work between the replays
+                x.mul_(1.5 + replay)
+            got.fill_(9.0)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            fa.reduce_slice_static(eager, xs, scale_mode=fa.SCALE_MUL, scale=1.0 / k)
+            torch.cuda.synchronize()
+            assert_bits_equal(bits16(got), bits16(eager), "replay %d" % replay)
+            assert_bits_equal(bits16(got), oracle.sum_bf16([bits16(x) for x in xs], oracle.SCALE_MUL,
+                                                           1.0 / k, threads=8), "oracle, replay %d" % replay)
+    finally:
+        dev.close()
