@@ -41,11 +41,13 @@ on the kernel's own stream) and a CPU baseline timed on this host's cores. The
 default run (c2) then measures the other workloads as well, briefly, and adds
 them to the same line under "configs" (--no-extra-configs leaves them out).
 
-The default warm-up is 120 steps (0.9 s of sustained load), the default timed
-region 100 steps: under sustained load the device's rate steps up by about 2 %
-some 0.6 to 0.7 s in (6,565 -> 6,712 GB/s in one process, measured in chunks
-of 40 steps), and a timed region that starts earlier straddles that step and
-reports something between the two.
+The default warm-up is 120 steps (0.9 s), the default timed region 100 steps.
+A process that starts right after another one has released tens of GB of
+device memory runs about 4 % slower while the device deals with that memory
+(about a second per 40 GiB; 6,608 -> 6,750 GB/s one second into such a
+process), and a short timed region at the very start of the process sits
+inside that window. For the same reason nothing is handed back to the driver
+between the workloads of one run.
 """
 import argparse
 import json
@@ -69,6 +71,8 @@ def parse_args():
     ap.add_argument("--workload", default="c2",
                     choices=["c2", "c3", "c4", "c5", "c5pg", "c5sep", "gather", "copy", "hook",
                              "smallops", "placement"])
+    ap.add_argument("--extras", default="c5,c5pg,gather,c5sep,c4,hook,c3",
+                    help="default workload only: the workloads measured afterwards, in this order")
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="default workload only: do not measure the other workloads afterwards")
     ap.add_argument("--numel", type=int, default=0, help="override the workload's element count")
@@ -657,11 +661,18 @@ def run_c5sep(args, np, torch, fa, oracle):
     buckets = max(1, numel // n)
     g = torch.Generator(device="cuda:0")
     g.manual_seed(515)
+    # (In the default run this workload's tensors come from a memory pool of their own, see
+    # main(): each is a segment from the driver, not a piece cut from a block that an earlier
+    # workload left in torch's cache. Cut from 5 GB blocks the buckets start 25 MiB apart, 0
+    # to 3 MiB past a multiple of a round of their allocation, and the stream runs 1.6 %
+    # slower for it. The record says how many tensors start their allocation.)
     fresh = [torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(buckets)]
     owns = [t.clone() for t in fresh]
     peers = [[torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(k - 1)]
              for _ in range(buckets)]
     torch.cuda.synchronize()
+    starts = {seg["address"] for seg in torch.cuda.memory_snapshot()}
+    own_allocation = sum(t.data_ptr() in starts for row in [owns] + peers for t in row)
     o = _fairring.ProcessGroup.Options(
         max_memory_allocated_in_bytes=args.total_memory, max_padding_allocated_in_bytes=MiB,
         min_parallelism=2, is_high_priority_stream=True,
@@ -722,6 +733,7 @@ def run_c5sep(args, np, torch, fa, oracle):
                     "(configs[4] with DistributedDataParallel's own bucket layout)" % (
                         buckets, args.slice_bytes, k - 1, k),
         "k": k, "numel": n * buckets, "buckets": buckets, "staging_total_bytes": args.total_memory,
+        "tensors_at_the_start_of_their_allocation": "%d of %d" % (own_allocation, buckets * k),
         "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
                    "staging_slots": layout[3]},
     }
@@ -914,7 +926,8 @@ def run_hook(args, np, torch, fa, oracle):
 def run_placement(args, torch, fa):
     """The 8-way fp32 reduction of a 400 M-element gradient at several placements of its nine
     buffers in one process: before each placement something else takes memory first, of
-    another size each time, so the buffers land elsewhere in HBM. Prints its own JSON line
+    another size each time, so the buffers land elsewhere in HBM (everything stays allocated
+    until the end). Prints its own JSON line
     with the rate at each placement (host clock over `--steps` passes after one warm-up
     pass). Under `rocprofv3 --pmc` (dispatches serialised) the per-dispatch counter records
     of each placement are what shows whether placements differ in how they load the memory
@@ -924,7 +937,7 @@ def run_placement(args, torch, fa):
     dev = fa.DeviceFairring(0, slice_size_in_bytes=args.slice_bytes,
                             max_memory_allocated_in_bytes=args.total_memory)
     g = torch.Generator(device="cuda:0")
-    spacers, report = [], []
+    spacers, report, held = [], [], []
     for r in range(6):
         g.manual_seed(100 + r)
         spacers.append(torch.empty((r * 777 + 300) << 20, dtype=torch.uint8, device="cuda:0"))
@@ -944,8 +957,9 @@ def run_placement(args, torch, fa):
         dt = time.perf_counter() - t0
         report.append({"out": "%#x" % out.data_ptr(), "first_contribution": "%#x" % xs[0].data_ptr(),
                        "GBps": round((k + 1) * 4 * n * args.steps / dt / 1e9, 1)})
-        del xs, out
-        torch.cuda.empty_cache()
+        # nothing is freed between placements (14 GB each): memory that has just gone back to
+        # the driver slows down whatever runs next, which is not what is measured here
+        held.append((xs, out))
     dev.close()
     rates = sorted(p["GBps"] for p in report)
     print(json.dumps({"metric": "reduce GB/s (bytes read+written), 8-way fp32, by placement of the "
@@ -1103,19 +1117,35 @@ def main():
         # they are run on their own, fewer steps, no CPU baseline.
         shared = tuple(keep) if keep else None
         extra = {}
-        for name in ("c5", "c5pg", "gather", "c5sep", "c4", "hook", "c3"):
+        pools = []
+        for name in [x for x in args.extras.split(",") if x]:
             sub = argparse.Namespace(**vars(args))
             sub.workload, sub.no_cpu_baseline = name, True
-            # (the device has been under load for seconds by now; c3 moves 1.7 GB
-            # over the host link per step, the others 11 to 49 GB within HBM)
-            sub.steps = min(args.steps, 3 if name == "c3" else 30)
-            sub.warmup = min(args.warmup, 2 if name == "c3" else 20)
+            # (c3 moves 1.7 GB over the host link per step, the others 11 to 49 GB
+            # within HBM)
+            # As many steps and warm-up steps as the headline, up to 50 after 100.
+            sub.steps = min(args.steps, 3 if name == "c3" else 50)
+            sub.warmup = min(args.warmup, 2 if name == "c3" else 100)
+            if name == "c5sep":
+                sub.warmup = min(args.warmup * 4, 400)     # a step of it is 11 GB, not 49
             if name in ("c5sep", "c4"):
                 shared = None
                 keep.clear()       # the fp32 inputs go before other ones are made
+            # (Memory is not handed back to the driver between workloads: what is allocated
+            # right after tens of GB were released is slower for it. The bf16 workload ran at
+            # 6,230 GB/s on such memory against 6,618 on blocks torch had kept and 6,659 in a
+            # fresh process; a staging pool allocated then took host copies at half the link's
+            # rate, 27 against 54 GB/s, until 3 s had passed.)
             try:
-                r = measure(sub, name, np, torch, fa, oracle,
-                            shared=shared if name in ("c5", "c5pg", "gather") else None)
+                if name in ("c5", "c5pg", "gather"):
+                    r = measure(sub, name, np, torch, fa, oracle, shared=shared)
+                else:
+                    # Tensors of its own, from the driver, as in a run of its own: a memory
+                    # pool per workload, kept until the process ends (see above: memory must
+                    # not go back to the driver in between).
+                    pools.append(torch.cuda.MemPool())
+                    with torch.cuda.use_mem_pool(pools[-1]):
+                        r = measure(sub, name, np, torch, fa, oracle)
                 # compact: the whole record stays one line of a few KB
                 roof = {key: r["roofline"][key] for key in (
                     "bound", "achieved", "peak", "nominal", "unit", "frac", "traffic",

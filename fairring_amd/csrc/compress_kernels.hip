@@ -316,7 +316,7 @@ template <typename WV, typename WS, bool OUT32, int KW, int SC>
 __global__ void __launch_bounds__(kBlock)
     compressedKernel(void* out, const float* raw, Ptrs<KW> wire, int Kw, int rawPos, int scaleMode,
                      float scale, int64_t head, int lead, int64_t nvec, int64_t tail,
-                     int64_t roundTiles, int64_t pieces) {
+                     int64_t roundTiles, int64_t pieces, int chunkShift) {
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
   const int64_t grid = gridDim.x;
   // the first `lead` groups are a piece of their own, so that the tiles start
@@ -328,7 +328,15 @@ __global__ void __launch_bounds__(kBlock)
   constexpr bool kStaged = WV::kLanes == 8 && kBlock % 64 == 0;
   __shared__ f32x4 stageAll[kStaged ? (kBlock / 64) * 128 : 1];
   f32x4* stage = stageAll + (kStaged ? (threadIdx.x >> 6) * 128 : 0);
-  for (int64_t t = blockIdx.x; t < roundTiles; t += grid) {
+  for (int64_t t0 = blockIdx.x; t0 < roundTiles; t0 += grid) {
+    // runs of 2^chunkShift consecutive tiles for the blocks of one XCD (the
+    // hardware deals blocks to the 8 XCDs in turn), as in the plain kernel
+    int64_t t = t0;
+    if (chunkShift > 0) {
+      const int64_t low = (int64_t{1} << chunkShift) - 1;
+      t = ((t0 >> (3 + chunkShift)) << (3 + chunkShift)) | ((t0 & 7) << chunkShift) |
+          ((t0 >> 3) & low);
+    }
     const int64_t elemBase = bodyBase + t * kTile * WV::kLanes;
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
@@ -390,16 +398,26 @@ hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptr
     lead = l < nvec ? static_cast<int>(l) : 0;
   }
   const GridPlan plan = planGrid(nvec - lead, a.K, numCus);
+  // Runs per XCD as in the plain kernel, with at least two groups of 8 runs in
+  // flight on the grid (512 blocks here: runs of 32 tiles; runs of 128, one
+  // group wider than the grid, measured 10 % slower than none).
+  int shift = xcdChunkShift();
+  while (shift > 0 && (int64_t{16} << shift) > plan.grid) --shift;
+  const int chunkShift = (shift > 0 && plan.grid % 8 == 0 && plan.roundTiles > 0 &&
+                          plan.roundTiles % (int64_t{8} << shift) == 0)
+                             ? shift
+                             : 0;
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
     hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
                           dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream,
                           a.startEvent, a.stopEvent, 0, a.out, raw, wire, Kw, rawPos, a.scale_mode,
-                          a.scale, head, lead, nvec, tail, plan.roundTiles, plan.pieces);
+                          a.scale, head, lead, nvec, tail, plan.roundTiles, plan.pieces,
+                          chunkShift);
   } else {
     hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
                        dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream, a.out, raw,
                        wire, Kw, rawPos, a.scale_mode, a.scale, head, lead, nvec, tail,
-                       plan.roundTiles, plan.pieces);
+                       plan.roundTiles, plan.pieces, chunkShift);
   }
   return hipGetLastError();
 }

@@ -162,6 +162,7 @@ void setTuning(int blocksPerCu);
 // log2 of the consecutive 4 KiB tiles the blocks of one XCD take in a row (6 by
 // default: 256 KiB; 0: tile = block index). For measurements.
 void setXcdChunkShift(int shift);
+int xcdChunkShift();
 
 // Compute units of a device (cached).
 int computeUnits(int device);

@@ -661,6 +661,7 @@ bool isFloating(int dtype) {
 void setTuning(int blocksPerCu) { gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0; }
 
 void setXcdChunkShift(int shift) { gXcdChunkShift = shift >= 0 && shift <= 12 ? shift : 0; }
+int xcdChunkShift() { return gXcdChunkShift; }
 
 int launchSegmented(const SegmentedArgs& a, hipStream_t stream, std::string* err) {
   auto fail = [&](int code, const std::string& msg) {

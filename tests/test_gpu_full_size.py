@@ -264,7 +264,7 @@ def test_c5_ddp_bucket_stream_inputs_ready(dev):
 
 @pytest.mark.skip(reason="went silent for 180 s on its only GPU run (killed by the harness, GPU "
                          "still answering) while 211 operations were submitted with the producer "
-                         "(default) stream still busy; no cause found by reading the code, so the "
+                         "(default) stream still busy; no cause found by reading the code or on the CPU stand-in (either event semantics), so the "
                          "case stays off the GPU. The same bucket schedule with an idle producer "
                          "stream runs in bench.py --workload c5, parity-checked.")
 def test_c5_ddp_bucket_stream(dev):

@@ -148,6 +148,27 @@ def _compressed_case(wire, tdt, k, n, raw, rng, shift=0, in_place=True, out_f32=
 
 
 @pytest.mark.parametrize("wire,tdt", WIRES)
+def test_compressed_results_do_not_depend_on_the_tile_runs(wire, tdt):
+    # Whole rounds of the 512-block grid (2,048 elements per tile): the blocks of one XCD take
+    # runs of consecutive tiles, a permutation of which block reduces which tile and nothing
+    # else. Two and three rounds plus a ragged rest, an off-boundary start, the hook's own
+    # shape (K = 8, fp32 bucket in place) and the general body (K = 5, wire output).
+    _print_case("compressed, tile runs", wire)
+    from fairring_amd import _capi
+    rng = np.random.default_rng(8100)
+    try:
+        for runs in (6, 0, 3, 5):
+            _capi.check(_capi.lib().frg_set_tile_runs(runs))
+            for n, shift in ((2 * 512 * 2048 + 77, 0), (3 * 512 * 2048 + 4099, 8)):
+                got, want = _compressed_case(wire, tdt, 8, n, 3, rng, shift=shift, mode="mul")
+                assert_bits_equal(got, want, "%s K 8 n %d runs %d" % (wire, n, runs))
+            got, want = _compressed_case(wire, tdt, 5, 2 * 512 * 2048 + 9, 1, rng, out_f32=False)
+            assert_bits_equal(got, want, "%s K 5 wire output, runs %d" % (wire, runs))
+    finally:
+        _capi.lib().frg_set_tile_runs(6)
+
+
+@pytest.mark.parametrize("wire,tdt", WIRES)
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 8, 9, 17, 64])
 @pytest.mark.parametrize("n", [1, 7, 8, 9, 2051, 262147])
 def test_compressed_sizes(wire, tdt, k, n):

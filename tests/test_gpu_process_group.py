@@ -206,7 +206,7 @@ def test_pinned_peers_are_switched_off_by_default():
 
 @pytest.mark.skip(reason="went silent for 180 s on one GPU run (killed by the harness, GPU still "
                          "answering) after passing on every earlier run; no cause found by reading "
-                         "the code, so the case stays off the GPU and the process group refuses "
+                         "the code or on the CPU stand-in, so the case stays off the GPU and the process group refuses "
                          "pinned peers unless FAIRRING_PINNED_PEERS is set. The same staging "
                          "through the C ABI runs in test_gpu_parity.py and "
                          "test_gpu_random_matrix.py.")
