@@ -24,10 +24,11 @@ Other workloads (the remaining configurations of the benchmark definition, for t
   c5sep the bucket stream as DistributedDataParallel lays it out: 48 buckets of
         25 MiB, every bucket and every peer's copy of it an allocation of its
         own, one _fairring.ProcessGroup.allreduce per bucket
-  gather the c5 bucket stream with the bucket's own contribution still in six
-        gradient tensors of its own (ProcessGroup._allreduce_from_grads'
-        path): the copy into the bucket is part of the reduction; the record
-        also holds the rate of copy-then-allreduce on the same data
+  gather the c5sep layout with the bucket's own contribution still in six
+        gradient tensors of its own per bucket, through
+        ProcessGroup._allreduce_from_grads: the copy into the bucket is part of
+        the reduction; the record also holds the rate of copy-then-allreduce
+        on the same data
   copy  K = 1 (a plain copy of known size), the calibration for HBM counters
   placement  the c2 reduction on 400 M elements at six placements of its buffers
         in one process (diagnostic, prints its own line)
@@ -71,7 +72,7 @@ def parse_args():
     ap.add_argument("--workload", default="c2",
                     choices=["c2", "c3", "c4", "c5", "c5pg", "c5sep", "gather", "copy", "hook",
                              "smallops", "placement"])
-    ap.add_argument("--extras", default="c5,c5pg,gather,c5sep,c4,hook,c3",
+    ap.add_argument("--extras", default="c5,c5pg,c4,c5sep,gather,hook,c3",
                     help="default workload only: the workloads measured afterwards, in this order")
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="default workload only: do not measure the other workloads afterwards")
@@ -745,115 +746,127 @@ GATHER_SEGMENTS = [4194304, 2048, 2048, 2097152, 2048, 256000]
 
 
 def run_gather(args, np, torch, fa, oracle, shared=None):
-    """The bucket stream with this rank's contribution read from the gradient tensors
-    themselves (frg_allreduce_gathered): per 25 MiB bucket six tensors of their own, the
-    bucket written once; beside it the same stream the way DistributedDataParallel does it by
-    default, every gradient copied into its bucket first and the bucket reduced in place."""
-    k, numel = args.k or 8, args.numel or 1_370_000_000
-    slice_elems = args.slice_bytes // 4
-    spans = ddp_buckets(numel, slice_elems, MiB // 4)
-    dev = fa.DeviceFairring(0, max_memory_allocated_in_bytes=args.total_memory,
-                            slice_size_in_bytes=args.slice_bytes,
-                            num_reduce_streams=args.streams, max_launch_bytes=args.launch_bytes)
-    if shared is not None:
-        xs, out = shared
-    else:
-        xs = synth(torch, numel, k, "f32", 20240)
-        out = torch.empty(numel, dtype=torch.float32, device="cuda:0")
+    """The bucket stream of DistributedDataParallel with gradient_as_bucket_view=False (its
+    default): every bucket an allocation of its own (48 of 25 MiB, as in c5sep), this rank's
+    contribution still in the gradient tensors autograd left it in (six per bucket, tensors of
+    their own), one `_fairring.ProcessGroup._allreduce_from_grads` per bucket, which reads the
+    gradients themselves and writes the bucket once. Beside it the same stream the way the
+    reducer does it: every gradient copied into its bucket first (one copy kernel per tensor),
+    then `allreduce` on the bucket in place."""
+    import datetime
+
+    import torch.distributed as dist
+
+    import fairring  # noqa: F401  (registers the backend, loads the extension)
+    from fairring_amd import _fairring
+
+    k = args.k or 8
+    n = args.slice_bytes // 4
+    buckets = max(1, (args.numel or 48 * n) // n)
+    seg_lens = [ln for ln in GATHER_SEGMENTS]
+    if sum(seg_lens) != n:                      # another slice size: one tensor takes the rest
+        seg_lens = [min(ln, n) for ln in GATHER_SEGMENTS[:1]] + [max(0, n - min(GATHER_SEGMENTS[0], n))]
+        seg_lens = [ln for ln in seg_lens if ln > 0]
+    g = torch.Generator(device="cuda:0")
+    g.manual_seed(616)
+
+    def fresh(numel):
+        return torch.empty(numel, device="cuda:0").normal_(0.0, 0.01, generator=g)
+
+    grads = [[fresh(ln) for ln in seg_lens] for _ in range(buckets)]
+    bucket_of = [torch.empty(n, device="cuda:0") for _ in range(buckets)]
+    peers = [[fresh(n) for _ in range(k - 1)] for _ in range(buckets)]
     torch.cuda.synchronize()
-    # this rank's gradients: tensors of their own holding what xs[0] holds
-    grads = []
-    for lo, hi in spans:
-        segs, at = [], lo
-        for ln in GATHER_SEGMENTS:
-            ln = min(ln, hi - at)
-            if ln > 0:
-                segs.append(xs[0][at:at + ln].clone())
-                at += ln
-        if at < hi:
-            segs.append(xs[0][at:hi].clone())
-        grads.append(segs)
-    torch.cuda.synchronize()
-    views = [(out[lo:hi], [x[lo:hi] for x in xs]) for lo, hi in spans]
-    prepared = {}
+    o = _fairring.ProcessGroup.Options(
+        max_memory_allocated_in_bytes=args.total_memory, max_padding_allocated_in_bytes=MiB,
+        min_parallelism=2, is_high_priority_stream=True,
+        timeout=datetime.timedelta(seconds=60), slice_size_in_bytes=args.slice_bytes)
+    pg = _fairring.ProcessGroup(dist.HashStore(), 0, k, o)
+    pg._set_fused_divide(True)
 
-    class Last:
-        def __init__(self, works):
-            self.works = works
-
-        def wait(self):
-            for w in self.works:
-                w.wait()
-
-    def step(d):
-        if id(d) not in prepared:
-            prepared[id(d)] = [d.prepare(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k,
-                                         gathered=(0, segs))
-                               for (o, cs), segs in zip(views, grads)]
-        return Last([submit() for submit in prepared[id(d)]])
-
-    elapsed, recs = timed(torch, dev, args.steps, args.warmup, step)
-    step_bytes = (k + 1) * numel * 4
-    value = step_bytes * args.steps / elapsed / 1e9
-    roof = roofline_from_records(recs, (k + 1) * 4,
-                                 launch_elems(args, slice_elems, slice_elems, 4, k), SPAN_HOW)
-    roof["kernel"] = "ksumSegmentedKernel<F32Vec, K=%d, x1/%d>" % (k, k)
-    segmented = dev.progress()["segmented_launches"]
-    step(dev).wait()
-    checked = check_parity(oracle, np, torch, xs, out, numel, slice_elems, k, "f32", True)
-    # the default way: copy every gradient to its place in the bucket (one copy kernel per
-    # tensor, as the reducer issues them), then reduce the bucket in place
-    bucket = torch.empty(numel, dtype=torch.float32, device="cuda:0")
-    bviews = [(bucket[lo:hi], [bucket[lo:hi]] + [x[lo:hi] for x in xs[1:]]) for lo, hi in spans]
-    targets = []
-    for (lo, hi), segs in zip(spans, grads):
-        at, row = lo, []
-        for sg in segs:
-            row.append(bucket[at:at + sg.numel()])
-            at += sg.numel()
-        targets.append(row)
-    plain = [dev.prepare(o, cs, scale_mode=fa.SCALE_MUL, scale=1.0 / k) for o, cs in bviews]
+    def step():
+        works = []
+        for b, gr, pv in zip(bucket_of, grads, peers):
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg._allreduce_from_grads(b, gr))
+        return works
 
     def two_pass():
         works = []
-        for submit, row, segs in zip(plain, targets, grads):
-            for dst, src in zip(row, segs):
-                dst.copy_(src)
-            works.append(submit())
-        return Last(works)
+        for b, gr, pv in zip(bucket_of, grads, peers):
+            at = 0
+            for t in gr:
+                b[at:at + t.numel()].copy_(t)
+                at += t.numel()
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg.allreduce([b]))
+        return works
 
-    two_pass().wait()
-    dev.synchronize()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    w = None
-    for _ in range(args.steps):
-        w = two_pass()
-    w.wait()
-    dev.synchronize()
-    torch.cuda.synchronize()
-    two = step_bytes * args.steps / (time.perf_counter() - t0) / 1e9
-    same = torch.equal(bucket.view(torch.int32), out.view(torch.int32))
-    if not same:
-        raise SystemExit("parity FAILED: gathered differs from copy + allreduce")
-    layout = dev.layout
-    dev.close()
+    def finish(works):
+        for w in works:
+            w.wait()
+
+    def run(fn, steps, marks):
+        for _ in range(max(args.warmup, 1)):
+            finish(fn())
+        pg._synchronize()
+        torch.cuda.synchronize()
+        pg._launch_records()
+        t0 = time.perf_counter()
+        if marks:
+            pg._profile_mark()
+        pending = [fn() for _ in range(steps)]
+        if marks:
+            pg._profile_mark()
+        for works in pending:
+            finish(works)
+        pg._synchronize()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    steps = args.steps * 4          # a step is 11 GB: a few more of them for a steady figure
+    step_bytes = (k + 1) * n * buckets * 4
+    elapsed = run(step, steps, True)
+    recs = pg._launch_records()
+    value = step_bytes * steps / elapsed / 1e9
+    roof = roofline_from_records(recs, (k + 1) * 4, launch_elems(args, n, n, 4, k), SPAN_HOW)
+    roof["kernel"] = ("ksumKernel<F32Vec, SUM, K=%d> for launches within one gradient, "
+                      "ksumSegmentedKernel<F32Vec, K=%d, x1/%d> for those that hold several" % (k, k, k))
+    # parity of three buckets against the oracle, and of every bucket against copy + allreduce
+    got = [b.clone() for b in bucket_of]
+    checked = []
+    for i in sorted({0, buckets // 2, buckets - 1}):
+        own = torch.cat(grads[i]).cpu().numpy()
+        host = [own] + [p.cpu().numpy() for p in peers[i]]
+        want = oracle.sum_f32(host, oracle.SCALE_MUL, 1.0 / k, threads=os.cpu_count() or 1)
+        if not (got[i].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all():
+            raise SystemExit("parity FAILED on bucket %d (gather)" % i)
+        checked.append(i)
+    two = step_bytes * steps / run(two_pass, steps, False) / 1e9
+    for i, (a, b) in enumerate(zip(got, bucket_of)):
+        if not torch.equal(a.view(torch.int32), b.view(torch.int32)):
+            raise SystemExit("parity FAILED: gathered differs from copy + allreduce (bucket %d)" % i)
+    layout = pg._layout()
+    del pg
     cfg = {
-        "workload": "DDP bucket stream with this rank's contribution read from its gradient "
-                    "tensors: %d fp32 elements as %d buckets of %d B, %d tensors of their own per "
-                    "bucket (%s elements), K=%d, fused x1/%d; the copy of every gradient into its "
-                    "bucket (8 bytes per element) is not made" % (
-                        numel, len(spans), args.slice_bytes, len(GATHER_SEGMENTS),
-                        "/".join(str(v) for v in GATHER_SEGMENTS), k, k),
-        "k": k, "numel": numel, "buckets": len(spans), "tensors": sum(len(sg) for sg in grads),
-        "segmented_launches": segmented,
+        "workload": "DDP-shaped bucket stream with this rank's contribution read from its gradient "
+                    "tensors: %d buckets of %d B, each bucket, each of its %d peer copies and each "
+                    "of its %d gradient tensors (%s elements) an allocation of its own, one "
+                    "_fairring.ProcessGroup._allreduce_from_grads per bucket, fused x1/%d; the copy "
+                    "of every gradient into its bucket (8 bytes per element) is not made" % (
+                        buckets, n * 4, k - 1, len(seg_lens), "/".join(str(v) for v in seg_lens),
+                        k),
+        "k": k, "numel": n * buckets, "buckets": buckets, "tensors": buckets * len(seg_lens),
         "copy_then_allreduce_GBps": round(two, 1),
         "copy_then_allreduce_note": "same algorithmic bytes over the time of copying every "
-                                    "gradient into its bucket and reducing the bucket in place; "
-                                    "results equal bit for bit",
-        "layout": layout,
+                                    "gradient into its bucket (torch's copy kernels) and "
+                                    "ProcessGroup.allreduce on the bucket in place; results equal "
+                                    "bit for bit",
+        "staging_total_bytes": args.total_memory,
+        "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
+                   "staging_slots": layout[3]},
     }
-    return value, elapsed, cfg, roof, checked, None, "f32"
+    return value, elapsed / 4, cfg, roof, checked, None, "f32"
 
 
 def run_hook(args, np, torch, fa, oracle):
@@ -1126,9 +1139,9 @@ def main():
             # As many steps and warm-up steps as the headline, up to 50 after 100.
             sub.steps = min(args.steps, 3 if name == "c3" else 50)
             sub.warmup = min(args.warmup, 2 if name == "c3" else 100)
-            if name == "c5sep":
-                sub.warmup = min(args.warmup * 4, 400)     # a step of it is 11 GB, not 49
-            if name in ("c5sep", "c4"):
+            if name in ("c5sep", "gather"):
+                sub.warmup = min(args.warmup * 4, 400)     # a step of them is 11 GB, not 49
+            if name in ("gather", "c5sep", "c4"):
                 shared = None
                 keep.clear()       # the fp32 inputs go before other ones are made
             # (Memory is not handed back to the driver between workloads: what is allocated
@@ -1137,7 +1150,7 @@ def main():
             # fresh process; a staging pool allocated then took host copies at half the link's
             # rate, 27 against 54 GB/s, until 3 s had passed.)
             try:
-                if name in ("c5", "c5pg", "gather"):
+                if name in ("c5", "c5pg"):
                     r = measure(sub, name, np, torch, fa, oracle, shared=shared)
                 else:
                     # Tensors of its own, from the driver, as in a run of its own: a memory

@@ -1547,6 +1547,26 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
       waited[si] = 1;
     }
     lastIdx = si;
+    if (u.segmented && u.pieces.size() == 1) {
+      // A launch that holds one piece (a weight matrix fills whole launches on
+      // its own) is the plain kernel's: its pointers sit in registers from the
+      // start, where the segmented kernel first reads the table's prefix sums
+      // and then the piece's row (two dependent loads ahead of every block's
+      // first tile; 8 MiB launches of one piece: 3 % slower through the table).
+      const SegPiece& one = u.pieces[0];
+      ReduceArgs a;
+      a.out = one.out;
+      a.contribs = one.contribs;
+      a.K = total;
+      a.n = one.n;
+      a.dtype = req.dtype;
+      a.op = req.op;
+      a.scale_mode = req.scaleMode;
+      a.scale = req.scale;
+      a.blocks_per_cu = 4;
+      launch(a, s);
+      continue;
+    }
     if (u.segmented) {
       SegmentedArgs a;
       a.pieces = u.pieces.data();
