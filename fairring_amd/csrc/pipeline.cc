@@ -1625,14 +1625,16 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
 // Contribution 0 lands directly in `out`; the later ones are copied into
 // staging slots and folded into `out` in index order.
 //
-// The pool's slots are dealt in groups of `batch` (half the pool from four slots
-// on, else one slot), and every group belongs to one of the staging streams:
-// that stream copies a batch of contributions into the group's slots and then
-// runs the fold that reads them, so a slot is never overwritten before its last
-// reader has finished (the slot rule of device.cc:543-545,587-589) by stream
-// order alone. What crosses streams is the order of the folds: each one waits
-// for an event recorded behind the fold before it, when that ran on another
-// stream. While one stream folds, the other's copies keep the host link busy.
+// The pool's slots are split evenly among the staging streams (one by default,
+// which then owns the whole pool), and a stream works through its share batch
+// by batch: it copies a batch of contributions into its slots and then runs the
+// fold that reads them, so a slot is never overwritten before its last reader
+// has finished (the slot rule of device.cc:543-545,587-589) by stream order
+// alone. What crosses streams, when there are several, is the order of the
+// folds: each one waits for an event recorded behind the fold before it, when
+// that ran on another stream. (Two streams, each copying under the other's
+// fold, measured no faster than one: 53.9 against 54.3 GB/s. Two concurrent
+// host copies share the link and end together.)
 //
 // (The folds used to run on a reduce stream, with a "filled" event from the copy
 // stream to it and a "free" event back per slot. On MI355X / ROCm 7.2
@@ -1640,7 +1642,8 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
 // to 11 ms, whenever the copy stream's last packet was such a wait, so the
 // command thread paced the copies one at a time: 64 contributions of 25 MiB
 // crossed the link at 46 to 50 GB/s. In this form the same call returns in 1.5
-// us and the link runs at what bare copies get, 56 GB/s on the same box.)
+// us and the link runs at 54 of the 56 GB/s that bare copies get on the same
+// box.)
 std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t initialEvent) {
   const int64_t elsize = elementSize(req.dtype);
   // A staged slice must fit a slot as well as the slice size.
