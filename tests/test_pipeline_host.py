@@ -63,6 +63,10 @@ def test_pipeline_host_scenarios(variant, waits, tmp_path_factory):
                # ordered after them), so leak checking is off
                ASAN_OPTIONS="detect_leaks=0 abort_on_error=1",
                UBSAN_OPTIONS="print_stacktrace=1")
+    # ThreadSanitizer slows the scenarios tenfold; it runs them in the topology of a GPU
+    # process (4 shared hardware queues) only: what it looks for does not depend on that
+    if variant == "tsan":
+        env["HOST_TEST_TOPOLOGY"] = "4"
     mode = [waits] if waits == "latest-record-waits" else []
     run = subprocess.run([exe] + mode, capture_output=True, text=True, timeout=380, env=env)
     assert run.returncode == 0, (run.stdout[-2000:], run.stderr[-4000:])
