@@ -32,6 +32,8 @@ def test_defaults_are_the_headline_configuration():
         sys.argv = old
     assert (a.gpus, a.workload, a.slice_bytes, a.total_memory) == (1, "c2", 25 * MiB, 50 * MiB)
     assert a.steps >= 1 and a.warmup >= 1
+    # the driver's record carries every other workload of the benchmark definition too
+    assert sorted(a.extras.split(",")) == sorted(["c5", "c5pg", "c5sep", "gather", "c4", "hook", "c3"])
 
 
 @pytest.mark.parametrize("op_elems,slice_elems,elsize,lb,want", [
