@@ -484,12 +484,15 @@ FRG_API int frg_launch_records(frg_ctx* ctx, frg_launch_record* records, int cap
  * CU (0 keeps the built-in default, which depends on the loads per lane). */
 FRG_API int frg_set_tuning(int blocks_per_cu);
 
-/* Launch-shape knob of the reduction kernel: log2 of the number of consecutive
+/* Launch-shape knob of the reduction kernels: log2 of the number of consecutive
  * 4 KiB tiles that the blocks running on one XCD take in a row within a round
  * of the grid (the hardware deals the blocks of a launch to the 8 XCDs in
- * turn). 6, the default, gives every XCD runs of 256 KiB; 0 gives every block
- * the tile of its own index, so that an XCD reads every eighth tile. Results do
- * not depend on it. For measurements. */
+ * turn). 6, the default, gives every XCD runs of 256 KiB in sums of 8 or more
+ * contributions (fewer contributions keep the plain order) and runs of 128 KiB
+ * of wire in the compressed reduction (whose grid is half as large: a run is
+ * at most a sixteenth of the grid); 0 gives every block the tile of its own
+ * index, so that an XCD reads every eighth tile. Results do not depend on it.
+ * For measurements. */
 FRG_API int frg_set_tile_runs(int log2_tiles);
 
 /* Message of the last failure on the calling thread (or of the failed work). */
