@@ -846,6 +846,45 @@ def run_gather(args, np, torch, fa, oracle, shared=None):
     for i, (a, b) in enumerate(zip(got, bucket_of)):
         if not torch.equal(a.view(torch.int32), b.view(torch.int32)):
             raise SystemExit("parity FAILED: gathered differs from copy + allreduce (bucket %d)" % i)
+    # The same buckets under torch's bf16 compression hook: 7 peers' bf16 tensors per bucket,
+    # the own fp32 contribution read from the gradients (frg_allreduce_compressed_gathered),
+    # against copy-then-compressed-allreduce; 4 + 7 x 2 + 4 = 22 algorithmic bytes per element.
+    wire_peers = [[p.to(torch.bfloat16) for p in pv] for pv in peers]
+    del peers
+    torch.cuda.synchronize()
+
+    def hook_step():
+        works = []
+        for b, gr, pv in zip(bucket_of, grads, wire_peers):
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg._allreduce_compressed(b, torch.bfloat16, gr))
+        return works
+
+    def hook_two_pass():
+        works = []
+        for b, gr, pv in zip(bucket_of, grads, wire_peers):
+            at = 0
+            for t in gr:
+                b[at:at + t.numel()].copy_(t)
+                at += t.numel()
+            pg._set_simulated_peer_contributions(pv)
+            works.append(pg._allreduce_compressed(b, torch.bfloat16))
+        return works
+
+    hook_bytes = (4 + 2 * (k - 1) + 4) * n * buckets
+    hook_one = hook_bytes * steps / run(hook_step, steps, False) / 1e9
+    got_hook = [b.clone() for b in bucket_of]
+    hook_two = hook_bytes * steps / run(hook_two_pass, steps, False) / 1e9
+    for i, (a, b) in enumerate(zip(got_hook, bucket_of)):
+        if not torch.equal(a.view(torch.int32), b.view(torch.int32)):
+            raise SystemExit("parity FAILED: compressed from gradients differs from copy + "
+                             "compressed allreduce (bucket %d)" % i)
+    own0 = torch.cat(grads[0]).cpu().numpy()
+    want0 = oracle.compressed_sum(
+        [own0] + [p.view(torch.int16).cpu().numpy().view(np.uint16) for p in wire_peers[0]], 0,
+        "bf16", oracle.SCALE_MUL, float(np.float32(1) / np.float32(k)), threads=os.cpu_count() or 1)
+    if not (got_hook[0].cpu().numpy().view(np.uint32) == want0.view(np.uint32)).all():
+        raise SystemExit("parity FAILED on bucket 0 (compressed from gradients)")
     layout = pg._layout()
     del pg
     cfg = {
@@ -862,6 +901,12 @@ def run_gather(args, np, torch, fa, oracle, shared=None):
                                     "gradient into its bucket (torch's copy kernels) and "
                                     "ProcessGroup.allreduce on the bucket in place; results equal "
                                     "bit for bit",
+        "bf16_hook_from_grads_GBps": round(hook_one, 1),
+        "bf16_hook_copy_then_allreduce_GBps": round(hook_two, 1),
+        "bf16_hook_note": "the same buckets with torch's bf16 compression hook folded in (7 bf16 "
+                          "peers per bucket, 22 algorithmic bytes per element): own fp32 "
+                          "contribution read from the gradients, against copying them into the "
+                          "bucket first; results equal bit for bit, bucket 0 against the oracle",
         "staging_total_bytes": args.total_memory,
         "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
                    "staging_slots": layout[3]},
@@ -1168,7 +1213,8 @@ def main():
                                "steps": r["steps"], "ms_per_step": r["ms_per_step"],
                                "dtype": r["dtype"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
                                "parity": r["parity"].split(";")[0], "roofline": roof}
-                for key in ("host_link_GBps", "copy_then_allreduce_GBps"):
+                for key in ("host_link_GBps", "copy_then_allreduce_GBps",
+                            "bf16_hook_from_grads_GBps", "bf16_hook_copy_then_allreduce_GBps"):
                     if key in r["config"]:
                         extra[name][key] = r["config"][key]
             except (SystemExit, Exception) as e:  # noqa: BLE001  (reported, and the run fails)

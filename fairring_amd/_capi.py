@@ -20,7 +20,7 @@ EXPORTS = (
     "frg_compute_layout", "frg_num_slices", "frg_slice_bounds", "frg_plan_launches", "frg_reduce_slice", "frg_reduce_slice_static",
     "frg_reduce_slice_compressed", "frg_allreduce_compressed",
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
-    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_allreduce_gathered", "frg_reduce_pieces", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
+    "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_allreduce_gathered", "frg_allreduce_compressed_gathered", "frg_reduce_pieces", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
     "frg_set_tuning", "frg_set_tile_runs",
     "frg_last_error", "frg_version",
@@ -108,6 +108,9 @@ def lib():
                                            DONE_FN, vp, pvp]
     L.frg_allreduce_gathered.argtypes = [vp, vp, pvp, i32, i32, ctypes.POINTER(Segment), i32, i64,
                                          i32, i32, i32, f32, vp, DONE_FN, vp, pvp]
+    L.frg_allreduce_compressed_gathered.argtypes = [vp, vp, i32, pvp, i32, i32,
+                                                    ctypes.POINTER(Segment), i32, i64, i32, i32, f32,
+                                                    vp, DONE_FN, vp, pvp]
     L.frg_reduce_pieces.argtypes = [ctypes.POINTER(Piece), i32, i32, i32, i32, i32, f32, vp]
     L.frg_allreduce_host.argtypes = [vp, vp, pvp, i32, i64, i32, i32, i32, f32, i32, vp,
                                      DONE_FN, vp, pvp]

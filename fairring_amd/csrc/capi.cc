@@ -376,6 +376,52 @@ int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype, const void*
   });
 }
 
+int frg_allreduce_compressed_gathered(frg_ctx* ctx, void* out, int out_dtype,
+                                      const void* const* contribs, int K, int raw_index,
+                                      const frg_segment* segments, int num_segments, int64_t numel,
+                                      int wire_dtype, int scale_mode, float scale,
+                                      void* producer_stream, frg_done_fn done, void* user,
+                                      frg_work** work) {
+  if (work) *work = nullptr;
+  if (ctx == nullptr) return fail(FRG_ERR_INVALID, "null context");
+  if (K < 1 || contribs == nullptr) {
+    return fail(FRG_ERR_INVALID, "at least one contribution is required");
+  }
+  if (num_segments < 0 || (num_segments > 0 && segments == nullptr)) {
+    return fail(FRG_ERR_INVALID, "bad segment list");
+  }
+  if (raw_index < 0 || raw_index >= K) {
+    return fail(FRG_ERR_INVALID, "raw_index out of range (the piecewise contribution is the raw one)");
+  }
+  return guarded([&] {
+    Context::Request r;
+    r.out = out;
+    r.contribs.assign(contribs, contribs + K);
+    r.numel = numel;
+    r.dtype = wire_dtype;
+    r.op = FRG_SUM;
+    r.scaleMode = scale_mode;
+    r.scale = scale;
+    r.compressed = true;
+    r.outDtype = out_dtype;
+    r.rawIndex = raw_index;
+    r.gatheredIndex = raw_index;
+    r.gathered.reserve(static_cast<size_t>(num_segments));
+    for (int i = 0; i < num_segments; ++i) {
+      r.gathered.push_back(Context::Request::Segment{segments[i].ptr, segments[i].numel});
+    }
+    r.producerStream = static_cast<hipStream_t>(producer_stream);
+    r.done = done;
+    r.user = user;
+    std::string err;
+    Work* w = nullptr;
+    const int rc = asCtx(ctx)->submit(std::move(r), work ? &w : nullptr, &err);
+    if (rc != FRG_OK) return fail(rc, err);
+    if (work) *work = reinterpret_cast<frg_work*>(w);
+    return static_cast<int>(FRG_OK);
+  });
+}
+
 int frg_allreduce_host(frg_ctx* ctx, void* out, const void* const* host_contribs, int K,
                        int64_t numel, int dtype, int op, int scale_mode, float scale, int carry,
                        void* producer_stream, frg_done_fn done, void* user, frg_work** work) {

@@ -766,12 +766,17 @@ int Context::submit(Request req, Work** workOut, std::string* err) {
   }
   if (!req.gathered.empty() || req.gatheredIndex >= 0) {
     const int K = static_cast<int>(req.contribs.size());
-    if (req.fromHost || req.compressed) {
-      *err = "a piecewise contribution goes with device-resident, uncompressed contributions";
+    if (req.fromHost) {
+      *err = "a piecewise contribution goes with device-resident contributions";
       return FRG_ERR_UNSUPPORTED;
     }
     if (req.gatheredIndex < 0 || req.gatheredIndex >= K) {
       *err = "gathered_index out of range";
+      return FRG_ERR_INVALID;
+    }
+    if (req.compressed && req.gatheredIndex != req.rawIndex) {
+      // the gradients are what is still uncompressed
+      *err = "with compression folded in, the piecewise contribution is the raw fp32 one";
       return FRG_ERR_INVALID;
     }
     int64_t sum = 0;
@@ -1084,9 +1089,10 @@ Context::OpSpans Context::spansOf(const Request& req) {
       const uintptr_t es = (req.compressed && static_cast<int>(k) == req.rawIndex) ? 4 : wireSize;
       op.reads.push_back(Span{p, p + n * es});
     }
+    const uintptr_t segSize = req.compressed ? 4 : wireSize;  // the raw contribution is fp32
     for (const Request::Segment& g : req.gathered) {
       const uintptr_t p = reinterpret_cast<uintptr_t>(g.ptr);
-      if (g.numel > 0) op.reads.push_back(Span{p, p + static_cast<uintptr_t>(g.numel) * wireSize});
+      if (g.numel > 0) op.reads.push_back(Span{p, p + static_cast<uintptr_t>(g.numel) * segSize});
     }
   }
   return op;
@@ -1417,6 +1423,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req,
 // contributions, other element types), runs as a plain launch of its own.
 std::vector<hipStream_t> Context::runGathered(const Request& req,
                                               const std::vector<hipEvent_t>& initialEvents) {
+  if (req.compressed) return runGatheredCompressed(req, initialEvents);
   const int64_t elsize = elementSize(req.dtype);
   const int total = static_cast<int>(req.contribs.size());
   const int g = req.gatheredIndex;
@@ -1602,6 +1609,114 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
     }
   }
   if (!units.empty()) {
+    std::vector<size_t> ran;
+    for (size_t si = 0; si < nStreams; ++si) {
+      if (waited[si]) ran.push_back(si);
+    }
+    remember(spans, ran);
+  }
+  if (!waited[lastIdx]) {
+    waitInitials(reduceStreams_[lastIdx]);
+    waited[lastIdx] = 1;
+  }
+  std::vector<hipStream_t> used;
+  for (size_t si = 0; si < nStreams; ++si) {
+    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
+  }
+  used.push_back(reduceStreams_[lastIdx]);
+  return used;
+}
+
+// The reduction with a compression hook folded in, with the raw fp32
+// contribution still in the gradient tensors it is assembled from (what
+// torch's bf16 / fp16 compression hooks see with gradient_as_bucket_view=False
+// is a bucket that the reducer has just copied those tensors into): every
+// tensor is a launch of the compressed kernel of its own, or several for a
+// large one, with the tensor as the raw term and the output and the peers'
+// wire tensors at its offset in the bucket. The kernel takes the raw term by
+// its own pointer already (in place it is the output's), so this is the plain
+// compressed reduction cut where the gradients end; no table is involved, and
+// a tensor of a few KiB costs a launch, as the copy kernel it replaces did.
+std::vector<hipStream_t> Context::runGatheredCompressed(
+    const Request& req, const std::vector<hipEvent_t>& initialEvents) {
+  const int64_t wireSize = elementSize(req.dtype);
+  const int64_t outSize = elementSize(req.outDtype);
+  const int total = static_cast<int>(req.contribs.size());
+  const int g = req.gatheredIndex;
+  nextStagingSlot_ += numSlices(req.numel, layout_.sliceSizeInBytes, wireSize);
+  struct Part {
+    int64_t off;  // in the bucket, elements
+    int64_t len;
+    const void* raw;
+  };
+  std::vector<Part> parts;
+  const int64_t quantum = kLaunchQuantumBytes / wireSize;
+  int64_t off = 0;
+  for (const Request::Segment& seg : req.gathered) {
+    if (seg.numel <= 0) continue;
+    const int64_t launchBytes = defaultCompressedLaunchBytes(
+        total, /*hasRaw=*/true, req.outDtype == FRG_F32, seg.numel * wireSize);
+    int64_t partLen = roundDownToNearestMultiple(launchBytes / wireSize, quantum);
+    if (partLen < quantum) partLen = quantum;
+    int64_t at = 0;
+    while (2 * (seg.numel - at) > 3 * partLen) {
+      parts.push_back(Part{off + at, partLen, static_cast<const float*>(seg.ptr) + at});
+      at += partLen;
+    }
+    parts.push_back(Part{off + at, seg.numel - at, static_cast<const float*>(seg.ptr) + at});
+    off += seg.numel;
+  }
+  const size_t nStreams = reduceStreams_.size();
+  std::vector<char> initialsFired(initialEvents.size(), 0);
+  auto waitInitials = [&](hipStream_t stream) {
+    for (size_t i = 0; i < initialEvents.size(); ++i) {
+      bool fired = initialsFired[i] != 0;
+      waitInitial(stream, initialEvents[i], &fired);
+      initialsFired[i] = fired ? 1 : 0;
+    }
+  };
+  std::vector<char> waited(nStreams, 0);
+  const bool oneStream = parts.size() <= static_cast<size_t>(oneStreamLaunches_);
+  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
+  size_t lastIdx = opStream;
+  if (oneStream && !parts.empty()) ++nextLaunch_;
+  const OpSpans spans = spansOf(req);
+  if (!parts.empty()) {
+    std::vector<size_t> targets;
+    if (oneStream) {
+      targets.push_back(opStream);
+    } else {
+      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
+    }
+    orderAfterConflicts(spans, targets);
+  }
+  std::vector<const void*> ptrs(static_cast<size_t>(total));
+  for (const Part& part : parts) {
+    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
+    hipStream_t s = reduceStreams_[si];
+    if (!waited[si]) {
+      waitInitials(s);
+      waited[si] = 1;
+    }
+    lastIdx = si;
+    for (int k = 0; k < total; ++k) {
+      ptrs[static_cast<size_t>(k)] =
+          k == g ? part.raw
+                 : static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + part.off * wireSize;
+    }
+    CompressedArgs a;
+    a.out = static_cast<char*>(req.out) + part.off * outSize;
+    a.out_dtype = req.outDtype;
+    a.contribs = ptrs.data();
+    a.K = total;
+    a.raw_index = g;
+    a.n = part.len;
+    a.wire_dtype = req.dtype;
+    a.scale_mode = req.scaleMode;
+    a.scale = req.scale;
+    launchCompressed(a, s);
+  }
+  if (!parts.empty()) {
     std::vector<size_t> ran;
     for (size_t si = 0; si < nStreams; ++si) {
       if (waited[si]) ran.push_back(si);

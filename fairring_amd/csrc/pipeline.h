@@ -189,6 +189,8 @@ class Context {
                       int (*enqueue)(const Args&, hipStream_t, std::string*));
   void launch(const struct ReduceArgs& args, hipStream_t stream);
   void launchCompressed(const struct CompressedArgs& args, hipStream_t stream);
+  std::vector<hipStream_t> runGatheredCompressed(const Request& req,
+                                                 const std::vector<hipEvent_t>& initialEvents);
   void chainThroughScratch(const Request& req, const std::vector<const void*>& ptrs, int64_t off,
                            int64_t len, size_t streamIdx, bool acc);
   char* scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize);

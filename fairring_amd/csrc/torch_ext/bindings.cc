@@ -56,7 +56,8 @@ void bind(py::module& m) {
   group.def("_allreduce_pre_divided", &PG::allreducePreDivided, py::arg("bucket"),
             py::call_guard<py::gil_scoped_release>());
   group.def("_allreduce_compressed", &PG::allreduceCompressed, py::arg("bucket"),
-            py::arg("wire_dtype"), py::call_guard<py::gil_scoped_release>());
+            py::arg("wire_dtype"), py::arg("grads") = std::vector<at::Tensor>(),
+            py::call_guard<py::gil_scoped_release>());
   // the allreduce of a bucket read from the gradient tensors it is assembled from
   group.def("_allreduce_from_grads", &PG::allreduceFromGrads, py::arg("bucket"), py::arg("grads"),
             py::arg("pre_divide") = false, py::call_guard<py::gil_scoped_release>());

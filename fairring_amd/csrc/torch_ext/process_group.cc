@@ -887,8 +887,8 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceFromGrads(
       c10::intrusive_ptr<c10d::Backend>::unsafe_reclaim_from_nonowning(this), ctx);
 }
 
-c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Tensor bucket,
-                                                                         at::ScalarType wire) {
+c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(
+    at::Tensor bucket, at::ScalarType wire, std::vector<at::Tensor> grads) {
   FRG_CHECK(bucket.layout() == at::kStrided);
   FRG_CHECK(bucket.is_cuda());
   FRG_CHECK(bucket.is_non_overlapping_and_dense());
@@ -897,6 +897,21 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
   TORCH_CHECK(wire == at::kBFloat16 || wire == at::kHalf,
               "fairring: the wire type must be bfloat16 or float16, got ", wire);
   at::Tensor t = viewAsFlat(bucket);
+  // the bucket's own contribution, where it is still in the gradients it is assembled from
+  std::vector<frg_segment> segments;
+  segments.reserve(grads.size());
+  int64_t held = 0;
+  for (at::Tensor& gr : grads) {
+    TORCH_CHECK(gr.is_cuda() && gr.device() == t.device() && gr.scalar_type() == at::kFloat,
+                "fairring: a gradient must be a float32 tensor on the bucket's device");
+    TORCH_CHECK(gr.layout() == at::kStrided && gr.is_non_overlapping_and_dense(),
+                "fairring: a gradient must be dense");
+    gr = viewAsFlat(gr);
+    segments.push_back(frg_segment{gr.data_ptr(), gr.numel()});
+    held += gr.numel();
+  }
+  TORCH_CHECK(grads.empty() || held == t.numel(), "fairring: the gradients hold ", held,
+              " elements, the bucket ", t.numel());
 
   std::lock_guard<std::mutex> g(mutex_);
   const c10::DeviceIndex device = t.device().index();
@@ -922,18 +937,27 @@ c10::intrusive_ptr<c10d::Work> ProcessGroupFairring::allreduceCompressed(at::Ten
     table.push_back(r == rank ? t.data_ptr() : peers[pi].data_ptr());
     if (r != rank) ++pi;
   }
-  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&t}, nullptr);
+  recordOnPipelineStreams(device, /*copyStreamsToo=*/false, {&t}, grads.empty() ? nullptr : &grads);
   auto future = c10::make_intrusive<c10::ivalue::Future>(
       c10::ListType::ofTensors(), std::vector<c10::Device>{t.device()});
   hipStream_t current = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device).stream();
-  // the peers are held until the operation is enqueued (see reduceCommon)
-  auto* pending = new Pending{future, t, peers, device};
+  // the peers (and the gradients) are held until the operation is enqueued (see reduceCommon)
+  std::vector<at::Tensor> keep = peers;
+  keep.insert(keep.end(), grads.begin(), grads.end());
+  auto* pending = new Pending{future, t, std::move(keep), device};
   // buffer.to(wire).div_(size): on the GPU a multiply by the reciprocal, in
   // the wire type's arithmetic
-  const int rc = frg_allreduce_compressed(
-      ctx, t.data_ptr(), FRG_F32, table.data(), size, rank, n,
-      wire == at::kBFloat16 ? FRG_BF16 : FRG_F16, size > 1 ? FRG_SCALE_MUL : FRG_SCALE_NONE,
-      1.0f / static_cast<float>(size), current, &onDone, pending, nullptr);
+  const int wireCode = wire == at::kBFloat16 ? FRG_BF16 : FRG_F16;
+  const int scaleMode = size > 1 ? FRG_SCALE_MUL : FRG_SCALE_NONE;
+  const float scale = 1.0f / static_cast<float>(size);
+  const int rc =
+      segments.empty()
+          ? frg_allreduce_compressed(ctx, t.data_ptr(), FRG_F32, table.data(), size, rank, n,
+                                     wireCode, scaleMode, scale, current, &onDone, pending, nullptr)
+          : frg_allreduce_compressed_gathered(ctx, t.data_ptr(), FRG_F32, table.data(), size, rank,
+                                              segments.data(), static_cast<int>(segments.size()),
+                                              n, wireCode, scaleMode, scale, current, &onDone,
+                                              pending, nullptr);
   if (rc != FRG_OK) {
     delete pending;
     TORCH_CHECK(false, "fairring: ", frg_last_error());

@@ -156,7 +156,10 @@ class ProcessGroupFairring : public c10d::Backend {
   // their buckets already compressed (tensors of `wire`, scaled by 1/size);
   // this rank's bucket is compressed in registers, the sum is rounded to
   // `wire` once and written back widened into `bucket`.
-  c10::intrusive_ptr<c10d::Work> allreduceCompressed(at::Tensor bucket, at::ScalarType wire);
+  // With `grads`, the bucket's own contribution is read from those tensors (in
+  // bucket order) instead of from the bucket (frg_allreduce_compressed_gathered).
+  c10::intrusive_ptr<c10d::Work> allreduceCompressed(at::Tensor bucket, at::ScalarType wire,
+                                                     std::vector<at::Tensor> grads = {});
   // allreduceFromGrads: the allreduce of a bucket together with the copy that
   // fills it. With DDP's default (gradient_as_bucket_view=False) the reducer
   // copies every gradient to its place in the bucket just before the allreduce

@@ -327,25 +327,62 @@ class DeviceFairring:
         return self._submit(out, contribs, op, scale_mode, scale, stream, host=False, done=done)
 
     def allreduce_compressed(self, out, contribs, raw_index=-1, scale_mode=SCALE_NONE, scale=1.0,
-                             wire_dtype=None, stream=None):
+                             wire_dtype=None, stream=None, segments=None):
         """reduce_slice_compressed through the slice pipeline (sliced by the
-        wire type's element size). Returns at once."""
+        wire type's element size). With `segments`, the raw fp32 contribution
+        is that list of tensors, in the order they lie in the bucket
+        (frg_allreduce_compressed_gathered; contribs[raw_index] is ignored and
+        may be None, `wire_dtype` must then be given unless there are peers).
+        Returns at once."""
         import torch
         _check_dense(out, "output")
-        for c in contribs:
+        if segments is None:
+            for c in contribs:
+                _check_dense(c, "contribution")
+            wire = _check_compressed(out, contribs, raw_index)
+            if wire_dtype is not None:
+                wire = BF16 if wire_dtype == torch.bfloat16 else F16
+            stream = torch.cuda.current_stream(out.device) if stream is None else stream
+            tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+            wh = ctypes.c_void_p()
+            self._record_on_streams([out] + list(contribs))
+            _capi.check(_capi.lib().frg_allreduce_compressed(
+                self._h, out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index,
+                out.numel(), wire, scale_mode, scale, stream.cuda_stream, _capi.DONE_FN(), None,
+                ctypes.byref(wh)))
+            return Work(wh, (out, list(contribs)))
+        peers = [c for k, c in enumerate(contribs) if k != raw_index]
+        total = 0
+        for t in segments:
+            _check_dense(t, "segment")
+            if t.dtype != torch.float32 or t.device != out.device:
+                raise FairringError(_capi.ERR_INVALID, "segments are fp32 tensors on the output's device")
+            total += t.numel()
+        if total != out.numel():
+            raise FairringError(_capi.ERR_INVALID, "the segments hold %d elements, the output %d"
+                                % (total, out.numel()))
+        for c in peers:
             _check_dense(c, "contribution")
-        wire = _check_compressed(out, contribs, raw_index)
-        if wire_dtype is not None:
-            wire = BF16 if wire_dtype == torch.bfloat16 else F16
+            if c.numel() != out.numel() or c.dtype not in (torch.bfloat16, torch.float16):
+                raise FairringError(_capi.ERR_INVALID, "peers are bf16 / fp16 tensors of the output's length")
+        if wire_dtype is None:
+            if not peers:
+                raise FairringError(_capi.ERR_INVALID, "wire_dtype is required without peers")
+            wire_dtype = peers[0].dtype
+        wire = BF16 if wire_dtype == torch.bfloat16 else F16
         stream = torch.cuda.current_stream(out.device) if stream is None else stream
-        tab = _capi.ptr_table([c.data_ptr() for c in contribs])
+        tab = _capi.ptr_table([0 if k == raw_index else c.data_ptr() for k, c in enumerate(contribs)])
+        segs = (_capi.Segment * max(1, len(segments)))()
+        for i, t in enumerate(segments):
+            segs[i].ptr = t.data_ptr()
+            segs[i].numel = t.numel()
         wh = ctypes.c_void_p()
-        self._record_on_streams([out] + list(contribs))
-        _capi.check(_capi.lib().frg_allreduce_compressed(
-            self._h, out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index,
-            out.numel(), wire, scale_mode, scale, stream.cuda_stream, _capi.DONE_FN(), None,
-            ctypes.byref(wh)))
-        return Work(wh, (out, list(contribs)))
+        self._record_on_streams([out] + peers + list(segments))
+        _capi.check(_capi.lib().frg_allreduce_compressed_gathered(
+            self._h, out.data_ptr(), _dtype_code(out), tab, len(contribs), raw_index, segs,
+            len(segments), out.numel(), wire, scale_mode, scale, stream.cuda_stream,
+            _capi.DONE_FN(), None, ctypes.byref(wh)))
+        return Work(wh, (out, peers, list(segments)))
 
     def allreduce_gathered(self, out, contribs, gathered_index, segments, op=SUM,
                            scale_mode=SCALE_NONE, scale=1.0, stream=None, done=None):

@@ -366,12 +366,28 @@ FRG_API int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype,
                                      void* producer_stream, frg_done_fn done, void* user,
                                      frg_work** work);
 
+/* The same with the raw fp32 contribution still in the tensors the bucket is
+ * assembled from (what torch's compression hooks meet with DDP's default
+ * gradient_as_bucket_view=False, after the reducer has copied every gradient
+ * into the bucket: torch:csrc/distributed/c10d/reducer.cpp, copy_grad_to_bucket):
+ * contribution `raw_index` is read from `segments` (fp32, in bucket order,
+ * lengths adding up to `numel`; contribs[raw_index] is ignored), every tensor
+ * a launch of the compressed reduction of its own or, when large, several. */
+FRG_API int frg_allreduce_compressed_gathered(frg_ctx* ctx, void* out, int out_dtype,
+                                              const void* const* contribs, int K,
+                                              int raw_index, const frg_segment* segments,
+                                              int num_segments, int64_t numel, int wire_dtype,
+                                              int scale_mode, float scale,
+                                              void* producer_stream, frg_done_fn done,
+                                              void* user, frg_work** work);
+
 /* Server-side accumulation with contributions in pinned host memory
- * (device.cc:543-589: collect into a staging slot, then reduce): contribution
- * k is copied with hipMemcpyAsync on the copy stream into staging slot
- * (next++) % numSlots once the event recorded after that slot's previous
- * consumer has fired, and folded into `out` on the reduce stream in
- * contribution order. `host_contribs[k]` are host pointers (hipHostMalloc'd).
+ * (device.cc:543-589: collect into a staging slot, then reduce): the staging
+ * slots are taken in rotation, (next++) % numSlots, a batch of contributions
+ * is copied with hipMemcpyAsync into the slots of its turn and folded into
+ * `out`, in contribution order, by the stream that copied them, so that a
+ * slot is not filled again before its last reader has run.
+ * `host_contribs[k]` are host pointers (hipHostMalloc'd).
  * carry = 0: the K host contributions are all there is (the first one is
  * copied straight into `out`). carry = 1: `out` already holds the device's own
  * contribution, which comes first in the order (the reference reduces the
@@ -502,7 +518,8 @@ FRG_API const char* frg_last_error(void);
  * frg_reduce_slice_static added (and frg_progress grew in place, which 0.3
  * takes back). 0.3: frg_progress has its four fields of 0.1 again and
  * frg_get_progress2 carries the later counters with the caller's struct size;
- * frg_allreduce_gathered, frg_reduce_pieces and frg_set_tile_runs added. */
+ * frg_allreduce_gathered, frg_allreduce_compressed_gathered, frg_reduce_pieces
+ * and frg_set_tile_runs added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus

@@ -215,6 +215,39 @@ void scenarioPreScaleAndCompressed() {
   CHECK(frg_work_wait(w) == FRG_OK);
   CHECK(same(raw, want));
   frg_work_release(w);
+  // the same with the raw contribution in four tensors of its own (one of them empty, one of
+  // a single element), into a separate bucket: a launch per tensor, same result
+  {
+    const Vec rawAgain = randomContribs(1, n, 22)[0];
+    const int64_t cuts[6] = {0, 4096, 4096, 4097, 9000, n};
+    std::vector<Vec> tensors;
+    std::vector<frg_segment> segs;
+    for (int i = 0; i < 5; ++i) {
+      tensors.emplace_back(rawAgain.begin() + cuts[i], rawAgain.begin() + cuts[i + 1]);
+    }
+    for (const Vec& v : tensors) segs.push_back(frg_segment{v.data(), static_cast<int64_t>(v.size())});
+    Vec bucket(static_cast<size_t>(n), -3.f);
+    std::vector<const void*> gtab = tab;
+    gtab[rawIndex] = nullptr;  // ignored
+    frg_progress before = {};
+    CHECK(frg_get_progress(ctx, &before) == FRG_OK);
+    CHECK(frg_allreduce_compressed_gathered(ctx, bucket.data(), FRG_F32, gtab.data(), K, rawIndex,
+                                            segs.data(), 5, n, FRG_BF16, FRG_SCALE_MUL, 0.2f,
+                                            nullptr, nullptr, nullptr, &w) == FRG_OK);
+    CHECK(frg_work_wait(w) == FRG_OK);
+    CHECK(same(bucket, want));
+    frg_work_release(w);
+    frg_progress after = {};
+    CHECK(frg_get_progress(ctx, &after) == FRG_OK);
+    CHECK(after.launches - before.launches == 4);  // one per tensor that holds anything
+    // the piecewise contribution is the raw one, and its lengths must add up
+    CHECK(frg_allreduce_compressed_gathered(ctx, bucket.data(), FRG_F32, gtab.data(), K, -1,
+                                            segs.data(), 5, n, FRG_BF16, 0, 1.f, nullptr, nullptr,
+                                            nullptr, nullptr) == FRG_ERR_INVALID);
+    CHECK(frg_allreduce_compressed_gathered(ctx, bucket.data(), FRG_F32, gtab.data(), K, rawIndex,
+                                            segs.data(), 4, n, FRG_BF16, 0, 1.f, nullptr, nullptr,
+                                            nullptr, nullptr) == FRG_ERR_INVALID);
+  }
   // under graph capture the pipeline refuses (the one-launch entry points are the ones to capture)
   fake_hip_set_capturing(1);
   CHECK(frg_allreduce(ctx, out.data(), t.data(), 3, 3001, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.f,

@@ -158,6 +158,52 @@ def test_allreduce_from_grads(kind, tdt, rank, size):
         pg._allreduce_from_grads(bucket, grads[:-1], True)
 
 
+@pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+@pytest.mark.parametrize("rank,size", [(0, 2), (5, 8), (2, 3)])
+def test_allreduce_compressed_from_grads(wire, tdt, rank, size):
+    # the compression hooks' reduction with the bucket's own fp32 contribution read from the
+    # gradient tensors: the bucket holds garbage on the way in and the oracle's result on the
+    # way out, and the hook gives the bits of the hook that reads an assembled bucket
+    print("[case] pg compressed from grads", wire, rank, size, flush=True)
+    shapes = [(1024, 512), (512,), (1,), (300, 7), (64, 64, 3), (5,)]
+    n = sum(int(np.prod(sh)) for sh in shapes)
+    rng = np.random.default_rng(50 * size + rank)
+    x = (rng.standard_normal((size, n)) * 0.01).astype(np.float32)
+    bits = oracle.np_f32_to_bf16_rne(x) if wire == "bf16" else x.astype(np.float16).view(np.uint16)
+    pg = make_pg(rank, size)
+    pg._set_simulated_peer_contributions(
+        [torch.from_numpy(bits[r].view(np.int16).copy()).to(DEV).view(tdt)
+         for r in range(size) if r != rank])
+    grads, off = [], 0
+    for sh in shapes:
+        ln = int(np.prod(sh))
+        grads.append(torch.from_numpy(x[rank, off:off + ln].copy()).to(DEV).view(sh))
+        off += ln
+    bucket = torch.full((n,), float("nan"), device=DEV)
+    pg._allreduce_compressed(bucket, tdt, grads).wait()
+    torch.cuda.synchronize()
+    contribs = [bits[r] for r in range(size)]
+    contribs[rank] = x[rank]
+    s = float(np.float32(1) / np.float32(size))
+    assert_bits_equal(bucket.cpu().numpy(),
+                      oracle.compressed_sum(contribs, rank, wire, oracle.SCALE_MUL, s))
+    params = []
+    for gr in grads:
+        p = torch.nn.Parameter(torch.zeros_like(gr))
+        p.grad = gr
+        params.append(p)
+    assembled = torch.cat([gr.reshape(-1) for gr in grads])
+    hook = getattr(ddp_comm_hooks, "%s_compress_from_grads_hook" % ("bf16" if wire == "bf16" else "fp16"))
+    plain = getattr(ddp_comm_hooks, "%s_compress_hook" % ("bf16" if wire == "bf16" else "fp16"))
+    got = hook(pg, GradBucket(assembled.clone().fill_(7), params)).wait()
+    torch.cuda.synchronize()
+    want = plain(pg, Bucket(assembled)).wait()
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    with pytest.raises(RuntimeError, match="gradients hold"):
+        pg._allreduce_compressed(bucket, tdt, grads[:-1])
+
+
 def test_hook_contract_errors():
     print("[case] pg hook errors", flush=True)
     pg = make_pg(0, 2)
@@ -215,6 +261,12 @@ for a, b in zip(plain, grads(ours.allreduce_hook)):
 for a, b in zip(grads(torch_hooks.allreduce_hook), grads(ours.allreduce_from_grads_hook)):
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
 print("allreduce_from_grads_hook ok", flush=True)
+for name in ("bf16_compress", "fp16_compress"):
+    want = grads(getattr(torch_hooks, name + "_hook"))
+    got = grads(getattr(ours, name + "_from_grads_hook"))
+    for a, b in zip(want, got):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), name
+    print(name + "_from_grads_hook ok", flush=True)
 print("ddp hooks ok")
 dist.destroy_process_group()
 """

@@ -206,3 +206,75 @@ def test_allreduce_gathered_waits_for_the_gradients_and_orders_what_follows():
         assert float(out[n_big:].min()) == rest + 200.0 == float(out[n_big:].max())
         assert float(grads[0].min()) == 2.0 == float(grads[0].max())
     dev.close()
+
+
+# ---- the compression hooks' reduction with the raw contribution in tensors of its own ---------
+
+@pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+@pytest.mark.parametrize("k,g", [(8, 0), (8, 5), (2, 1), (4, 3), (17, 9)])
+def test_allreduce_compressed_gathered_vs_oracle(wire, tdt, k, g):
+    # The raw fp32 contribution (rank g) as the gradient tensors of a layer, the peers'
+    # contributions as wire tensors of the bucket's length, the fp32 bucket written once:
+    # the oracle's compressed sum over the concatenated gradients, and the bits of the
+    # one-pass reduction over an assembled bucket (frg_allreduce_compressed in place).
+    rng = np.random.default_rng(131 * k + g)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    try:
+        for name, mode, omode, scale_of in SCALES[:3]:
+            _print_case("compressed gathered", wire, k, g, name)
+            lens = LAYER if name != "div" else [2048 * 2048 * 2, 5, 2048 * 512 + 3]   # the last: large tensors, odd ends
+            n = int(sum(lens))
+            x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+            bits = oracle.np_f32_to_bf16_rne(x) if wire == "bf16" else x.astype(np.float16).view(np.uint16)
+            host = [bits[j] for j in range(k)]
+            host[g] = x[g]
+            peers = [None if j == g else to_gpu(wire, bits[j]) for j in range(k)]
+            segs, off = [], 0
+            for ln in lens:
+                segs.append(to_gpu("f32", x[g, off:off + ln]))
+                off += ln
+            s = scale_of(k) if name != "mul" else float(np.float32(1) / np.float32(k))
+            out = torch.full((n,), 7.0, device=DEV)
+            dev.allreduce_compressed(out, peers, g, scale_mode=mode, scale=s, wire_dtype=tdt,
+                                     segments=segs).wait()
+            want = oracle.compressed_sum(host, g, wire, omode, s)
+            assert_bits_equal(out.cpu().numpy(), want, "%s k=%d g=%d %s" % (wire, k, g, name))
+            # the assembled bucket, reduced in place
+            bucket = to_gpu("f32", x[g])
+            contribs = list(peers)
+            contribs[g] = bucket
+            dev.allreduce_compressed(bucket, contribs, g, scale_mode=mode, scale=s, wire_dtype=tdt).wait()
+            assert bool(torch.equal(bucket.view(torch.int32), out.view(torch.int32)))
+    finally:
+        dev.close()
+
+
+def test_allreduce_compressed_gathered_wire_output_and_contract():
+    _print_case("compressed gathered: wire output, contract")
+    rng = np.random.default_rng(9)
+    k, g = 4, 2
+    lens = [4099, 0, 262147, 1]
+    n = int(sum(lens))
+    x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+    bits = oracle.np_f32_to_bf16_rne(x)
+    host = [bits[j] for j in range(k)]
+    host[g] = x[g]
+    peers = [None if j == g else to_gpu("bf16", bits[j]) for j in range(k)]
+    segs, off = [], 0
+    for ln in lens:
+        segs.append(to_gpu("f32", x[g, off:off + ln]))
+        off += ln
+    dev = fa.DeviceFairring(0)
+    try:
+        out = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+        dev.allreduce_compressed(out, peers, g, wire_dtype=torch.bfloat16, segments=segs).wait()
+        want = oracle.compressed_sum(host, g, "bf16", oracle.SCALE_NONE, 1.0, out_f32=False)
+        assert_bits_equal(from_gpu("bf16", out), want, "wire output")
+        with pytest.raises(fa.FairringError):                       # lengths must add up
+            dev.allreduce_compressed(torch.empty(n, device=DEV), peers, g, wire_dtype=torch.bfloat16,
+                                     segments=segs[:-1])
+        with pytest.raises(fa.FairringError):                       # segments are fp32
+            dev.allreduce_compressed(torch.empty(n, device=DEV), peers, g, wire_dtype=torch.bfloat16,
+                                     segments=[s.to(torch.bfloat16) for s in segs])
+    finally:
+        dev.close()
