@@ -20,6 +20,8 @@
 #include <hip/hip_ext.h>
 #include <hip/hip_runtime.h>
 
+#include <limits>
+
 #include "../../include/fairring_hip.h"
 #include "device_traits.h"
 #include "ksum_kernels.h"
@@ -45,14 +47,37 @@ struct StagedChunks {
   f32x4 lo, hi;
 };
 
-__device__ __forceinline__ StagedChunks issueStaged(const float* base, int64_t elemBase,
+// Where the raw fp32 term of element e is read from: `origin(e) + e`. One
+// buffer; or the tensors a bucket is assembled from, each given by its address
+// minus its offset in the bucket (so that adding the element's index lands in
+// it) and the element it starts at. Every 16-byte access lies within one
+// tensor (the launch code sees to it), so a lane looks its tensor up once per
+// access, by straight-line compares over the few entries.
+struct RawPlain {
+  const float* base;
+  __device__ __forceinline__ const float* origin(int64_t) const { return base; }
+};
+constexpr int kMaxRawPieces = 8;
+struct RawPieces {
+  const float* adj[kMaxRawPieces];
+  long long off[kMaxRawPieces];  // off[0] = 0; unused entries hold the largest value
+  __device__ __forceinline__ const float* origin(int64_t e) const {
+    const float* p = adj[0];
+#pragma unroll
+    for (int i = 1; i < kMaxRawPieces; ++i) p = e >= off[i] ? adj[i] : p;
+    return p;
+  }
+};
+
+template <typename RAW>
+__device__ __forceinline__ StagedChunks issueStaged(const RAW& raw, int64_t elemBase,
                                                     unsigned int lane) {
   const unsigned int waveLane = lane & 63u;
   const int64_t waveBase = elemBase + static_cast<int64_t>(lane - waveLane) * 8;
-  const f32x4* p = reinterpret_cast<const f32x4*>(base + waveBase) + waveLane;
+  const int64_t lo = waveBase + 4 * static_cast<int64_t>(waveLane);
   StagedChunks c;
-  c.lo = ldStream(p);
-  c.hi = ldStream(p + 64);
+  c.lo = ldStream(reinterpret_cast<const f32x4*>(raw.origin(lo) + lo));
+  c.hi = ldStream(reinterpret_cast<const f32x4*>(raw.origin(lo + 256) + lo + 256));
   return c;
 }
 
@@ -170,8 +195,8 @@ __device__ __forceinline__ void foldWire(Fold<W>& st, const Ptrs<0>& in, int k0,
 // `raw` this rank's fp32 buffer (rawPos = its place in the chain, -1: absent).
 // STAGED (whole tiles of the 8-element variant only): the fp32 side goes
 // through loadStaged / storeStaged.
-template <typename W, bool OUT32, bool STAGED = false>
-__device__ __forceinline__ void compressedOne(void* out, const float* raw, const Ptrs<0>& wire,
+template <typename W, bool OUT32, bool STAGED = false, typename RAW = RawPlain>
+__device__ __forceinline__ void compressedOne(void* out, const RAW& raw, const Ptrs<0>& wire,
                                               int Kw, int rawPos, int scaleMode, float scale,
                                               int64_t elemBase, unsigned int lane,
                                               f32x4* stage = nullptr) {
@@ -186,7 +211,8 @@ __device__ __forceinline__ void compressedOne(void* out, const float* raw, const
       st.stage = stage;
       st.lane = lane;
     } else {
-      rawRegs = Side::load(raw + elemBase, lane);
+      rawRegs = Side::load(
+          raw.origin(elemBase + static_cast<int64_t>(lane) * W::kLanes) + elemBase, lane);
     }
   }
   int k = 0;
@@ -232,8 +258,8 @@ __device__ __forceinline__ void compressedOne(void* out, const float* raw, const
 // lasts 20 us and every CU starts it with a cold instruction cache). Same
 // arithmetic, in the same order, as compressedOne.
 // STAGED (whole tiles): the fp32 side goes through loadStaged / storeStaged.
-template <typename W, int KW, int SC, bool STAGED = false>
-__device__ __forceinline__ void compressedFixed(float* out, const float* raw, const Ptrs<KW>& wire,
+template <typename W, int KW, int SC, bool STAGED = false, typename RAW = RawPlain>
+__device__ __forceinline__ void compressedFixed(float* out, const RAW& raw, const Ptrs<KW>& wire,
                                                 int rawPos, float scale, int64_t elemBase,
                                                 unsigned int lane, f32x4* stage = nullptr) {
   using vec_t = typename W::vec_t;
@@ -245,7 +271,8 @@ __device__ __forceinline__ void compressedFixed(float* out, const float* raw, co
   if constexpr (STAGED) {
     chunks = issueStaged(raw, elemBase, lane);
   } else {
-    rawRegs = Side::load(raw + elemBase, lane);
+    rawRegs = Side::load(
+        raw.origin(elemBase + static_cast<int64_t>(lane) * W::kLanes) + elemBase, lane);
   }
   vec_t v[KW];
 #pragma unroll
@@ -299,22 +326,24 @@ __device__ __forceinline__ void compressedFixed(float* out, const float* raw, co
 
 // KW > 0: the fixed shape above (OUT32, raw term present, scale mode SC);
 // KW == 0: the general body.
-template <typename W, bool OUT32, int KW, int SC>
-__device__ __forceinline__ void compressedLane(void* out, const float* raw, const Ptrs<KW>& wire,
+template <typename W, bool OUT32, int KW, int SC, typename RAW>
+__device__ __forceinline__ void compressedLane(void* out, const RAW& raw, const Ptrs<KW>& wire,
                                                int Kw, int rawPos, int scaleMode, float scale,
                                                int64_t elemBase, unsigned int lane) {
   if constexpr (KW > 0) {
-    compressedFixed<W, KW, SC>(static_cast<float*>(out), raw, wire, rawPos, scale, elemBase, lane);
+    compressedFixed<W, KW, SC, false, RAW>(static_cast<float*>(out), raw, wire, rawPos, scale,
+                                           elemBase, lane);
   } else {
-    compressedOne<W, OUT32>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase, lane);
+    compressedOne<W, OUT32, false, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
+                                        lane);
   }
 }
 
 // Same dealing of tiles, remainder pieces and ragged edges as the plain
 // reduction kernel; a "vector" is a lane's group of 8 elements.
-template <typename WV, typename WS, bool OUT32, int KW, int SC>
+template <typename WV, typename WS, bool OUT32, int KW, int SC, typename RAW>
 __global__ void __launch_bounds__(kBlock)
-    compressedKernel(void* out, const float* raw, Ptrs<KW> wire, int Kw, int rawPos, int scaleMode,
+    compressedKernel(void* out, const RAW raw, Ptrs<KW> wire, int Kw, int rawPos, int scaleMode,
                      float scale, int64_t head, int lead, int64_t nvec, int64_t tail,
                      int64_t roundTiles, int64_t pieces, int chunkShift) {
   constexpr int64_t kTile = static_cast<int64_t>(kBlock) * kUnroll;
@@ -342,13 +371,13 @@ __global__ void __launch_bounds__(kBlock)
     for (int u = 0; u < kUnroll; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
       if constexpr (kStaged && KW > 0) {
-        compressedFixed<WV, KW, SC, true>(static_cast<float*>(out), raw, wire, rawPos, scale,
-                                          elemBase, lane, stage);
+        compressedFixed<WV, KW, SC, true, RAW>(static_cast<float*>(out), raw, wire, rawPos,
+                                               scale, elemBase, lane, stage);
       } else if constexpr (kStaged) {
-        compressedOne<WV, OUT32, true>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
-                                       lane, stage);
+        compressedOne<WV, OUT32, true, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale,
+                                            elemBase, lane, stage);
       } else {
-        compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
+        compressedLane<WV, OUT32, KW, SC, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
                                           lane);
       }
     }
@@ -362,28 +391,30 @@ __global__ void __launch_bounds__(kBlock)
     for (int u = 0; u < kPiece; ++u) {
       const unsigned int lane = threadIdx.x + u * kBlock;
       if (v0 + lane < bodyVecs) {
-        compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale,
+        compressedLane<WV, OUT32, KW, SC, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale,
                                           bodyBase + v0 * WV::kLanes, lane);
       }
     }
   }
   if (lead > 0 && blockIdx.x == gridDim.x - 1) {
     for (unsigned int lane = threadIdx.x; lane < static_cast<unsigned int>(lead); lane += kBlock) {
-      compressedLane<WV, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, head, lane);
+      compressedLane<WV, OUT32, KW, SC, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale, head, lane);
     }
   }
   if (blockIdx.x == 0 && threadIdx.x < head + tail) {
     const int64_t e = threadIdx.x < head
                           ? static_cast<int64_t>(threadIdx.x)
                           : head + nvec * WV::kLanes + (threadIdx.x - head);
-    compressedLane<WS, OUT32, KW, SC>(out, raw, wire, Kw, rawPos, scaleMode, scale, e, 0u);
+    compressedLane<WS, OUT32, KW, SC, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale, e, 0u);
   }
 }
 
-template <typename WV, typename WS, bool OUT32, int KW = 0, int SC = 0>
-hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptrs<0>& all, int Kw,
-                            int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
-                            hipStream_t stream) {
+// `leadRef`: the address whose 4 KiB grid the tiles follow when there is no wire
+// contribution (the raw buffer's; the output's when the raw term comes in pieces).
+template <typename WV, typename WS, bool OUT32, int KW, int SC, typename RAW>
+hipError_t launchCompressed(const CompressedArgs& a, const RAW& raw, uintptr_t leadRef,
+                            const Ptrs<0>& all, int Kw, int rawPos, int64_t head, int64_t nvec,
+                            int64_t tail, int numCus, hipStream_t stream) {
   Ptrs<KW> wire;
   for (int k = 0; k < (KW > 0 ? KW : kMaxContribsPerLaunch); ++k) wire.p[k] = all.p[k];
   // groups between the first one and the next 4 KiB boundary of the first wire
@@ -392,7 +423,7 @@ hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptr
   if (sizeof(typename WV::vec_t) == 16) {
     const uintptr_t first =
         Kw > 0 ? reinterpret_cast<uintptr_t>(all.p[0]) + static_cast<uintptr_t>(head) * 2
-               : (reinterpret_cast<uintptr_t>(raw) + static_cast<uintptr_t>(head) * 4) / 2;
+               : (leadRef + static_cast<uintptr_t>(head) * 4) / 2;
     const int64_t l = static_cast<int64_t>(
         ((kLaunchAlignBytes - (first & (kLaunchAlignBytes - 1))) & (kLaunchAlignBytes - 1)) / 16);
     lead = l < nvec ? static_cast<int>(l) : 0;
@@ -408,13 +439,13 @@ hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptr
                              ? shift
                              : 0;
   if (a.startEvent != nullptr || a.stopEvent != nullptr) {
-    hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
+    hipExtLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC, RAW>),
                           dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream,
                           a.startEvent, a.stopEvent, 0, a.out, raw, wire, Kw, rawPos, a.scale_mode,
                           a.scale, head, lead, nvec, tail, plan.roundTiles, plan.pieces,
                           chunkShift);
   } else {
-    hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC>),
+    hipLaunchKernelGGL((compressedKernel<WV, WS, OUT32, KW, SC, RAW>),
                        dim3(static_cast<unsigned>(plan.grid)), dim3(kBlock), 0, stream, a.out, raw,
                        wire, Kw, rawPos, a.scale_mode, a.scale, head, lead, nvec, tail,
                        plan.roundTiles, plan.pieces, chunkShift);
@@ -422,23 +453,22 @@ hipError_t launchCompressed(const CompressedArgs& a, const float* raw, const Ptr
   return hipGetLastError();
 }
 
-template <typename WV, typename WS>
-hipError_t dispatchOut(const CompressedArgs& a, const float* raw, const Ptrs<0>& wire, int Kw,
-                       int rawPos, int64_t head, int64_t nvec, int64_t tail, int numCus,
-                       hipStream_t stream) {
+template <typename WV, typename WS, typename RAW>
+hipError_t dispatchOut(const CompressedArgs& a, const RAW& raw, bool hasRaw, uintptr_t leadRef,
+                       const Ptrs<0>& wire, int Kw, int rawPos, int64_t head, int64_t nvec,
+                       int64_t tail, int numCus, hipStream_t stream) {
   if (nvec > 0) {
     // the hook's own shapes: a raw fp32 bucket and 1, 3 or 7 peers, fp32 output,
     // no scale or the multiply by 1/K
-    if (a.out_dtype == FRG_F32 && raw != nullptr &&
+    if (a.out_dtype == FRG_F32 && hasRaw &&
         (a.scale_mode == FRG_SCALE_NONE || a.scale_mode == FRG_SCALE_MUL)) {
       const bool mul = a.scale_mode == FRG_SCALE_MUL;
-#define FRG_FIXED_CASE(KK)                                                                        \
-  case KK:                                                                                        \
-    return mul ? launchCompressed<WV, WS, true, KK, FRG_SCALE_MUL>(a, raw, wire, Kw, rawPos, head, \
-                                                                   nvec, tail, numCus, stream)     \
-               : launchCompressed<WV, WS, true, KK, FRG_SCALE_NONE>(a, raw, wire, Kw, rawPos,      \
-                                                                    head, nvec, tail, numCus,      \
-                                                                    stream);
+#define FRG_FIXED_CASE(KK)                                                                   \
+  case KK:                                                                                   \
+    return mul ? launchCompressed<WV, WS, true, KK, FRG_SCALE_MUL, RAW>(                     \
+                     a, raw, leadRef, wire, Kw, rawPos, head, nvec, tail, numCus, stream)    \
+               : launchCompressed<WV, WS, true, KK, FRG_SCALE_NONE, RAW>(                    \
+                     a, raw, leadRef, wire, Kw, rawPos, head, nvec, tail, numCus, stream);
       switch (Kw) {
         FRG_FIXED_CASE(1)
         FRG_FIXED_CASE(3)
@@ -449,16 +479,24 @@ hipError_t dispatchOut(const CompressedArgs& a, const float* raw, const Ptrs<0>&
 #undef FRG_FIXED_CASE
     }
     return a.out_dtype == FRG_F32
-               ? launchCompressed<WV, WS, true>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus,
-                                                stream)
-               : launchCompressed<WV, WS, false>(a, raw, wire, Kw, rawPos, head, nvec, tail,
-                                                 numCus, stream);
+               ? launchCompressed<WV, WS, true, 0, 0, RAW>(a, raw, leadRef, wire, Kw, rawPos, head,
+                                                           nvec, tail, numCus, stream)
+               : launchCompressed<WV, WS, false, 0, 0, RAW>(a, raw, leadRef, wire, Kw, rawPos,
+                                                            head, nvec, tail, numCus, stream);
   }
   // element-wise: pointers that cannot be brought to 16-byte boundaries by one
   // common head, or fewer elements than a group
   return a.out_dtype == FRG_F32
-             ? launchCompressed<WS, WS, true>(a, raw, wire, Kw, rawPos, 0, a.n, 0, numCus, stream)
-             : launchCompressed<WS, WS, false>(a, raw, wire, Kw, rawPos, 0, a.n, 0, numCus, stream);
+             ? launchCompressed<WS, WS, true, 0, 0, RAW>(a, raw, leadRef, wire, Kw, rawPos, 0, a.n,
+                                                         0, numCus, stream)
+             : launchCompressed<WS, WS, false, 0, 0, RAW>(a, raw, leadRef, wire, Kw, rawPos, 0,
+                                                          a.n, 0, numCus, stream);
+}
+
+// The raw term's address for element 0 of the launch if tensor `pc` went on
+// for ever in both directions (what RawPieces::adj holds).
+uintptr_t virtualOrigin(const RawPiece& pc) {
+  return reinterpret_cast<uintptr_t>(pc.ptr) - static_cast<uintptr_t>(pc.off) * 4;
 }
 
 }  // namespace
@@ -507,10 +545,33 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
   };
   want(o, outElsize);
 
+  const bool pieces = a.num_raw_pieces > 0;
+  if (pieces) {
+    if (a.raw_index < 0) return fail(FRG_ERR_INVALID, "raw pieces without a raw contribution");
+    if (a.num_raw_pieces > kMaxRawPieces || a.raw_pieces == nullptr) {
+      return fail(FRG_ERR_INVALID, "at most " + std::to_string(kMaxRawPieces) + " raw pieces per launch");
+    }
+    for (int i = 0; i < a.num_raw_pieces; ++i) {
+      const RawPiece& pc = a.raw_pieces[i];
+      const int64_t end = i + 1 < a.num_raw_pieces ? a.raw_pieces[i + 1].off : a.n;
+      if (pc.ptr == nullptr || reinterpret_cast<uintptr_t>(pc.ptr) % 4 != 0 || pc.off < 0 ||
+          pc.off >= end) {
+        return fail(FRG_ERR_INVALID, "bad raw piece " + std::to_string(i));
+      }
+      const uintptr_t lo = reinterpret_cast<uintptr_t>(pc.ptr);
+      const uintptr_t hi = lo + static_cast<uintptr_t>(end - pc.off) * 4;
+      if (lo < o + outBytes && o < hi) {
+        return fail(FRG_ERR_INVALID, "output overlaps raw piece " + std::to_string(i));
+      }
+      want(virtualOrigin(pc), 4);
+    }
+    if (a.raw_pieces[0].off != 0) return fail(FRG_ERR_INVALID, "the first raw piece starts at 0");
+  }
   Ptrs<0> wire;
   int Kw = 0;
   const float* raw = nullptr;
   for (int k = 0; k < a.K; ++k) {
+    if (pieces && k == a.raw_index) continue;  // given piecewise
     const uintptr_t p = reinterpret_cast<uintptr_t>(a.contribs[k]);
     if (p == 0) return fail(FRG_ERR_INVALID, "null contribution " + std::to_string(k));
     const uintptr_t elsize = k == a.raw_index ? 4 : 2;
@@ -530,7 +591,7 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
       wire.p[Kw++] = a.contribs[k];
     }
   }
-  for (int k = Kw; k < kMaxContribsPerLaunch; ++k) wire.p[k] = a.contribs[0];
+  for (int k = Kw; k < kMaxContribsPerLaunch; ++k) wire.p[k] = Kw > 0 ? wire.p[0] : a.out;
   // the own term goes in ahead of wire contribution rawPos
   const int rawPos = a.raw_index;
 
@@ -541,21 +602,78 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
     if (head > a.n) head = a.n;
     nvec = (a.n - head) / 8;
     tail = a.n - head - nvec * 8;
+    // a lane's group of 8 must lie within one tensor of the raw term
+    for (int i = 1; i < a.num_raw_pieces && pieces; ++i) {
+      const int64_t at = a.raw_pieces[i].off;
+      if (at > head && at < head + nvec * 8 && (at - head) % 8 != 0) vectorOk = false;
+    }
+    if (!vectorOk) head = nvec = tail = 0;
   }
 
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess) return fail(FRG_ERR_HIP, "hipGetDevice failed");
   const int numCus = computeUnits(device);
   hipError_t e;
-  if (a.wire_dtype == FRG_BF16) {
-    e = dispatchOut<Bf16Vec, Bf16Scalar>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus, stream);
+  if (pieces) {
+    RawPieces table;
+    for (int i = 0; i < kMaxRawPieces; ++i) {
+      const bool used = i < a.num_raw_pieces;
+      table.adj[i] = reinterpret_cast<const float*>(virtualOrigin(a.raw_pieces[used ? i : 0]));
+      table.off[i] = used ? a.raw_pieces[i].off : std::numeric_limits<long long>::max();
+    }
+    e = a.wire_dtype == FRG_BF16
+            ? dispatchOut<Bf16Vec, Bf16Scalar, RawPieces>(a, table, true, o, wire, Kw, rawPos, head,
+                                                          nvec, tail, numCus, stream)
+            : dispatchOut<F16Vec, F16Scalar, RawPieces>(a, table, true, o, wire, Kw, rawPos, head,
+                                                        nvec, tail, numCus, stream);
   } else {
-    e = dispatchOut<F16Vec, F16Scalar>(a, raw, wire, Kw, rawPos, head, nvec, tail, numCus, stream);
+    const RawPlain plain{raw};
+    const uintptr_t ref = reinterpret_cast<uintptr_t>(raw);
+    e = a.wire_dtype == FRG_BF16
+            ? dispatchOut<Bf16Vec, Bf16Scalar, RawPlain>(a, plain, raw != nullptr, ref, wire, Kw,
+                                                         rawPos, head, nvec, tail, numCus, stream)
+            : dispatchOut<F16Vec, F16Scalar, RawPlain>(a, plain, raw != nullptr, ref, wire, Kw,
+                                                       rawPos, head, nvec, tail, numCus, stream);
   }
   if (e != hipSuccess) {
     return fail(FRG_ERR_HIP, std::string("kernel launch failed: ") + hipGetErrorString(e));
   }
   return FRG_OK;
+}
+
+// Whether a launch over `n` elements at `out` / `contribs` can take the raw
+// term from these tensors at full speed (launchCompressedReduce takes them
+// either way; tensors that start within a lane's group of 8 elements, or off
+// the others' 16-byte phase, send it down the element-wise variant).
+bool rawPiecesVectorize(const void* out, int outDtype, const void* const* contribs, int K,
+                        int rawIndex, const RawPiece* pieces, int count, int64_t n) {
+  if (count < 1 || count > kMaxRawPieces) return false;
+  const uintptr_t outElsize = outDtype == FRG_F32 ? 4 : 2;
+  int64_t headWire = -1, headF32 = -1;
+  bool ok = true;
+  auto want = [&](uintptr_t p, uintptr_t elsize) {
+    const int64_t h = static_cast<int64_t>(((16 - (p & 15)) & 15) / elsize);
+    int64_t& slot = elsize == 2 ? headWire : headF32;
+    if (slot < 0) {
+      slot = h;
+    } else if (slot != h) {
+      ok = false;
+    }
+  };
+  want(reinterpret_cast<uintptr_t>(out), outElsize);
+  for (int k = 0; k < K; ++k) {
+    if (k != rawIndex) want(reinterpret_cast<uintptr_t>(contribs[k]), 2);
+  }
+  for (int i = 0; i < count; ++i) want(virtualOrigin(pieces[i]), 4);
+  if (headWire >= 0 && headF32 >= 0 && headWire % 4 != headF32) ok = false;
+  if (!ok) return false;
+  const int64_t head = headWire >= 0 ? headWire : headF32;
+  const int64_t nvec = n > head ? (n - head) / 8 : 0;
+  for (int i = 1; i < count; ++i) {
+    const int64_t at = pieces[i].off;
+    if (at > head && at < head + nvec * 8 && (at - head) % 8 != 0) return false;
+  }
+  return true;
 }
 
 }  // namespace frg

@@ -181,6 +181,15 @@ GridPlan planGrid(int64_t nvec, int numContribs, int numCus, int blocksPerCuHint
 // The reduction around torch's gradient-compression hooks: peers' tensors in
 // the wire type (bf16 or fp16), this rank's own fp32 buffer compressed in
 // registers, the result stored in the wire type or widened into fp32.
+// A tensor of the raw fp32 contribution and the element of the launch it starts at.
+struct RawPiece {
+  const void* ptr = nullptr;
+  int64_t off = 0;
+};
+constexpr int kMaxRawPiecesPerLaunch = 8;
+bool rawPiecesVectorize(const void* out, int outDtype, const void* const* contribs, int K,
+                        int rawIndex, const RawPiece* pieces, int count, int64_t n);
+
 struct CompressedArgs {
   void* out = nullptr;
   int out_dtype = 0;                      // FRG_F32 or the wire dtype
@@ -191,6 +200,11 @@ struct CompressedArgs {
   int wire_dtype = 0;  // FRG_BF16 / FRG_F16
   int scale_mode = 0;  // applied to the raw contribution after the cast: NONE / MUL / DIV
   float scale = 1.0f;
+  // The raw contribution in up to kMaxRawPiecesPerLaunch tensors instead of one
+  // buffer (contribs[raw_index] is then ignored): in order, the first at
+  // element 0, every one up to where the next starts (the last up to n).
+  const RawPiece* raw_pieces = nullptr;
+  int num_raw_pieces = 0;
   hipEvent_t startEvent = nullptr;
   hipEvent_t stopEvent = nullptr;
 };

@@ -1630,13 +1630,15 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
 // The reduction with a compression hook folded in, with the raw fp32
 // contribution still in the gradient tensors it is assembled from (what
 // torch's bf16 / fp16 compression hooks see with gradient_as_bucket_view=False
-// is a bucket that the reducer has just copied those tensors into): every
-// tensor is a launch of the compressed kernel of its own, or several for a
-// large one, with the tensor as the raw term and the output and the peers'
-// wire tensors at its offset in the bucket. The kernel takes the raw term by
-// its own pointer already (in place it is the output's), so this is the plain
-// compressed reduction cut where the gradients end; no table is involved, and
-// a tensor of a few KiB costs a launch, as the copy kernel it replaces did.
+// is a bucket that the reducer has just copied those tensors into). The bucket
+// is cut into launches as an assembled one would be (a bucket of 25 MiB: one),
+// and a launch reads its raw term from the tensors that lie in its range: up
+// to eight, by a table in the kernel arguments, provided every tensor starts
+// where a lane's group of 8 elements does and on the others' 16-byte phase
+// (layer sizes that are multiples of 8 and the allocator's alignment give
+// that); a launch whose tensors do not fit goes tensor by tensor, each a
+// launch with that tensor as its raw buffer, as the copy kernel it replaces
+// was.
 std::vector<hipStream_t> Context::runGatheredCompressed(
     const Request& req, const std::vector<hipEvent_t>& initialEvents) {
   const int64_t wireSize = elementSize(req.dtype);
@@ -1647,24 +1649,67 @@ std::vector<hipStream_t> Context::runGatheredCompressed(
   struct Part {
     int64_t off;  // in the bucket, elements
     int64_t len;
-    const void* raw;
+    std::vector<RawPiece> pieces;  // offsets counted from `off`
   };
+  // the tensors that hold anything, and where they start in the bucket
+  struct Tensor {
+    const float* ptr;
+    int64_t off, len;
+  };
+  std::vector<Tensor> tensors;
+  {
+    int64_t off = 0;
+    for (const Request::Segment& seg : req.gathered) {
+      if (seg.numel > 0) tensors.push_back(Tensor{static_cast<const float*>(seg.ptr), off, seg.numel});
+      off += seg.numel;
+    }
+  }
   std::vector<Part> parts;
   const int64_t quantum = kLaunchQuantumBytes / wireSize;
-  int64_t off = 0;
-  for (const Request::Segment& seg : req.gathered) {
-    if (seg.numel <= 0) continue;
-    const int64_t launchBytes = defaultCompressedLaunchBytes(
-        total, /*hasRaw=*/true, req.outDtype == FRG_F32, seg.numel * wireSize);
-    int64_t partLen = roundDownToNearestMultiple(launchBytes / wireSize, quantum);
-    if (partLen < quantum) partLen = quantum;
-    int64_t at = 0;
-    while (2 * (seg.numel - at) > 3 * partLen) {
-      parts.push_back(Part{off + at, partLen, static_cast<const float*>(seg.ptr) + at});
-      at += partLen;
+  int64_t partLen = roundDownToNearestMultiple(
+      defaultCompressedLaunchBytes(total, /*hasRaw=*/true, req.outDtype == FRG_F32,
+                                   req.numel * wireSize) / wireSize, quantum);
+  if (partLen < quantum) partLen = quantum;
+  std::vector<const void*> probe(static_cast<size_t>(total));
+  size_t ti = 0;  // first tensor that reaches into what is left
+  for (int64_t lo = 0; lo < req.numel;) {
+    int64_t hi = 2 * (req.numel - lo) > 3 * partLen ? lo + partLen : req.numel;
+    while (ti < tensors.size() && tensors[ti].off + tensors[ti].len <= lo) ++ti;
+    Part part;
+    part.off = lo;
+    for (size_t t = ti; t < tensors.size() && tensors[t].off < hi; ++t) {
+      if (static_cast<int>(part.pieces.size()) == kMaxRawPiecesPerLaunch) {
+        hi = tensors[t].off;  // the launch ends where the ninth tensor starts
+        break;
+      }
+      const int64_t from = tensors[t].off > lo ? tensors[t].off : lo;
+      part.pieces.push_back(RawPiece{tensors[t].ptr + (from - tensors[t].off), from - lo});
     }
-    parts.push_back(Part{off + at, seg.numel - at, static_cast<const float*>(seg.ptr) + at});
-    off += seg.numel;
+    part.len = hi - lo;
+    for (int k = 0; k < total; ++k) {
+      probe[static_cast<size_t>(k)] =
+          static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + lo * wireSize;
+    }
+    const bool fits =
+        part.pieces.size() == 1 ||
+        rawPiecesVectorize(static_cast<char*>(req.out) + lo * outSize, req.outDtype, probe.data(),
+                           total, g, part.pieces.data(), static_cast<int>(part.pieces.size()),
+                           part.len);
+    if (fits) {
+      parts.push_back(std::move(part));
+    } else {
+      // tensor by tensor
+      for (size_t i = 0; i < part.pieces.size(); ++i) {
+        const int64_t from = part.pieces[i].off;
+        const int64_t to = i + 1 < part.pieces.size() ? part.pieces[i + 1].off : part.len;
+        Part one;
+        one.off = lo + from;
+        one.len = to - from;
+        one.pieces.push_back(RawPiece{part.pieces[i].ptr, 0});
+        parts.push_back(std::move(one));
+      }
+    }
+    lo = hi;
   }
   const size_t nStreams = reduceStreams_.size();
   std::vector<char> initialsFired(initialEvents.size(), 0);
@@ -1701,10 +1746,14 @@ std::vector<hipStream_t> Context::runGatheredCompressed(
     lastIdx = si;
     for (int k = 0; k < total; ++k) {
       ptrs[static_cast<size_t>(k)] =
-          k == g ? part.raw
+          k == g ? part.pieces[0].ptr
                  : static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + part.off * wireSize;
     }
     CompressedArgs a;
+    if (part.pieces.size() > 1) {
+      a.raw_pieces = part.pieces.data();
+      a.num_raw_pieces = static_cast<int>(part.pieces.size());
+    }
     a.out = static_cast<char*>(req.out) + part.off * outSize;
     a.out_dtype = req.outDtype;
     a.contribs = ptrs.data();

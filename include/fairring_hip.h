@@ -371,8 +371,12 @@ FRG_API int frg_allreduce_compressed(frg_ctx* ctx, void* out, int out_dtype,
  * gradient_as_bucket_view=False, after the reducer has copied every gradient
  * into the bucket: torch:csrc/distributed/c10d/reducer.cpp, copy_grad_to_bucket):
  * contribution `raw_index` is read from `segments` (fp32, in bucket order,
- * lengths adding up to `numel`; contribs[raw_index] is ignored), every tensor
- * a launch of the compressed reduction of its own or, when large, several. */
+ * lengths adding up to `numel`; contribs[raw_index] is ignored). The bucket is
+ * cut into launches as an assembled one would be, and a launch reads its raw
+ * term from up to eight tensors through a table in its arguments, provided
+ * every tensor starts where a lane's group of 8 elements does and on the
+ * others' 16-byte phase (sizes that are multiples of 8, 16-byte aligned
+ * tensors); a launch whose tensors do not fit goes tensor by tensor. */
 FRG_API int frg_allreduce_compressed_gathered(frg_ctx* ctx, void* out, int out_dtype,
                                               const void* const* contribs, int K,
                                               int raw_index, const frg_segment* segments,

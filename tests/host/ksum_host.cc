@@ -106,7 +106,16 @@ struct CompressedJob {
   int64_t n;
   int scaleMode;
   float scale;
+  std::vector<RawPiece> pieces;  // the raw term in tensors of its own, when given
 };
+
+// the raw term of element i
+float rawAt(const CompressedJob* j, int64_t i) {
+  if (j->pieces.empty()) return static_cast<const float*>(j->in[static_cast<size_t>(j->rawIndex)])[i];
+  size_t s = 0;
+  while (s + 1 < j->pieces.size() && i >= j->pieces[s + 1].off) ++s;
+  return static_cast<const float*>(j->pieces[s].ptr)[i - j->pieces[s].off];
+}
 
 void runCompressedJob(void* p) {
   CompressedJob* j = static_cast<CompressedJob*>(p);
@@ -115,7 +124,7 @@ void runCompressedJob(void* p) {
     for (size_t k = 0; k < j->in.size(); ++k) {
       float t;
       if (static_cast<int>(k) == j->rawIndex) {
-        t = widen(narrow(static_cast<const float*>(j->in[k])[i]));
+        t = widen(narrow(rawAt(j, i)));
         if (j->scaleMode == FRG_SCALE_MUL) t = widen(narrow(t * j->scale));
         if (j->scaleMode == FRG_SCALE_DIV) t = widen(narrow(t / j->scale));
       } else {
@@ -142,11 +151,24 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
   if (a.wire_dtype != FRG_BF16) return fail(FRG_ERR_UNSUPPORTED, "host test build: bf16 wire only");
   if (a.K < 1 || a.K > kMaxContribsPerLaunch) return fail(FRG_ERR_INVALID, "K out of range");
   if (a.n == 0) return FRG_OK;
+  if (a.num_raw_pieces > kMaxRawPiecesPerLaunch) return fail(FRG_ERR_INVALID, "too many raw pieces");
   CompressedJob* j = new CompressedJob{a.out, a.out_dtype == FRG_F32, {}, a.raw_index,
-                                       a.n,   a.scale_mode,          a.scale};
+                                       a.n,   a.scale_mode,          a.scale, {}};
   for (int k = 0; k < a.K; ++k) j->in.push_back(a.contribs[k]);
+  for (int i = 0; i < a.num_raw_pieces; ++i) j->pieces.push_back(a.raw_pieces[i]);
   fake_hip_enqueue(stream, &runCompressedJob, j);
   return FRG_OK;
+}
+
+// the real rule's core: every tensor starts where a group of 8 elements does, on a 16-byte boundary
+bool rawPiecesVectorize(const void* out, int, const void* const*, int, int, const RawPiece* pieces,
+                        int count, int64_t) {
+  if (count < 1 || count > kMaxRawPiecesPerLaunch) return false;
+  if (reinterpret_cast<uintptr_t>(out) % 16 != 0) return false;
+  for (int i = 0; i < count; ++i) {
+    if (pieces[i].off % 8 != 0 || reinterpret_cast<uintptr_t>(pieces[i].ptr) % 16 != 0) return false;
+  }
+  return true;
 }
 
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err);

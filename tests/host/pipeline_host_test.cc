@@ -239,7 +239,32 @@ void scenarioPreScaleAndCompressed() {
     frg_work_release(w);
     frg_progress after = {};
     CHECK(frg_get_progress(ctx, &after) == FRG_OK);
-    CHECK(after.launches - before.launches == 4);  // one per tensor that holds anything
+    // a tensor that starts within a lane's group of 8 elements: tensor by tensor, one launch
+    // for each that holds anything
+    CHECK(after.launches - before.launches == 4);
+    // tensors that start where groups of 8 do (and on 16-byte boundaries): one launch reads
+    // all of them through its table
+    {
+      const int64_t even[5] = {0, 4096, 4104, 9000, n};
+      std::vector<Vec> parts;
+      std::vector<frg_segment> esegs;
+      for (int i = 0; i < 4; ++i) parts.emplace_back(rawAgain.begin() + even[i], rawAgain.begin() + even[i + 1]);
+      bool aligned = reinterpret_cast<uintptr_t>(bucket.data()) % 16 == 0;
+      for (const Vec& v : parts) {
+        esegs.push_back(frg_segment{v.data(), static_cast<int64_t>(v.size())});
+        aligned = aligned && reinterpret_cast<uintptr_t>(v.data()) % 16 == 0;
+      }
+      std::fill(bucket.begin(), bucket.end(), -3.f);
+      CHECK(frg_allreduce_compressed_gathered(ctx, bucket.data(), FRG_F32, gtab.data(), K, rawIndex,
+                                              esegs.data(), 4, n, FRG_BF16, FRG_SCALE_MUL, 0.2f,
+                                              nullptr, nullptr, nullptr, &w) == FRG_OK);
+      CHECK(frg_work_wait(w) == FRG_OK);
+      CHECK(same(bucket, want));
+      frg_work_release(w);
+      frg_progress last = {};
+      CHECK(frg_get_progress(ctx, &last) == FRG_OK);
+      if (aligned) CHECK(last.launches - after.launches == 1);
+    }
     // the piecewise contribution is the raw one, and its lengths must add up
     CHECK(frg_allreduce_compressed_gathered(ctx, bucket.data(), FRG_F32, gtab.data(), K, -1,
                                             segs.data(), 5, n, FRG_BF16, 0, 1.f, nullptr, nullptr,

@@ -210,6 +210,53 @@ def test_allreduce_gathered_waits_for_the_gradients_and_orders_what_follows():
 
 # ---- the compression hooks' reduction with the raw contribution in tensors of its own ---------
 
+# ten tensors that all start where a lane's group of 8 elements does: a launch reads up to
+# eight of them through its table
+ALIGNED_LAYER = [2048 * 2048, 2048, 2048, 2048 * 512, 2048, 8, 4096, 16, 2048 * 64 + 8, 24]
+
+
+@pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+@pytest.mark.parametrize("k,g", [(8, 0), (8, 5), (2, 1), (4, 3), (17, 9)])
+def test_allreduce_compressed_gathered_through_the_table(wire, tdt, k, g):
+    # Layer sizes that are multiples of 8 (and the allocator's alignment): the bucket is cut as
+    # an assembled one would be, and each launch reads its raw term from up to eight gradient
+    # tensors by a table in its arguments: two launches for these ten tensors. With the bucket
+    # and the peers 4 elements into a group of 8 (the groups then start 4 elements into every
+    # tensor) no launch takes the table, and every tensor is a launch of its own: ten.
+    rng = np.random.default_rng(171 * k + g)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    try:
+        lens = ALIGNED_LAYER
+        n = int(sum(lens))
+        for name, mode, omode, scale_of in SCALES[:3]:
+            for skew in (0, 4):
+                _print_case("compressed gathered, table", wire, k, g, name, skew)
+                x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+                bits = oracle.np_f32_to_bf16_rne(x) if wire == "bf16" else x.astype(np.float16).view(np.uint16)
+                host = [bits[j] for j in range(k)]
+                host[g] = x[g]
+                peers = [None if j == g else to_gpu(wire, bits[j], skew) for j in range(k)]
+                segs, off = [], 0
+                for ln in lens:
+                    segs.append(to_gpu("f32", x[g, off:off + ln], skew))
+                    off += ln
+                s = scale_of(k) if name != "mul" else float(np.float32(1) / np.float32(k))
+                out = torch.full((n + 16,), 7.0, device=DEV)[skew:skew + n]
+                before = dev.progress()["launches"]
+                dev.allreduce_compressed(out, peers, g, scale_mode=mode, scale=s, wire_dtype=tdt,
+                                         segments=segs).wait()
+                launches = dev.progress()["launches"] - before
+                if skew == 0:
+                    # (17 contributions: launches of about 80 MB cut the bucket in three)
+                    assert launches == (2 if k <= 8 else 4)
+                else:
+                    assert launches >= 10
+                want = oracle.compressed_sum(host, g, wire, omode, s)
+                assert_bits_equal(out.cpu().numpy(), want, "%s k=%d g=%d %s skew %d" % (wire, k, g, name, skew))
+    finally:
+        dev.close()
+
+
 @pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
 @pytest.mark.parametrize("k,g", [(8, 0), (8, 5), (2, 1), (4, 3), (17, 9)])
 def test_allreduce_compressed_gathered_vs_oracle(wire, tdt, k, g):
