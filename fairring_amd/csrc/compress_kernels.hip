@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <limits>
+#include <type_traits>
 
 #include "../../include/fairring_hip.h"
 #include "device_traits.h"
@@ -60,14 +61,34 @@ struct RawPlain {
 constexpr int kMaxRawPieces = 8;
 struct RawPieces {
   const float* adj[kMaxRawPieces];
-  long long off[kMaxRawPieces];  // off[0] = 0; unused entries hold the largest value
+  // off[0] = 0; unused entries hold the largest value. 32 bits (a launch of
+  // this kind has fewer than 2^31 elements): compares that the scalar unit has.
+  int off[kMaxRawPieces];
   __device__ __forceinline__ const float* origin(int64_t e) const {
+    const int e32 = static_cast<int>(e);
     const float* p = adj[0];
 #pragma unroll
-    for (int i = 1; i < kMaxRawPieces; ++i) p = e >= off[i] ? adj[i] : p;
+    for (int i = 1; i < kMaxRawPieces; ++i) p = e32 >= off[i] ? adj[i] : p;
     return p;
   }
 };
+
+// origin(e) for a lane of a wave whose accesses cover the `span` elements from
+// `waveFirst` on: nearly always one tensor holds them all, which two look-ups
+// on the scalar unit tell; only a wave that straddles tensors looks up per lane.
+template <typename RAW>
+__device__ __forceinline__ const float* rawOrigin(const RAW& raw, int64_t waveFirst, int span,
+                                                  int64_t e) {
+  if constexpr (sizeof(RAW) == sizeof(RawPlain)) {
+    return raw.origin(e);
+  } else {
+    const int first = __builtin_amdgcn_readfirstlane(static_cast<int>(waveFirst));
+    const float* a = raw.origin(first);
+    const float* b = raw.origin(first + span - 1);
+    if (a == b) return a;
+    return raw.origin(e);
+  }
+}
 
 template <typename RAW>
 __device__ __forceinline__ StagedChunks issueStaged(const RAW& raw, int64_t elemBase,
@@ -76,8 +97,8 @@ __device__ __forceinline__ StagedChunks issueStaged(const RAW& raw, int64_t elem
   const int64_t waveBase = elemBase + static_cast<int64_t>(lane - waveLane) * 8;
   const int64_t lo = waveBase + 4 * static_cast<int64_t>(waveLane);
   StagedChunks c;
-  c.lo = ldStream(reinterpret_cast<const f32x4*>(raw.origin(lo) + lo));
-  c.hi = ldStream(reinterpret_cast<const f32x4*>(raw.origin(lo + 256) + lo + 256));
+  c.lo = ldStream(reinterpret_cast<const f32x4*>(rawOrigin(raw, waveBase, 512, lo) + lo));
+  c.hi = ldStream(reinterpret_cast<const f32x4*>(rawOrigin(raw, waveBase, 512, lo + 256) + lo + 256));
   return c;
 }
 
@@ -212,7 +233,10 @@ __device__ __forceinline__ void compressedOne(void* out, const RAW& raw, const P
       st.lane = lane;
     } else {
       rawRegs = Side::load(
-          raw.origin(elemBase + static_cast<int64_t>(lane) * W::kLanes) + elemBase, lane);
+          rawOrigin(raw, elemBase + static_cast<int64_t>(lane - (lane & 63u)) * W::kLanes,
+                    64 * W::kLanes, elemBase + static_cast<int64_t>(lane) * W::kLanes) +
+              elemBase,
+          lane);
     }
   }
   int k = 0;
@@ -272,7 +296,10 @@ __device__ __forceinline__ void compressedFixed(float* out, const RAW& raw, cons
     chunks = issueStaged(raw, elemBase, lane);
   } else {
     rawRegs = Side::load(
-        raw.origin(elemBase + static_cast<int64_t>(lane) * W::kLanes) + elemBase, lane);
+        rawOrigin(raw, elemBase + static_cast<int64_t>(lane - (lane & 63u)) * W::kLanes,
+                  64 * W::kLanes, elemBase + static_cast<int64_t>(lane) * W::kLanes) +
+            elemBase,
+        lane);
   }
   vec_t v[KW];
 #pragma unroll
@@ -367,18 +394,39 @@ __global__ void __launch_bounds__(kBlock)
           ((t0 >> 3) & low);
     }
     const int64_t elemBase = bodyBase + t * kTile * WV::kLanes;
+    // one tile with the raw term read as `src` says
+    auto tile = [&](const auto& src) {
+      using SRC = std::remove_cv_t<std::remove_reference_t<decltype(src)>>;
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const unsigned int lane = threadIdx.x + u * kBlock;
-      if constexpr (kStaged && KW > 0) {
-        compressedFixed<WV, KW, SC, true, RAW>(static_cast<float*>(out), raw, wire, rawPos,
-                                               scale, elemBase, lane, stage);
-      } else if constexpr (kStaged) {
-        compressedOne<WV, OUT32, true, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale,
-                                            elemBase, lane, stage);
+      for (int u = 0; u < kUnroll; ++u) {
+        const unsigned int lane = threadIdx.x + u * kBlock;
+        if constexpr (kStaged && KW > 0) {
+          compressedFixed<WV, KW, SC, true, SRC>(static_cast<float*>(out), src, wire, rawPos,
+                                                 scale, elemBase, lane, stage);
+        } else if constexpr (kStaged) {
+          compressedOne<WV, OUT32, true, SRC>(out, src, wire, Kw, rawPos, scaleMode, scale,
+                                              elemBase, lane, stage);
+        } else {
+          compressedLane<WV, OUT32, KW, SC, SRC>(out, src, wire, Kw, rawPos, scaleMode, scale,
+                                                 elemBase, lane);
+        }
+      }
+    };
+    if constexpr (sizeof(RAW) == sizeof(RawPlain)) {
+      tile(raw);
+    } else {
+      // Nearly every tile lies within one tensor of the raw term: it then runs
+      // the very code of the one-buffer kernel, on that tensor's origin; only
+      // a tile that straddles tensors looks them up access by access. (With
+      // the look-ups in every tile's code, uniform as they were, the kernel ran
+      // 14 % slower: a launch lasts 20 us and starts with cold instruction
+      // caches.)
+      const float* a = raw.origin(elemBase);
+      const float* b = raw.origin(elemBase + kTile * WV::kLanes - 1);
+      if (a == b) {
+        tile(RawPlain{a});
       } else {
-        compressedLane<WV, OUT32, KW, SC, RAW>(out, raw, wire, Kw, rawPos, scaleMode, scale, elemBase,
-                                          lane);
+        tile(raw);
       }
     }
   }
@@ -548,6 +596,9 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
   const bool pieces = a.num_raw_pieces > 0;
   if (pieces) {
     if (a.raw_index < 0) return fail(FRG_ERR_INVALID, "raw pieces without a raw contribution");
+    if (a.n > std::numeric_limits<int>::max()) {
+      return fail(FRG_ERR_INVALID, "a launch with raw pieces takes fewer than 2^31 elements");
+    }
     if (a.num_raw_pieces > kMaxRawPieces || a.raw_pieces == nullptr) {
       return fail(FRG_ERR_INVALID, "at most " + std::to_string(kMaxRawPieces) + " raw pieces per launch");
     }
@@ -619,7 +670,7 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
     for (int i = 0; i < kMaxRawPieces; ++i) {
       const bool used = i < a.num_raw_pieces;
       table.adj[i] = reinterpret_cast<const float*>(virtualOrigin(a.raw_pieces[used ? i : 0]));
-      table.off[i] = used ? a.raw_pieces[i].off : std::numeric_limits<long long>::max();
+      table.off[i] = used ? static_cast<int>(a.raw_pieces[i].off) : std::numeric_limits<int>::max();
     }
     e = a.wire_dtype == FRG_BF16
             ? dispatchOut<Bf16Vec, Bf16Scalar, RawPieces>(a, table, true, o, wire, Kw, rawPos, head,
@@ -647,7 +698,7 @@ int launchCompressedReduce(const CompressedArgs& a, hipStream_t stream, std::str
 // the others' 16-byte phase, send it down the element-wise variant).
 bool rawPiecesVectorize(const void* out, int outDtype, const void* const* contribs, int K,
                         int rawIndex, const RawPiece* pieces, int count, int64_t n) {
-  if (count < 1 || count > kMaxRawPieces) return false;
+  if (count < 1 || count > kMaxRawPieces || n > std::numeric_limits<int>::max()) return false;
   const uintptr_t outElsize = outDtype == FRG_F32 ? 4 : 2;
   int64_t headWire = -1, headF32 = -1;
   bool ok = true;
