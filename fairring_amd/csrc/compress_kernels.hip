@@ -81,6 +81,10 @@ __device__ __forceinline__ const float* rawOrigin(const RAW& raw, int64_t waveFi
                                                   int64_t e) {
   if constexpr (sizeof(RAW) == sizeof(RawPlain)) {
     return raw.origin(e);
+  } else if (span < 512) {
+    // the element-wise variant: its lanes need not sit side by side (the
+    // scalars at a launch's two ends are reduced by one block)
+    return raw.origin(e);
   } else {
     const int first = __builtin_amdgcn_readfirstlane(static_cast<int>(waveFirst));
     const float* a = raw.origin(first);

@@ -260,6 +260,42 @@ def test_allreduce_compressed_gathered_through_the_table(wire, tdt, k, g):
 
 
 @pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+@pytest.mark.parametrize("k,g", [(8, 2), (4, 0), (5, 4)])
+def test_allreduce_compressed_gathered_table_with_scalar_ends(wire, tdt, k, g):
+    # The peers' wire tensors 8 bytes past a 16-byte boundary: a launch then has a head of 4
+    # scalar elements, its groups of 8 start 4 elements in, and the gradient tensors fit the
+    # table when they start there too (the first one 4 elements longer than a multiple of 8);
+    # 3 elements are left behind the last group. The scalars at both ends are reduced by lanes
+    # of one block that sit in different tensors.
+    rng = np.random.default_rng(191 * k + g)
+    lens = [2048 * 2048 + 4, 2048, 2048 * 512, 8, 2048 * 64 + 8 + 3]
+    n = int(sum(lens))
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    try:
+        for name, mode, omode, scale_of in SCALES[:2]:
+            _print_case("compressed gathered, table, scalar ends", wire, k, g, name)
+            x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+            bits = oracle.np_f32_to_bf16_rne(x) if wire == "bf16" else x.astype(np.float16).view(np.uint16)
+            host = [bits[j] for j in range(k)]
+            host[g] = x[g]
+            peers = [None if j == g else to_gpu(wire, bits[j], 4) for j in range(k)]
+            segs, off = [], 0
+            for ln in lens:
+                segs.append(to_gpu("f32", x[g, off:off + ln], 0))
+                off += ln
+            s = scale_of(k) if name != "mul" else float(np.float32(1) / np.float32(k))
+            out = torch.full((n + 16,), 7.0, device=DEV)[4:4 + n]
+            before = dev.progress()["launches"]
+            dev.allreduce_compressed(out, peers, g, scale_mode=mode, scale=s, wire_dtype=tdt,
+                                     segments=segs).wait()
+            assert dev.progress()["launches"] - before == 1
+            want = oracle.compressed_sum(host, g, wire, omode, s)
+            assert_bits_equal(out.cpu().numpy(), want, "%s k=%d g=%d %s" % (wire, k, g, name))
+    finally:
+        dev.close()
+
+
+@pytest.mark.parametrize("wire,tdt", [("bf16", torch.bfloat16), ("f16", torch.float16)])
 @pytest.mark.parametrize("k,g", [(8, 0), (8, 5), (2, 1), (4, 3), (17, 9)])
 def test_allreduce_compressed_gathered_vs_oracle(wire, tdt, k, g):
     # The raw fp32 contribution (rank g) as the gradient tensors of a layer, the peers'
