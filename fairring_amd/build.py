@@ -11,7 +11,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libfairring_hip.so")
 
-SOURCES = ["ksum_kernels.hip", "compress_kernels.hip", "static_scratch.hip", "pipeline.cc", "capi.cc"]
+SOURCES = ["ksum_kernels.hip", "compress_kernels.hip", "static_scratch.hip", "pipeline.cc",
+           "schedule_resident.cc", "schedule_gathered.cc", "schedule_host_staged.cc", "capi.cc"]
 
 # Bit-exactness depends on: no FMA contraction, IEEE fp32 division, fp32
 # denormals kept, and no packed-fp32 instructions.

@@ -1,5 +1,5 @@
 // The C ABI declared in include/fairring_hip.h: argument checks, error strings
-// and nothing else; the work is in pipeline.cc and ksum_kernels.hip.
+// and nothing else; the work is in pipeline.cc, the schedule_*.cc files and the kernels.
 #include <string>
 #include <vector>
 

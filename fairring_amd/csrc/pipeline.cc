@@ -6,50 +6,13 @@
 #include <stdexcept>
 
 #include "ksum_kernels.h"
+#include "pipeline_internal.h"
 
 namespace frg {
 
 namespace {
 
 thread_local std::string tlsError;
-
-struct HipFailure : std::runtime_error {
-  using std::runtime_error::runtime_error;
-};
-struct ContractFailure : std::runtime_error {
-  int code;
-  ContractFailure(int c, const std::string& m) : std::runtime_error(m), code(c) {}
-};
-
-// Throws on failure, like the reference's CUDA_CHECK (fairring/utils.h:35-45).
-#define FRG_HIP_CHECK(op)                                                        \
-  do {                                                                           \
-    hipError_t res_ = (op);                                                      \
-    if (res_ != hipSuccess) {                                                    \
-      (void)hipGetLastError();                                                   \
-      throw HipFailure(std::string("HIP error at ") + __FILE__ + ":" +           \
-                       std::to_string(__LINE__) + ": " + hipGetErrorString(res_)); \
-    }                                                                            \
-  } while (0)
-
-// Makes `device` current for the scope and restores the caller's device.
-class DeviceGuard {
- public:
-  explicit DeviceGuard(int device) {
-    FRG_HIP_CHECK(hipGetDevice(&prev_));
-    if (prev_ != device) {
-      FRG_HIP_CHECK(hipSetDevice(device));
-      changed_ = true;
-    }
-  }
-  ~DeviceGuard() {
-    if (changed_) (void)hipSetDevice(prev_);
-  }
-
- private:
-  int prev_ = 0;
-  bool changed_ = false;
-};
 
 }  // namespace
 
@@ -1001,56 +964,6 @@ void Context::launchSegments(const SegmentedArgs& args, hipStream_t stream) {
   if (rc != FRG_OK) throw ContractFailure(rc, err);
 }
 
-// The scratch region of a reduce stream (reused in stream order), placed so that the vector variant of the kernel still runs:
-// at the same position within 16 bytes as `like` for a buffer of the storage
-// type, or, for fp32 accumulators of a 2-byte type, such that it reaches a
-// 16-byte boundary after as many elements as `like` does.
-char* Context::scratchFor(size_t streamIdx, const void* like, bool acc, int64_t elsize) {
-  char* base = carryScratch_ + streamIdx * static_cast<size_t>(carryScratchBytes_ + 16);
-  return placeInScratch(base, like, acc, elsize);
-}
-
-// One part of a slice with more contributions than a launch takes, chained
-// through a scratch buffer in pieces of that buffer's size; only the last
-// launch of each piece writes `out`. Needed where `out` is itself one of the
-// contributions beyond the first launch's (the partial result must not land in
-// it early), and for bf16 / fp16 sums (`acc`: the partial sums stay in fp32).
-void Context::chainThroughScratch(const Request& req, const std::vector<const void*>& ptrs,
-                                  int64_t off, int64_t len, size_t streamIdx, bool acc) {
-  const int64_t elsize = elementSize(req.dtype);
-  const int total = static_cast<int>(ptrs.size());
-  hipStream_t s = reduceStreams_[streamIdx];
-  char* outBase = static_cast<char*>(req.out) + off * elsize;
-  char* scratch = scratchFor(streamIdx, acc ? ptrs[0] : outBase, acc, elsize);
-  const int64_t pieceLen = carryScratchBytes_ / (acc ? 4 : elsize);
-  std::vector<const void*> shifted(ptrs.size());
-  for (int64_t q = 0; q < len; q += pieceLen) {
-    const int64_t qlen = len - q < pieceLen ? len - q : pieceLen;
-    for (size_t k = 0; k < ptrs.size(); ++k) {
-      shifted[k] = static_cast<const char*>(ptrs[k]) + q * elsize;
-    }
-    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
-      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
-      const bool lastLaunch = k0 + kn == total;
-      ReduceArgs a;
-      a.out = lastLaunch ? outBase + q * elsize : scratch;
-      a.out_acc = acc && !lastLaunch;
-      a.contribs = shifted.data() + k0;
-      a.K = kn;
-      a.n = qlen;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
-                                                                        : FRG_SCALE_NONE;
-      a.scale = req.scale;
-      a.carry = k0 > 0;
-      a.carry_src = scratch;
-      a.carry_acc = acc;
-      launch(a, s);
-    }
-  }
-}
-
 // Start of the allocation that holds `p` (what hipMalloc returned for it), or 0
 // when the runtime does not know the pointer: physical memory is laid out from
 // there, so that is where the 4 MiB multiples that matter to the launch
@@ -1188,807 +1101,6 @@ void Context::waitInitial(hipStream_t stream, hipEvent_t initialEvent, bool* fir
     }
   }
   if (!*fired) FRG_HIP_CHECK(hipStreamWaitEvent(stream, initialEvent, 0));
-}
-
-// Device-resident contributions: the tensor is cut into launches of the launch
-// size (or one per slice of fairring/device.cc:315-326 when asked for), dealt
-// round-robin to the reduce streams so that neighbouring launches overlap.
-// Returns the streams the operation's work ended on.
-std::vector<hipStream_t> Context::runResident(const Request& req,
-                                              const std::vector<hipEvent_t>& initialEvents,
-                                              int64_t slices) {
-  const int64_t elsize = elementSize(req.dtype);
-  const int64_t nSlices =
-      slices >= 0 ? slices : numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
-  std::vector<char> initialsFired(initialEvents.size(), 0);
-  // the first launch on a stream follows every producer's event
-  auto waitInitials = [&](hipStream_t stream) {
-    for (size_t i = 0; i < initialEvents.size(); ++i) {
-      bool fired = initialsFired[i] != 0;
-      waitInitial(stream, initialEvents[i], &fired);
-      initialsFired[i] = fired ? 1 : 0;
-    }
-  };
-  const size_t nStreams = reduceStreams_.size();
-  std::vector<char> waited(nStreams, 0);
-  std::vector<const void*> ptrs(req.contribs.size());
-  const int total = static_cast<int>(ptrs.size());
-  // Launch size and grid go together (whole rounds of the grid); a size asked
-  // for by the caller leaves the grid to the kernel's own rule.
-  LaunchShape shape{maxLaunchBytes_, 0};
-  if (launchBytesByContribs_) {
-    shape = req.compressed
-                ? LaunchShape{defaultCompressedLaunchBytes(total, req.rawIndex >= 0,
-                                                           req.outDtype == FRG_F32,
-                                                           req.numel * elsize),
-                              0}
-                : defaultLaunchShape(total, req.numel * elsize);
-  }
-  const int64_t launchBytes = shape.bytes;
-  const int64_t maxLaunchElems = launchBytes > 0 ? launchBytes / elsize : 0;
-  size_t lastIdx = static_cast<size_t>(nextLaunch_) % nStreams;
-  // Reduced in place into a contribution that only a later launch of the chain
-  // reads: the partial result must not land in `out` before that.
-  bool lateAlias = false;
-  for (int k = kMaxContribsPerLaunch; k < total && !req.compressed; ++k) {
-    if (req.contribs[k] == req.out) lateAlias = true;
-  }
-  // A chain over bf16 / fp16 contributions keeps its partial sums in fp32
-  // between launches, so that it rounds once like a single launch.
-  const bool accChain = !req.compressed && total > kMaxContribsPerLaunch && req.op == FRG_SUM &&
-                        (req.dtype == FRG_BF16 || req.dtype == FRG_F16);
-
-  // Every slice takes its turn in the slot rotation (fairring/device.cc:482),
-  // but device-resident contributions need no slot, and the sum is elementwise:
-  // the launches need not follow the slice boundaries. The tensor is cut into
-  // launches of the launch size, on multiples of the kernel's 4 KiB tile from
-  // its start (a launch that starts off a tile boundary measured 8 % slower),
-  // whatever the slice size; the last launch takes up to one and a half times
-  // that. With the default layout (16 slices of 3.1 MiB in flight) launches cut
-  // at slice boundaries ran at 5.0 TB/s, these run at 6.3. A launch size of
-  // "whole slice" (max_launch_bytes < 0) keeps one launch per slice.
-  nextStagingSlot_ += nSlices;
-  struct Range {
-    int64_t first;   // offset in elements
-    int64_t second;  // length in elements
-    int blocksPerCu;
-    int64_t leadBytes;
-  };
-  std::vector<Range> ranges;
-  auto addRange = [&](int64_t off, int64_t len) {
-    ranges.push_back(Range{off, len, shape.blocksPerCu, -1});
-  };
-  const bool identity = !req.compressed && total == 1 && req.contribs[0] == req.out &&
-                        req.scaleMode == FRG_SCALE_NONE;
-  if (identity) {
-    // A lone contribution reduced in place: nothing to do (what the reference
-    // does for one machine and one device: device.cc:523,569).
-  } else if (maxLaunchElems <= 0) {
-    for (int64_t i = 0; i < nSlices; ++i) {
-      int64_t off, len;
-      sliceBounds(req.numel, layout_.sliceSizeInBytes, elsize, i, &off, &len);
-      addRange(off, len);
-    }
-  } else if (launchBytesByContribs_ && !req.compressed) {
-    // no launch size asked for: the library's own partition (layout.h)
-    const int numCus = computeUnits(device_);
-    const uint64_t outOffset = (reinterpret_cast<uint64_t>(req.out) - allocationBase(req.out)) %
-                               static_cast<uint64_t>(alignedRoundBytes(numCus));
-    const uint64_t first = reinterpret_cast<uint64_t>(req.contribs[0]);
-    const int64_t bytes = req.numel * elsize;
-    // A stream of short operations keeps one launch shape: they are aligned
-    // only once several in a row were cheap to align, and not again after one
-    // that is not until as many have been.
-    const bool shortOp = bytes / alignedRoundBytes(numCus) < kAlwaysAlignFromRounds;
-    if (shortOp) {
-      cheapStreak_ = alignmentIsCheap(outOffset, first, numCus) ? cheapStreak_ + 1 : 0;
-    }
-    const bool alignShort = cheapStreak_ > kAlignAfterStreak;
-    if (bytes != planBytes_ || outOffset != planOutOffset_ || first % kTileBytes != planFirst_ ||
-        total != planContribs_ || alignShort != planAlignShort_) {
-      plan_ = planDefaultLaunches(total, bytes, outOffset, first, numCus, alignShort);
-      planAlignShort_ = alignShort;
-      planBytes_ = bytes;
-      planOutOffset_ = outOffset;
-      planFirst_ = first % kTileBytes;
-      planContribs_ = total;
-    }
-    int64_t off = 0;
-    for (const LaunchPart& p : plan_) {
-      if (p.bytes > 0) ranges.push_back(Range{off, p.bytes / elsize, p.blocksPerCu, p.leadBytes});
-      off += p.bytes / elsize;
-    }
-  } else {
-    const int64_t quantum = kLaunchQuantumBytes / elsize;
-    int64_t partLen = roundDownToNearestMultiple(maxLaunchElems, quantum);
-    if (partLen < quantum) {  // launch sizes below a tile: 16-byte boundaries instead
-      partLen = roundUpToNearestMultiple(maxLaunchElems, 16 / elsize);
-    }
-    int64_t off = 0;
-    while (2 * (req.numel - off) > 3 * partLen) {
-      addRange(off, partLen);
-      off += partLen;
-    }
-    if (req.numel > off) addRange(off, req.numel - off);
-  }
-
-  // An operation of a few launches (a DDP bucket) stays on one stream and the
-  // next operation takes the next stream: neighbouring operations overlap, each
-  // ends on a single stream (nothing to join for its completion), and nothing is
-  // recorded between two launches. A large operation deals its own launches
-  // round-robin over the streams.
-  const bool oneStream = ranges.size() <= static_cast<size_t>(oneStreamLaunches_);
-  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
-  if (oneStream && !ranges.empty()) ++nextLaunch_;
-  const OpSpans spans = spansOf(req);
-  std::vector<size_t> targets;
-  if (!ranges.empty()) {
-    if (oneStream) {
-      targets.push_back(opStream);
-    } else {
-      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
-    }
-    orderAfterConflicts(spans, targets);
-  }
-
-  for (const auto& range : ranges) {
-    const int64_t off = range.first;
-    const int64_t len = range.second;
-    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
-    hipStream_t s = reduceStreams_[si];
-    if (!waited[si]) {
-      // Only the first launch on a stream needs the producer's event; later
-      // ones follow it in stream order (fairring/device.cc:334-336,507-509).
-      waitInitials(s);
-      waited[si] = 1;
-    }
-    for (size_t k = 0; k < ptrs.size(); ++k) {
-      const int64_t es = (req.compressed && static_cast<int>(k) == req.rawIndex) ? 4 : elsize;
-      ptrs[k] = static_cast<const char*>(req.contribs[k]) + off * es;
-    }
-    if (req.compressed) {
-      CompressedArgs a;
-      a.out = static_cast<char*>(req.out) + off * elementSize(req.outDtype);
-      a.out_dtype = req.outDtype;
-      a.contribs = ptrs.data();
-      a.K = total;
-      a.raw_index = req.rawIndex;
-      a.n = len;
-      a.wire_dtype = req.dtype;
-      a.scale_mode = req.scaleMode;
-      a.scale = req.scale;
-      launchCompressed(a, s);
-      lastIdx = si;
-      continue;
-    }
-    if (lateAlias || accChain) {
-      chainThroughScratch(req, ptrs, off, len, si, accChain);
-      lastIdx = si;
-      continue;
-    }
-    // More contributions than one launch takes: chain launches, carrying the
-    // partial result in `out`; the post-scale goes on the last one only.
-    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
-      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
-      const bool lastLaunch = k0 + kn == total;
-      ReduceArgs a;
-      a.out = static_cast<char*>(req.out) + off * elsize;
-      a.contribs = ptrs.data() + k0;
-      a.K = kn;
-      a.n = len;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      // a post-scale goes on the last launch only, a pre-scale on every one
-      a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
-                                                                        : FRG_SCALE_NONE;
-      a.scale = req.scale;
-      a.carry = k0 > 0;
-      a.blocks_per_cu = range.blocksPerCu;
-      a.lead_bytes = range.leadBytes;
-      launch(a, s);
-    }
-    lastIdx = si;
-  }
-  if (!ranges.empty()) {
-    std::vector<size_t> ran;
-    for (size_t si = 0; si < nStreams; ++si) {
-      if (waited[si]) ran.push_back(si);
-    }
-    remember(spans, ran);
-  }
-  // The streams that took part, the one of the last launch at the back.
-  if (!waited[lastIdx]) {
-    waitInitials(reduceStreams_[lastIdx]);
-    waited[lastIdx] = 1;
-  }
-  std::vector<hipStream_t> used;
-  for (size_t si = 0; si < nStreams; ++si) {
-    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
-  }
-  used.push_back(reduceStreams_[lastIdx]);
-  return used;
-}
-
-// One contribution given piecewise (a bucket's own gradients, each still in its
-// own tensor): the output is cut where the pieces end, every piece is an
-// elementwise reduction of its own (the output and the other contributions at
-// the piece's offset, the piece itself in the gathered contribution's place),
-// and the pieces are packed into segmented launches, cut on 4 KiB tiles of the
-// output, of about the size a plain operation's launches have. The copy of
-// every gradient into the bucket that DDP makes ahead of the allreduce
-// (torch:csrc/distributed/c10d/reducer.cpp, copy_grad_to_bucket) is thereby
-// part of the reduction: 8 bytes per element of HBM traffic less. A piece whose
-// pointers disagree modulo 16 (an odd-sized tensor ahead of it in the bucket),
-// and any reduction the segmented kernel does not cover (MAX, more than 16
-// contributions, other element types), runs as a plain launch of its own.
-std::vector<hipStream_t> Context::runGathered(const Request& req,
-                                              const std::vector<hipEvent_t>& initialEvents) {
-  if (req.compressed) return runGatheredCompressed(req, initialEvents);
-  const int64_t elsize = elementSize(req.dtype);
-  const int total = static_cast<int>(req.contribs.size());
-  const int g = req.gatheredIndex;
-  nextStagingSlot_ += numSlices(req.numel, layout_.sliceSizeInBytes, elsize);
-  const bool kindOk = segmentedKind(total, req.dtype, req.op, false);
-  const int maxSegs = maxSegmentsPerLaunch(total);
-  int64_t targetTiles = defaultLaunchShape(total, req.numel * elsize).bytes / kTileBytes;
-  if (targetTiles < 1) targetTiles = 1;
-  const bool accChain = total > kMaxContribsPerLaunch && req.op == FRG_SUM &&
-                        (req.dtype == FRG_BF16 || req.dtype == FRG_F16);
-
-  // A unit is one launch: several pieces through the segmented kernel, or one
-  // piece through the plain one.
-  struct Unit {
-    bool segmented = true;
-    std::vector<SegPiece> pieces;
-    int64_t off = 0;  // plain: offset of the piece in the output
-  };
-  std::vector<Unit> units;
-  std::deque<std::vector<const void*>> tables;  // the pieces' pointer tables stay put
-  auto tableOf = [&](const Request::Segment& seg, int64_t off) {
-    std::vector<const void*> tab(static_cast<size_t>(total));
-    for (int k = 0; k < total; ++k) {
-      tab[static_cast<size_t>(k)] =
-          k == g ? seg.ptr
-                 : static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + off * elsize;
-    }
-    return tab;
-  };
-  // Launches of `targetTiles` each, the last one with what is left over when
-  // that is less than half a launch's worth: a bucket of 25 MiB is 8 + 8 + 9
-  // MiB like a plain operation's, not three launches and a sliver.
-  int64_t segmentedTiles = 0;
-  {
-    int64_t off = 0;
-    for (const Request::Segment& seg : req.gathered) {
-      if (seg.numel <= 0) continue;
-      char* outp = static_cast<char*>(req.out) + off * elsize;
-      const std::vector<const void*> tab = tableOf(seg, off);
-      if (kindOk && segmentable(outp, tab.data(), total, elsize)) {
-        segmentedTiles += segmentTiles(outp, seg.numel, elsize);
-      }
-      off += seg.numel;
-    }
-  }
-  int64_t tilesLeft = segmentedTiles;  // not yet given to a launch
-  Unit cur;
-  int64_t curTiles = 0;
-  auto flush = [&] {
-    if (!cur.pieces.empty()) units.push_back(std::move(cur));
-    cur = Unit();
-    curTiles = 0;
-  };
-  int64_t off = 0;
-  for (const Request::Segment& seg : req.gathered) {
-    const int64_t len = seg.numel;
-    if (len <= 0) continue;
-    char* outp = static_cast<char*>(req.out) + off * elsize;
-    std::vector<const void*> tab = tableOf(seg, off);
-    if (!kindOk || !segmentable(outp, tab.data(), total, elsize)) {
-      flush();
-      tables.push_back(std::move(tab));
-      Unit plain;
-      plain.segmented = false;
-      plain.off = off;
-      plain.pieces.push_back(SegPiece{outp, tables.back().data(), len});
-      units.push_back(std::move(plain));
-      off += len;
-      continue;
-    }
-    const int64_t tiles = segmentTiles(outp, len, elsize);
-    for (int64_t t = 0; t < tiles;) {
-      int64_t take = tiles - t;
-      // a launch holds targetTiles, unless what would be left behind it is less
-      // than half a launch's worth: then it takes that too
-      const int64_t room = targetTiles - curTiles;
-      const bool openEnded = tilesLeft - room < targetTiles / 2;
-      if (!openEnded && take > room) take = room;
-      const int64_t e0 = segmentTileStart(outp, len, elsize, t);
-      const int64_t e1 = t + take == tiles ? len : segmentTileStart(outp, len, elsize, t + take);
-      std::vector<const void*> part(static_cast<size_t>(total));
-      for (int k = 0; k < total; ++k) {
-        part[static_cast<size_t>(k)] = static_cast<const char*>(tab[static_cast<size_t>(k)]) + e0 * elsize;
-      }
-      tables.push_back(std::move(part));
-      cur.pieces.push_back(SegPiece{outp + e0 * elsize, tables.back().data(), e1 - e0});
-      curTiles += take;
-      tilesLeft -= take;
-      t += take;
-      if ((!openEnded && curTiles >= targetTiles) ||
-          static_cast<int>(cur.pieces.size()) == maxSegs) {
-        flush();
-      }
-    }
-    off += len;
-  }
-  flush();
-
-  const size_t nStreams = reduceStreams_.size();
-  std::vector<char> initialsFired(initialEvents.size(), 0);
-  auto waitInitials = [&](hipStream_t stream) {
-    for (size_t i = 0; i < initialEvents.size(); ++i) {
-      bool fired = initialsFired[i] != 0;
-      waitInitial(stream, initialEvents[i], &fired);
-      initialsFired[i] = fired ? 1 : 0;
-    }
-  };
-  std::vector<char> waited(nStreams, 0);
-  const bool oneStream = units.size() <= static_cast<size_t>(oneStreamLaunches_);
-  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
-  size_t lastIdx = opStream;
-  if (oneStream && !units.empty()) ++nextLaunch_;
-  const OpSpans spans = spansOf(req);
-  if (!units.empty()) {
-    std::vector<size_t> targets;
-    if (oneStream) {
-      targets.push_back(opStream);
-    } else {
-      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
-    }
-    orderAfterConflicts(spans, targets);
-  }
-  for (const Unit& u : units) {
-    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
-    hipStream_t s = reduceStreams_[si];
-    if (!waited[si]) {
-      waitInitials(s);
-      waited[si] = 1;
-    }
-    lastIdx = si;
-    if (u.segmented && u.pieces.size() == 1) {
-      // A launch that holds one piece (a weight matrix fills whole launches on
-      // its own) is the plain kernel's: its pointers sit in registers from the
-      // start, where the segmented kernel first reads the table's prefix sums
-      // and then the piece's row (two dependent loads ahead of every block's
-      // first tile; 8 MiB launches of one piece: 3 % slower through the table).
-      const SegPiece& one = u.pieces[0];
-      ReduceArgs a;
-      a.out = one.out;
-      a.contribs = one.contribs;
-      a.K = total;
-      a.n = one.n;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = req.scaleMode;
-      a.scale = req.scale;
-      a.blocks_per_cu = 4;
-      launch(a, s);
-      continue;
-    }
-    if (u.segmented) {
-      SegmentedArgs a;
-      a.pieces = u.pieces.data();
-      a.numPieces = static_cast<int>(u.pieces.size());
-      a.K = total;
-      a.dtype = req.dtype;
-      a.scale_mode = req.scaleMode;
-      a.scale = req.scale;
-      launchSegments(a, s);
-      continue;
-    }
-    const SegPiece& pc = u.pieces[0];
-    if (accChain) {
-      std::vector<const void*> ptrs(pc.contribs, pc.contribs + total);
-      chainThroughScratch(req, ptrs, u.off, pc.n, si, true);
-      continue;
-    }
-    for (int k0 = 0; k0 < total; k0 += kMaxContribsPerLaunch) {
-      const int kn = total - k0 < kMaxContribsPerLaunch ? total - k0 : kMaxContribsPerLaunch;
-      const bool lastLaunch = k0 + kn == total;
-      ReduceArgs a;
-      a.out = pc.out;
-      a.contribs = pc.contribs + k0;
-      a.K = kn;
-      a.n = pc.n;
-      a.dtype = req.dtype;
-      a.op = req.op;
-      a.scale_mode = (lastLaunch || req.scaleMode >= FRG_SCALE_PRE_MUL) ? req.scaleMode
-                                                                        : FRG_SCALE_NONE;
-      a.scale = req.scale;
-      a.carry = k0 > 0;
-      launch(a, s);
-    }
-  }
-  if (!units.empty()) {
-    std::vector<size_t> ran;
-    for (size_t si = 0; si < nStreams; ++si) {
-      if (waited[si]) ran.push_back(si);
-    }
-    remember(spans, ran);
-  }
-  if (!waited[lastIdx]) {
-    waitInitials(reduceStreams_[lastIdx]);
-    waited[lastIdx] = 1;
-  }
-  std::vector<hipStream_t> used;
-  for (size_t si = 0; si < nStreams; ++si) {
-    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
-  }
-  used.push_back(reduceStreams_[lastIdx]);
-  return used;
-}
-
-// The reduction with a compression hook folded in, with the raw fp32
-// contribution still in the gradient tensors it is assembled from (what
-// torch's bf16 / fp16 compression hooks see with gradient_as_bucket_view=False
-// is a bucket that the reducer has just copied those tensors into). The bucket
-// is cut into launches as an assembled one would be (a bucket of 25 MiB: one),
-// and a launch reads its raw term from the tensors that lie in its range: up
-// to eight, by a table in the kernel arguments, provided every tensor starts
-// where a lane's group of 8 elements does and on the others' 16-byte phase
-// (layer sizes that are multiples of 8 and the allocator's alignment give
-// that); a launch whose tensors do not fit goes tensor by tensor, each a
-// launch with that tensor as its raw buffer, as the copy kernel it replaces
-// was.
-std::vector<hipStream_t> Context::runGatheredCompressed(
-    const Request& req, const std::vector<hipEvent_t>& initialEvents) {
-  const int64_t wireSize = elementSize(req.dtype);
-  const int64_t outSize = elementSize(req.outDtype);
-  const int total = static_cast<int>(req.contribs.size());
-  const int g = req.gatheredIndex;
-  nextStagingSlot_ += numSlices(req.numel, layout_.sliceSizeInBytes, wireSize);
-  struct Part {
-    int64_t off;  // in the bucket, elements
-    int64_t len;
-    std::vector<RawPiece> pieces;  // offsets counted from `off`
-  };
-  // the tensors that hold anything, and where they start in the bucket
-  struct Tensor {
-    const float* ptr;
-    int64_t off, len;
-  };
-  std::vector<Tensor> tensors;
-  {
-    int64_t off = 0;
-    for (const Request::Segment& seg : req.gathered) {
-      if (seg.numel > 0) tensors.push_back(Tensor{static_cast<const float*>(seg.ptr), off, seg.numel});
-      off += seg.numel;
-    }
-  }
-  std::vector<Part> parts;
-  const int64_t quantum = kLaunchQuantumBytes / wireSize;
-  int64_t partLen = roundDownToNearestMultiple(
-      defaultCompressedLaunchBytes(total, /*hasRaw=*/true, req.outDtype == FRG_F32,
-                                   req.numel * wireSize) / wireSize, quantum);
-  if (partLen < quantum) partLen = quantum;
-  std::vector<const void*> probe(static_cast<size_t>(total));
-  size_t ti = 0;  // first tensor that reaches into what is left
-  for (int64_t lo = 0; lo < req.numel;) {
-    int64_t hi = 2 * (req.numel - lo) > 3 * partLen ? lo + partLen : req.numel;
-    while (ti < tensors.size() && tensors[ti].off + tensors[ti].len <= lo) ++ti;
-    Part part;
-    part.off = lo;
-    for (size_t t = ti; t < tensors.size() && tensors[t].off < hi; ++t) {
-      if (static_cast<int>(part.pieces.size()) == kMaxRawPiecesPerLaunch) {
-        hi = tensors[t].off;  // the launch ends where the ninth tensor starts
-        break;
-      }
-      const int64_t from = tensors[t].off > lo ? tensors[t].off : lo;
-      part.pieces.push_back(RawPiece{tensors[t].ptr + (from - tensors[t].off), from - lo});
-    }
-    part.len = hi - lo;
-    for (int k = 0; k < total; ++k) {
-      probe[static_cast<size_t>(k)] =
-          static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + lo * wireSize;
-    }
-    const bool fits =
-        part.pieces.size() == 1 ||
-        rawPiecesVectorize(static_cast<char*>(req.out) + lo * outSize, req.outDtype, probe.data(),
-                           total, g, part.pieces.data(), static_cast<int>(part.pieces.size()),
-                           part.len);
-    if (fits) {
-      parts.push_back(std::move(part));
-    } else {
-      // tensor by tensor
-      for (size_t i = 0; i < part.pieces.size(); ++i) {
-        const int64_t from = part.pieces[i].off;
-        const int64_t to = i + 1 < part.pieces.size() ? part.pieces[i + 1].off : part.len;
-        Part one;
-        one.off = lo + from;
-        one.len = to - from;
-        one.pieces.push_back(RawPiece{part.pieces[i].ptr, 0});
-        parts.push_back(std::move(one));
-      }
-    }
-    lo = hi;
-  }
-  const size_t nStreams = reduceStreams_.size();
-  std::vector<char> initialsFired(initialEvents.size(), 0);
-  auto waitInitials = [&](hipStream_t stream) {
-    for (size_t i = 0; i < initialEvents.size(); ++i) {
-      bool fired = initialsFired[i] != 0;
-      waitInitial(stream, initialEvents[i], &fired);
-      initialsFired[i] = fired ? 1 : 0;
-    }
-  };
-  std::vector<char> waited(nStreams, 0);
-  const bool oneStream = parts.size() <= static_cast<size_t>(oneStreamLaunches_);
-  const size_t opStream = static_cast<size_t>(nextLaunch_) % nStreams;
-  size_t lastIdx = opStream;
-  if (oneStream && !parts.empty()) ++nextLaunch_;
-  const OpSpans spans = spansOf(req);
-  if (!parts.empty()) {
-    std::vector<size_t> targets;
-    if (oneStream) {
-      targets.push_back(opStream);
-    } else {
-      for (size_t si = 0; si < nStreams; ++si) targets.push_back(si);
-    }
-    orderAfterConflicts(spans, targets);
-  }
-  std::vector<const void*> ptrs(static_cast<size_t>(total));
-  for (const Part& part : parts) {
-    const size_t si = oneStream ? opStream : static_cast<size_t>(nextLaunch_++) % nStreams;
-    hipStream_t s = reduceStreams_[si];
-    if (!waited[si]) {
-      waitInitials(s);
-      waited[si] = 1;
-    }
-    lastIdx = si;
-    for (int k = 0; k < total; ++k) {
-      ptrs[static_cast<size_t>(k)] =
-          k == g ? part.pieces[0].ptr
-                 : static_cast<const char*>(req.contribs[static_cast<size_t>(k)]) + part.off * wireSize;
-    }
-    CompressedArgs a;
-    if (part.pieces.size() > 1) {
-      a.raw_pieces = part.pieces.data();
-      a.num_raw_pieces = static_cast<int>(part.pieces.size());
-    }
-    a.out = static_cast<char*>(req.out) + part.off * outSize;
-    a.out_dtype = req.outDtype;
-    a.contribs = ptrs.data();
-    a.K = total;
-    a.raw_index = g;
-    a.n = part.len;
-    a.wire_dtype = req.dtype;
-    a.scale_mode = req.scaleMode;
-    a.scale = req.scale;
-    launchCompressed(a, s);
-  }
-  if (!parts.empty()) {
-    std::vector<size_t> ran;
-    for (size_t si = 0; si < nStreams; ++si) {
-      if (waited[si]) ran.push_back(si);
-    }
-    remember(spans, ran);
-  }
-  if (!waited[lastIdx]) {
-    waitInitials(reduceStreams_[lastIdx]);
-    waited[lastIdx] = 1;
-  }
-  std::vector<hipStream_t> used;
-  for (size_t si = 0; si < nStreams; ++si) {
-    if (si != lastIdx && waited[si]) used.push_back(reduceStreams_[si]);
-  }
-  used.push_back(reduceStreams_[lastIdx]);
-  return used;
-}
-
-// Contributions in pinned host memory (server-side accumulation,
-// fairring/device.cc:543-589: collect into a staging slot, then reduce).
-// Contribution 0 lands directly in `out`; the later ones are copied into
-// staging slots and folded into `out` in index order.
-//
-// The pool's slots are split evenly among the staging streams (one by default,
-// which then owns the whole pool), and a stream works through its share batch
-// by batch: it copies a batch of contributions into its slots and then runs the
-// fold that reads them, so a slot is never overwritten before its last reader
-// has finished (the slot rule of device.cc:543-545,587-589) by stream order
-// alone. What crosses streams, when there are several, is the order of the
-// folds: each one waits for an event recorded behind the fold before it, when
-// that ran on another stream. (Two streams, each copying under the other's
-// fold, measured no faster than one: 53.9 against 54.3 GB/s. Two concurrent
-// host copies share the link and end together.)
-//
-// (The folds used to run on a reduce stream, with a "filled" event from the copy
-// stream to it and a "free" event back per slot. On MI355X / ROCm 7.2
-// hipMemcpyAsync then held the calling thread up for 0.2 to 0.45 ms per copy, up
-// to 11 ms, whenever the copy stream's last packet was such a wait, so the
-// command thread paced the copies one at a time: 64 contributions of 25 MiB
-// crossed the link at 46 to 50 GB/s. In this form the same call returns in 1.5
-// us and the link runs at 54 of the 56 GB/s that bare copies get on the same
-// box.)
-std::vector<hipStream_t> Context::runHostStaged(const Request& req, hipEvent_t initialEvent) {
-  const int64_t elsize = elementSize(req.dtype);
-  // A staged slice must fit a slot as well as the slice size.
-  int64_t sliceBytes =
-      layout_.sliceSizeInBytes < slotBytes_ ? layout_.sliceSizeInBytes : slotBytes_;
-  const int K = static_cast<int>(req.contribs.size());
-  hipStream_t s = reduceStreams_[0];
-  const std::vector<hipStream_t> all = copyStreams();  // created on first use
-  // the pool is split evenly among the staging streams: each fills its share, then folds it
-  int64_t batch = numSlots_ / static_cast<int64_t>(all.size());
-  if (batch < 1) batch = 1;
-  if (batch > kMaxContribsPerLaunch) batch = kMaxContribsPerLaunch;
-  const int64_t groups = numSlots_ / batch;
-  const size_t nStaging = static_cast<int64_t>(all.size()) < groups ? all.size()
-                                                                    : static_cast<size_t>(groups);
-  const std::vector<hipStream_t> staging(all.begin(), all.begin() + static_cast<long>(nStaging));
-  // The staging streams write `out` and the slots and know nothing of earlier
-  // operations: the whole operation is ordered after everything enqueued so far
-  // (it is bound by the host link; a few event packets do not show).
-  for (size_t src = 1; src < reduceStreams_.size(); ++src) {
-    if (!history_[src].empty()) joinTail(src, 0);
-  }
-  {
-    hipEvent_t tail = takeEvent();
-    hipError_t r = hipEventRecord(tail, s);
-    for (hipStream_t st : staging) {
-      if (r == hipSuccess) r = hipStreamWaitEvent(st, tail, 0);
-    }
-    giveEvent(tail);
-    FRG_HIP_CHECK(r);
-  }
-  bool initialFired = false;
-  for (hipStream_t st : staging) waitInitial(st, initialEvent, &initialFired);
-  // bf16 / fp16 sums folded in more than one batch keep their partial sums in
-  // fp32 between the launches (one rounding, like a single launch); the slices
-  // are then as short as the scratch buffer that holds those partial sums.
-  const bool accChain = req.op == FRG_SUM && (req.dtype == FRG_BF16 || req.dtype == FRG_F16) &&
-                        K - (req.carry ? 0 : 1) > batch;
-  if (accChain && sliceBytes > carryScratchBytes_ / 4 * elsize) {
-    sliceBytes = carryScratchBytes_ / 4 * elsize;
-  }
-  const int64_t nSlices = numSlices(req.numel, sliceBytes, elsize);
-
-  // The fold enqueued last, anywhere: the stream it ran on and an event behind it.
-  size_t lastFoldStream = nStaging;  // none yet
-  hipEvent_t lastFold = nullptr;
-  auto orderAfterLastFold = [&](size_t si) {
-    if (lastFold != nullptr && lastFoldStream != si) {
-      FRG_HIP_CHECK(hipStreamWaitEvent(staging[si], lastFold, 0));
-    }
-  };
-  auto foldEnqueued = [&](size_t si) {
-    giveEvent(lastFold);
-    lastFold = nullptr;
-    lastFold = takeEvent();
-    lastFoldStream = si;
-    FRG_HIP_CHECK(hipEventRecord(lastFold, staging[si]));
-  };
-  std::vector<char> took(nStaging, 0);
-  try {
-    for (int64_t i = 0; i < nSlices; ++i) {
-      int64_t off, len;
-      sliceBounds(req.numel, sliceBytes, elsize, i, &off, &len);
-      const size_t bytes = static_cast<size_t>(len * elsize);
-      char* outp = static_cast<char*>(req.out) + off * elsize;
-
-      int firstStaged = 0;
-      if (!req.carry) {
-        // Contribution 0 needs no staging: it lands in `out` directly, on the
-        // stream of the group that comes next, behind whatever fold wrote this
-        // part of `out` last (none within this operation: the slices are
-        // disjoint ranges; an earlier operation's is covered by the joins above).
-        const size_t si = static_cast<size_t>((nextStagingSlot_ / batch) % groups) % nStaging;
-        orderAfterLastFold(si);  // keeps the folds of all slices in one chain (they share the scratch)
-        FRG_HIP_CHECK(hipMemcpyAsync(outp,
-                                     static_cast<const char*>(req.contribs[0]) + off * elsize,
-                                     bytes, hipMemcpyHostToDevice, staging[si]));
-        took[si] = 1;
-        firstStaged = 1;
-        if (K == 1) {
-          if (req.scaleMode != FRG_SCALE_NONE) {
-            // nothing left to fold, but the post-scale is still owed
-            const void* self = outp;
-            ReduceArgs a;
-            a.out = outp;
-            a.contribs = &self;
-            a.K = 1;
-            a.n = len;
-            a.dtype = req.dtype;
-            a.op = req.op;
-            a.scale_mode = req.scaleMode;
-            a.scale = req.scale;
-            launch(a, staging[si]);
-          }
-          continue;
-        }
-        // the first fold of the slice reads what this copy wrote
-        giveEvent(lastFold);
-        lastFold = nullptr;
-        lastFold = takeEvent();
-        lastFoldStream = si;
-        FRG_HIP_CHECK(hipEventRecord(lastFold, staging[si]));
-      }
-
-      std::vector<const void*> staged;
-      char* accBuf = accChain ? scratchFor(0, outp, /*acc=*/true, elsize) : nullptr;
-      bool inAcc = false;  // the partial sum sits in accBuf (fp32), not in `out`
-      for (int k = firstStaged; k < K;) {
-        const int64_t group = (nextStagingSlot_ / batch) % groups;
-        nextStagingSlot_ += batch;  // the rotation of fairring/device.cc:482, a group at a time
-        const size_t si = static_cast<size_t>(group) % nStaging;
-        hipStream_t st = staging[si];
-        const int k0 = k;
-        const int kn = K - k < batch ? K - k : static_cast<int>(batch);
-        k += kn;
-        // Two streams that start their copies together share the link, finish
-        // together and then fold one after the other with the link idle (8 % of
-        // the time with 25 MiB slots). The first batch of every stream but the
-        // first therefore goes in two halves, copy and fold each: from then on
-        // that stream's copies end half a copy apart from its neighbour's, and
-        // one of them is always in flight.
-        int64_t cuts[3] = {0, len, len};
-        int parts = 1;
-        if (si > 0 && !took[si] && bytes >= (4u << 20)) {
-          cuts[1] = len / 2 / (kTileBytes / elsize) * (kTileBytes / elsize);
-          parts = 2;
-        }
-        took[si] = 1;
-        for (int part = 0; part < parts; ++part) {
-          const int64_t lo = cuts[part], hi = cuts[part + 1];
-          staged.clear();
-          for (int j = 0; j < kn; ++j) {
-            char* dst = stagingPool_ + (group * batch + j) * slotBytes_;
-            FRG_HIP_CHECK(hipMemcpyAsync(
-                dst + lo * elsize,
-                static_cast<const char*>(req.contribs[k0 + j]) + (off + lo) * elsize,
-                static_cast<size_t>((hi - lo) * elsize), hipMemcpyHostToDevice, st));
-            staged.push_back(dst + lo * elsize);
-          }
-          orderAfterLastFold(si);
-          ReduceArgs a;
-          a.out = outp + lo * elsize;
-          a.contribs = staged.data();
-          a.K = kn;
-          a.n = hi - lo;
-          a.dtype = req.dtype;
-          a.op = req.op;
-          a.scale_mode = k == K ? req.scaleMode : FRG_SCALE_NONE;
-          a.scale = req.scale;
-          a.carry = true;
-          if (accChain) {
-            a.carry_src = inAcc ? accBuf + lo * 4 : outp + lo * elsize;
-            a.carry_acc = inAcc;
-            if (k < K) {  // more batches follow
-              a.out = accBuf + lo * 4;
-              a.out_acc = true;
-            }
-          }
-          launch(a, st);
-          foldEnqueued(si);
-        }
-        if (accChain && k < K) inAcc = true;
-      }
-    }
-    // The operation ends on the first reduce stream, like any other: whatever
-    // comes later is ordered against that.
-    for (size_t si = 0; si < nStaging; ++si) {
-      if (!took[si]) continue;
-      hipEvent_t e = takeEvent();
-      hipError_t r = hipEventRecord(e, staging[si]);
-      if (r == hipSuccess) r = hipStreamWaitEvent(s, e, 0);
-      giveEvent(e);
-      FRG_HIP_CHECK(r);
-    }
-  } catch (...) {
-    giveEvent(lastFold);
-    throw;
-  }
-  giveEvent(lastFold);
-  if (req.numel > 0) remember(spansOf(req), {0});
-  return {s};
 }
 
 // Whether `next`, which was submitted right after `last`, continues it: the

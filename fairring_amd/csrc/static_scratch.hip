@@ -2,7 +2,7 @@
 // contributions on the caller's stream, for callers that cannot allocate (a
 // stream under HIP graph capture, a serving loop, a harness that forbids
 // hipMalloc). frg_allreduce chains the launches of more than 64 contributions
-// through a scratch buffer that the context allocates (pipeline.cc,
+// through a scratch buffer that the context allocates (schedule_resident.cc,
 // chainThroughScratch); here the same chain runs through an array that is part
 // of the library's device code, so the call allocates nothing.
 #include <hip/hip_runtime.h>

@@ -1,5 +1,5 @@
-// Host-logic tests of the slice pipeline (fairring_amd/csrc/pipeline.cc behind
-// the C ABI) on the fake HIP runtime: no GPU, meant to run under
+// Host-logic tests of the slice pipeline (fairring_amd/csrc/pipeline.cc and its
+// schedule_*.cc behind the C ABI) on the fake HIP runtime: no GPU, meant to run under
 // ThreadSanitizer and AddressSanitizer. Each scenario prints its name and
 // aborts on the first failed check.
 #include <hip/hip_runtime.h>

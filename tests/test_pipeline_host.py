@@ -21,6 +21,9 @@ SOURCES = [
     os.path.join(HOST, "ksum_host.cc"),
     os.path.join(HOST, "fake_hip", "fake_hip.cc"),
     os.path.join(ROOT, "fairring_amd", "csrc", "pipeline.cc"),
+    os.path.join(ROOT, "fairring_amd", "csrc", "schedule_resident.cc"),
+    os.path.join(ROOT, "fairring_amd", "csrc", "schedule_gathered.cc"),
+    os.path.join(ROOT, "fairring_amd", "csrc", "schedule_host_staged.cc"),
     os.path.join(ROOT, "fairring_amd", "csrc", "capi.cc"),
 ]
 
