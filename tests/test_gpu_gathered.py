@@ -334,6 +334,72 @@ def test_allreduce_compressed_gathered_vs_oracle(wire, tdt, k, g):
         dev.close()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_allreduce_compressed_gathered_random_layouts(seed):
+    # Random gradient tensors (between one and twelve, mostly multiples of 8 elements long,
+    # some not, some empty), random places of every buffer within 16 bytes, random group size,
+    # rank, wire type, scale and output type: launches that take their tensors through the
+    # table (with and without scalar ends, whole tiles and tiles that straddle tensors) and
+    # launches that fall back to a tensor each. Against the oracle, and for the launch count
+    # only that the result does not depend on it.
+    rng = np.random.default_rng(7000 + seed)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    through_table = tensor_each = 0
+    try:
+        for case in range(8):
+            k = int(rng.integers(1, 10))
+            g = int(rng.integers(0, k))
+            wire, tdt = [("bf16", torch.bfloat16), ("f16", torch.float16)][int(rng.integers(0, 2))]
+            name, mode, omode, scale_of = SCALES[int(rng.integers(0, 3))]
+            out_f32 = bool(rng.integers(0, 4) > 0)
+            pieces = int(rng.integers(1, 13))
+            tidy = bool(rng.integers(0, 3) > 0)          # two cases in three: everything lines up
+            base = int(rng.choice([0, 4])) if tidy else 0
+            lens = []
+            for i in range(pieces):
+                ln = 8 * int(rng.integers(1, 1 << int(rng.integers(4, 17))))
+                if i == 0:
+                    ln += base
+                if not tidy and rng.integers(0, 3) == 0:
+                    ln += int(rng.integers(-7, 8))
+                if rng.integers(0, 10) == 0:
+                    ln = 0 if i > 0 else ln
+                lens.append(max(ln, 0))
+            lens[-1] += int(rng.integers(0, 8))          # scalars behind the last group
+            n = int(sum(lens))
+            wskew = base if tidy else int(rng.integers(0, 8))
+            oskew = (base % 4 if out_f32 else base) if tidy else int(rng.integers(0, 4))
+            _print_case("compressed gathered, random", seed, case, wire, k, g, name, out_f32, tidy, lens)
+            x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+            bits = oracle.np_f32_to_bf16_rne(x) if wire == "bf16" else x.astype(np.float16).view(np.uint16)
+            host = [bits[j] for j in range(k)]
+            host[g] = x[g]
+            peers = [None if j == g else to_gpu(wire, bits[j], wskew) for j in range(k)]
+            segs, off = [], 0
+            for ln in lens:
+                segs.append(to_gpu("f32", x[g, off:off + ln], 0 if tidy else int(rng.integers(0, 4))))
+                off += ln
+            s = scale_of(k) if name != "mul" else float(np.float32(1) / np.float32(k))
+            if out_f32:
+                out = torch.full((n + 16,), 7.0, device=DEV)[oskew:oskew + n]
+            else:
+                out = torch.zeros(n + 16, dtype=tdt, device=DEV)[oskew:oskew + n]
+            before = dev.progress()["launches"]
+            dev.allreduce_compressed(out, peers, g, scale_mode=mode, scale=s, wire_dtype=tdt,
+                                     segments=segs).wait()
+            launches = dev.progress()["launches"] - before
+            filled = sum(1 for ln in lens if ln > 0)
+            through_table += int(filled > 1 and launches < filled)
+            tensor_each += int(filled > 1 and launches >= filled)
+            want = oracle.compressed_sum(host, g, wire, omode, s, out_f32=out_f32)
+            got = out.cpu().numpy() if out_f32 else from_gpu(wire, out)
+            assert_bits_equal(got, want, "seed %d case %d" % (seed, case))
+        print("through the table: %d, a tensor each: %d" % (through_table, tensor_each), flush=True)
+        assert through_table >= 1 and tensor_each >= 1     # both routes, for every seed here
+    finally:
+        dev.close()
+
+
 def test_allreduce_compressed_gathered_wire_output_and_contract():
     _print_case("compressed gathered: wire output, contract")
     rng = np.random.default_rng(9)
