@@ -448,12 +448,17 @@ __global__ void __launch_bounds__(kBlock)
 
 static_assert(static_cast<int64_t>(kBlock) * kUnroll == kSegmentTileVectors, "the tile of the kernels");
 
-template <typename TRV, typename TRS, int KT, int SC>
+// KT > 0: the number of contributions, fixed at compile time. KT == 0: any
+// number up to KCAP (8 or 16), which sizes the table's rows and with them the
+// number of pieces it holds: maxSegmentsPerLaunch(KCAP), which for every K is
+// what maxSegmentsPerLaunch(K) promises the callers.
+template <typename TRV, typename TRS, int KT, int SC, int KCAP = kMaxSegmentContribs>
 hipError_t launchSegmentedVariant(const SegmentedArgs& a, int numCus, hipStream_t stream) {
-  constexpr int KC = KT > 0 ? KT : kMaxSegmentContribs;
+  constexpr int KC = KT > 0 ? KT : KCAP;
   constexpr int S = maxSegmentsPerLaunch(KC);
   using Table = SegTable<KC, S>;
   static_assert(sizeof(Table) <= 3072, "the table travels in the kernel arguments");
+  if (a.K > KC) return hipErrorInvalidValue;
   Table tab = {};
   const int64_t elsize = static_cast<int64_t>(sizeof(typename TRV::elem_t));
   long long tiles = 0;
@@ -461,6 +466,7 @@ hipError_t launchSegmentedVariant(const SegmentedArgs& a, int numCus, hipStream_
   for (int i = 0; i < a.numPieces; ++i) {
     const SegPiece& pc = a.pieces[i];
     if (pc.n <= 0) continue;
+    if (nseg == S) return hipErrorInvalidValue;  // more pieces than the table holds
     const PieceSplit sp = splitPiece(pc.out, pc.n, elsize);
     tab.out[nseg] = pc.out;
     for (int k = 0; k < KC; ++k) tab.in[nseg][k] = pc.contribs[k < a.K ? k : 0];
@@ -510,13 +516,19 @@ hipError_t dispatchSegmented(const SegmentedArgs& a, int numCus, hipStream_t str
   FRG_SEG_CASE(2, FRG_SCALE_MUL, FRG_SCALE_MUL)
   FRG_SEG_CASE(2, FRG_SCALE_PRE_MUL, kPreMul)
 #undef FRG_SEG_CASE
+  // any other K or scale: the number of contributions at run time, in a table
+  // with rows of 8 (24 pieces) or of 16 (12 pieces)
+  const bool narrow = a.K <= 8;
   if (a.scale_mode == FRG_SCALE_PRE_MUL) {
-    return launchSegmentedVariant<TRV, TRS, 0, kPreMul>(a, numCus, stream);
+    return narrow ? launchSegmentedVariant<TRV, TRS, 0, kPreMul, 8>(a, numCus, stream)
+                  : launchSegmentedVariant<TRV, TRS, 0, kPreMul, 16>(a, numCus, stream);
   }
   if (a.scale_mode == FRG_SCALE_PRE_DIV) {
-    return launchSegmentedVariant<TRV, TRS, 0, kPreDiv>(a, numCus, stream);
+    return narrow ? launchSegmentedVariant<TRV, TRS, 0, kPreDiv, 8>(a, numCus, stream)
+                  : launchSegmentedVariant<TRV, TRS, 0, kPreDiv, 16>(a, numCus, stream);
   }
-  return launchSegmentedVariant<TRV, TRS, 0, -1>(a, numCus, stream);
+  return narrow ? launchSegmentedVariant<TRV, TRS, 0, -1, 8>(a, numCus, stream)
+                : launchSegmentedVariant<TRV, TRS, 0, -1, 16>(a, numCus, stream);
 }
 
 // FAST: also instantiate the compile-time-K variants (the gradient types);

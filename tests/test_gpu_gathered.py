@@ -83,6 +83,27 @@ def test_reduce_pieces_vs_oracle(kind, k):
                 kind, k, i, sizes[i], name), half=kind == "f16")
 
 
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+@pytest.mark.parametrize("k,scale", [(1, "none"), (3, "mul"), (5, "mul"), (7, "pre_mul"), (8, "div"),
+                                     (8, "pre_div"), (4, "div"), (9, "mul"), (16, "none")])
+def test_reduce_pieces_full_tables_at_every_group_size(kind, k, scale):
+    # 60 pieces that all fit the segmented kernel: launches with the table full (24 pieces up
+    # to 8 contributions, 12 beyond), also at group sizes and scales that have no variant of
+    # their own and share the one that takes the number of contributions at run time.
+    _print_case("pieces, full tables", kind, k, scale)
+    rng = np.random.default_rng(1000 * k + len(scale))
+    name, mode, omode, scale_of = [sc for sc in SCALES if sc[0] == scale][0]
+    per16 = 4 if kind == "f32" else 8
+    host = [host_values(kind, rng, (k, per16 * int(n))) for n in rng.integers(1, 700, size=60)]
+    pieces = [(torch.empty(x.shape[1], dtype=KINDS[kind], device=DEV), [to_gpu(kind, r) for r in x])
+              for x in host]
+    fa.reduce_pieces(pieces, scale_mode=mode, scale=scale_of(k))
+    torch.cuda.synchronize()
+    for i, ((out, _), x) in enumerate(zip(pieces, host)):
+        want = oracle.reduce(kind, list(x), "sum", omode, scale_of(k))
+        assert_bits_equal(from_gpu(kind, out), want, "piece %d" % i)
+
+
 def test_reduce_pieces_many_small_tensors_and_other_kinds():
     # more pieces than one launch takes; MAX and int32 go piece by piece through the plain kernel
     _print_case("pieces many")
@@ -176,6 +197,52 @@ def test_allreduce_gathered_misaligned_segments_other_reductions_and_the_copy_it
     with pytest.raises(fa.FairringError):
         dev.allreduce_gathered(out, peers, 69, segs[:-1])
     dev.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_allreduce_gathered_random_layouts(seed):
+    # Random gradient tensors (one to forty, from a few elements to a few MiB, some empty),
+    # every buffer at a random place within 16 bytes, random element type, group size, rank
+    # and scale: segmented launches of many pieces, single pieces as plain launches, pieces
+    # whose pointers disagree modulo 16. Against the oracle.
+    rng = np.random.default_rng(8000 + seed)
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    try:
+        for case in range(8):
+            kind = ["f32", "bf16", "f16"][int(rng.integers(0, 3))]
+            per16 = 4 if kind == "f32" else 8
+            k = int(rng.integers(1, 18))
+            g = int(rng.integers(0, k))
+            name, mode, omode, scale_of = SCALES[int(rng.integers(0, 5))]
+            tidy = bool(rng.integers(0, 2))
+            lens = []
+            for i in range(int(rng.integers(1, 41))):
+                ln = per16 * int(rng.integers(1, 1 << int(rng.integers(2, 19 if i < 3 else 14))))
+                if not tidy and rng.integers(0, 3) == 0:
+                    ln += int(rng.integers(-per16 + 1, per16))
+                if rng.integers(0, 10) == 0:
+                    ln = 0
+                lens.append(max(ln, 0))
+            if sum(lens) == 0:
+                lens[0] = 5
+            n = int(sum(lens))
+            _print_case("gathered, random", seed, case, kind, k, g, name, tidy, lens)
+            x = host_values(kind, rng, (k, n))
+            peers = [None if j == g else to_gpu(kind, x[j], 0 if tidy else int(rng.integers(0, per16)))
+                     for j in range(k)]
+            segs, off = [], 0
+            for ln in lens:
+                segs.append(to_gpu(kind, x[g, off:off + ln], 0 if tidy else int(rng.integers(0, per16))))
+                off += ln
+            oskew = 0 if tidy else int(rng.integers(0, per16))
+            out = torch.zeros(n + 16, dtype=KINDS[kind], device=DEV)[oskew:oskew + n]
+            dev.allreduce_gathered(out, peers, g, segs, scale_mode=mode, scale=scale_of(k)).wait()
+            want = oracle.reduce(kind, list(x), "sum", omode, scale_of(k))
+            assert_bits_equal(from_gpu(kind, out), want, "seed %d case %d" % (seed, case),
+                              half=kind == "f16")
+        assert dev.progress()["segmented_launches"] > 0
+    finally:
+        dev.close()
 
 
 def test_allreduce_gathered_waits_for_the_gradients_and_orders_what_follows():
