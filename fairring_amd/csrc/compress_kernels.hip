@@ -58,7 +58,7 @@ struct RawPlain {
   const float* base;
   __device__ __forceinline__ const float* origin(int64_t) const { return base; }
 };
-constexpr int kMaxRawPieces = 8;
+constexpr int kMaxRawPieces = kMaxRawPiecesPerLaunch;  // what the callers are told
 struct RawPieces {
   const float* adj[kMaxRawPieces];
   // off[0] = 0; unused entries hold the largest value. 32 bits (a launch of
