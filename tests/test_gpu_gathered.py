@@ -104,6 +104,42 @@ def test_reduce_pieces_full_tables_at_every_group_size(kind, k, scale):
         assert_bits_equal(from_gpu(kind, out), want, "piece %d" % i)
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_reduce_pieces_random_cases(seed):
+    # Random element type, number of contributions (1 to 20: beyond 16 every piece is a
+    # launch of its own), scale, number of pieces (1 to 70), and per piece a random length,
+    # a random place of every buffer within 16 bytes (tidy pieces share launches, the others
+    # go alone) and in place or not. Against the oracle.
+    rng = np.random.default_rng(9500 + seed)
+    for case in range(6):
+        kind = ["f32", "bf16", "f16"][int(rng.integers(0, 3))]
+        per16 = 4 if kind == "f32" else 8
+        k = int(rng.integers(1, 21))
+        name, mode, omode, scale_of = SCALES[int(rng.integers(0, 5))]
+        count = int(rng.integers(1, 71))
+        _print_case("pieces, random", seed, case, kind, k, name, count)
+        host, pieces = [], []
+        for i in range(count):
+            n = int(rng.integers(0, 1 << int(rng.integers(1, 16))))
+            x = host_values(kind, rng, (k, n))
+            tidy = rng.integers(0, 4) > 0
+            cs = [to_gpu(kind, x[j], 0 if tidy else int(rng.integers(0, per16))) for j in range(k)]
+            if rng.integers(0, 4) == 0:
+                out = cs[int(rng.integers(0, k))]
+            else:
+                out = torch.zeros(n + 16, dtype=KINDS[kind], device=DEV)
+                sk = 0 if tidy else int(rng.integers(0, per16))
+                out = out[sk:sk + n]
+            host.append(x)
+            pieces.append((out, cs))
+        fa.reduce_pieces(pieces, scale_mode=mode, scale=scale_of(k))
+        torch.cuda.synchronize()
+        for i, ((out, _), x) in enumerate(zip(pieces, host)):
+            want = oracle.reduce(kind, list(x), "sum", omode, scale_of(k))
+            assert_bits_equal(from_gpu(kind, out), want, "seed %d case %d piece %d" % (seed, case, i),
+                              half=kind == "f16")
+
+
 def test_reduce_pieces_many_small_tensors_and_other_kinds():
     # more pieces than one launch takes; MAX and int32 go piece by piece through the plain kernel
     _print_case("pieces many")

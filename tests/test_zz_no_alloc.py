@@ -181,3 +181,72 @@ def test_static_scratch_chain_captured_into_a_graph_and_replayed():
                                                            1.0 / k, threads=8), "oracle, replay %d" % replay)
     finally:
         dev.close()
+
+
+KINDS = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16, "f64": torch.float64,
+         "i32": torch.int32, "i64": torch.int64, "u8": torch.uint8}
+
+
+def _to_gpu(kind, a, skew):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if kind in ("bf16", "f16"):
+        t = t.view(torch.int16).view(KINDS[kind])
+    buf = torch.empty(a.size + skew + 16, dtype=KINDS[kind], device=DEV)
+    buf[skew:skew + a.size].copy_(t)
+    return buf[skew:skew + a.size]
+
+
+def _to_np(kind, t):
+    return bits16(t) if kind in ("bf16", "f16") else t.cpu().numpy()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_static_scratch_random_cases(seed):
+    # Random element type, reduction, scale, number of contributions (1 to 200: up to four
+    # launches chained through the static array), length, place of every buffer within 16
+    # bytes, and in place or not (also into a contribution beyond the first launch's). Against
+    # the oracle; consecutive cases share the array.
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(10):
+        kind = ["f32", "bf16", "f16", "f64", "i32", "i64", "u8"][int(rng.integers(0, 7))]
+        floating = kind in ("f32", "bf16", "f16", "f64")
+        op = "max" if rng.integers(0, 4) == 0 else "sum"
+        k = int(rng.integers(1, 201)) if rng.integers(0, 3) else int(rng.integers(1, 9))
+        n = int(rng.integers(1, 1 << int(rng.integers(1, 18))))
+        scale = "none"
+        if floating and op == "sum":
+            scale = ["none", "mul", "div", "premul", "prediv"][int(rng.integers(0, 5))]
+        modes = {"none": (fa.SCALE_NONE, oracle.SCALE_NONE, 1.0),
+                 "mul": (fa.SCALE_MUL, oracle.SCALE_MUL, float(np.float32(1) / np.float32(k))),
+                 "div": (fa.SCALE_DIV, oracle.SCALE_DIV, float(k)),
+                 "premul": (fa.SCALE_PRE_MUL, oracle.SCALE_PRE_MUL, float(np.float32(1) / np.float32(k))),
+                 "prediv": (fa.SCALE_PRE_DIV, oracle.SCALE_PRE_DIV, float(k))}
+        mode, omode, sc = modes[scale]
+        per16 = 16 // torch.empty(0, dtype=KINDS[kind]).element_size()
+        in_place = int(rng.integers(0, k)) if rng.integers(0, 3) == 0 else -1
+        print("[case] no-alloc entry point, random", seed, case, kind, op, scale, "k", k, "n", n,
+              "in place", in_place, flush=True)
+        if floating:
+            x = (rng.standard_normal((k, n)) * np.exp(rng.uniform(-3, 3, (k, n)))).astype(np.float32)
+            if kind == "bf16":
+                x = oracle.np_f32_to_bf16_rne(x).reshape(k, n)
+            elif kind == "f16":
+                x = x.astype(np.float16).view(np.uint16)
+            elif kind == "f64":
+                x = x.astype(np.float64)
+        else:
+            info = np.iinfo(oracle.TYPES[kind][0])
+            x = rng.integers(info.min, int(info.max) + 1, (k, n), dtype=oracle.TYPES[kind][0])
+        xs = [_to_gpu(kind, x[j], int(rng.integers(0, per16))) for j in range(k)]
+        room = None
+        if in_place >= 0:
+            out = xs[in_place]
+        else:
+            oskew = int(rng.integers(0, per16))
+            room = torch.zeros(n + 32, dtype=KINDS[kind], device=DEV)
+            out = room[oskew:oskew + n]
+        fa.reduce_slice_static(out, xs, op=fa.MAX if op == "max" else fa.SUM, scale_mode=mode, scale=sc)
+        torch.cuda.synchronize()
+        want = oracle.reduce(kind, list(x), op, omode, sc)
+        assert_bits_equal(_to_np(kind, out), want, "seed %d case %d" % (seed, case), half=kind == "f16")
+
