@@ -725,6 +725,42 @@ def run_c5sep(args, np, torch, fa, oracle):
         if not (owns[b].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all():
             raise SystemExit("parity FAILED on bucket %d (c5sep)" % b)
         checked.append(b)
+    # The same stream with peer copy j of every bucket starting j KiB into its allocation
+    # instead of at its start (still an allocation each): how much of this workload's rate is
+    # the relative position of the nine tensors of a bucket within 4 KiB, which a caller that
+    # owns the buffers the peers' contributions arrive in is free to choose.
+    staggered = None
+    if not args.numel:
+        peers_at_start = peers
+        peers = []
+        for b in range(buckets):
+            row = []
+            for j in range(1, k):
+                buf = torch.empty(n + 2048, device="cuda:0")
+                row.append(buf[256 * j:256 * j + n].copy_(peers_at_start[b][j - 1]))
+            peers.append(row)
+        torch.cuda.synchronize()
+        for _ in range(max(args.warmup, 1)):
+            finish(step())
+        pg._synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        pending = [step() for _ in range(steps)]
+        for works in pending:
+            finish(works)
+        pg._synchronize()
+        torch.cuda.synchronize()
+        staggered = (k + 1) * n * buckets * 4 * steps / (time.perf_counter() - t0) / 1e9
+        for t, f in zip(owns, fresh):
+            t.copy_(f)
+        finish(step())
+        pg._synchronize()
+        torch.cuda.synchronize()
+        for b in checked:
+            host = [fresh[b].cpu().numpy()] + [p.cpu().numpy() for p in peers[b]]
+            want = oracle.sum_f32(host, oracle.SCALE_MUL, 1.0 / k, threads=os.cpu_count() or 1)
+            if not (owns[b].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all():
+                raise SystemExit("parity FAILED on bucket %d (c5sep, staggered peers)" % b)
     layout = pg._layout()
     del pg
     cfg = {
@@ -738,6 +774,8 @@ def run_c5sep(args, np, torch, fa, oracle):
         "layout": {"slot": layout[0], "slice": layout[1], "padding_slots": layout[2],
                    "staging_slots": layout[3]},
     }
+    if staggered is not None:
+        cfg["peer_copy_j_starting_j_KiB_into_its_allocation_GBps"] = round(staggered, 1)
     return value, elapsed / 4, cfg, roof, checked, None, "f32"
 
 
