@@ -1252,7 +1252,9 @@ def main():
                                "dtype": r["dtype"], "pct_of_hbm_peak": r["pct_of_hbm_peak"],
                                "parity": r["parity"].split(";")[0], "roofline": roof}
                 for key in ("host_link_GBps", "copy_then_allreduce_GBps",
-                            "bf16_hook_from_grads_GBps", "bf16_hook_copy_then_allreduce_GBps"):
+                            "bf16_hook_from_grads_GBps", "bf16_hook_copy_then_allreduce_GBps",
+                            "tensors_at_the_start_of_their_allocation",
+                            "peer_copy_j_starting_j_KiB_into_its_allocation_GBps"):
                     if key in r["config"]:
                         extra[name][key] = r["config"][key]
             except (SystemExit, Exception) as e:  # noqa: BLE001  (reported, and the run fails)
