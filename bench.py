@@ -669,8 +669,10 @@ def run_c5sep(args, np, torch, fa, oracle):
     # slower for it. The record says how many tensors start their allocation.)
     fresh = [torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(buckets)]
     owns = [t.clone() for t in fresh]
-    peers = [[torch.empty(n, device="cuda:0").normal_(0.0, 0.01, generator=g) for _ in range(k - 1)]
-             for _ in range(buckets)]
+    # (8 KiB of room behind every peer copy, for the second placement below; the allocator rounds
+    # either size up to 26 MiB)
+    room = [[torch.empty(n + 2048, device="cuda:0") for _ in range(k - 1)] for _ in range(buckets)]
+    peers = [[buf[:n].normal_(0.0, 0.01, generator=g) for buf in row] for row in room]
     torch.cuda.synchronize()
     starts = {seg["address"] for seg in torch.cuda.memory_snapshot()}
     own_allocation = sum(t.data_ptr() in starts for row in [owns] + peers for t in row)
@@ -725,20 +727,14 @@ def run_c5sep(args, np, torch, fa, oracle):
         if not (owns[b].cpu().numpy().view(np.uint32) == want.view(np.uint32)).all():
             raise SystemExit("parity FAILED on bucket %d (c5sep)" % b)
         checked.append(b)
-    # The same stream with peer copy j of every bucket starting j KiB into its allocation
-    # instead of at its start (still an allocation each): how much of this workload's rate is
-    # the relative position of the nine tensors of a bucket within 4 KiB, which a caller that
-    # owns the buffers the peers' contributions arrive in is free to choose.
+    # The same stream in the same allocations with peer copy j of every bucket starting j KiB
+    # into its allocation instead of at its start: how much of this workload's rate is the
+    # relative position of the nine tensors of a bucket within 4 KiB, which a caller that owns
+    # the buffers the peers' contributions arrive in is free to choose.
     staggered = None
     if not args.numel:
-        peers_at_start = peers
-        peers = []
-        for b in range(buckets):
-            row = []
-            for j in range(1, k):
-                buf = torch.empty(n + 2048, device="cuda:0")
-                row.append(buf[256 * j:256 * j + n].copy_(peers_at_start[b][j - 1]))
-            peers.append(row)
+        peers = [[buf[256 * (j + 1):256 * (j + 1) + n].normal_(0.0, 0.01, generator=g)
+                  for j, buf in enumerate(row)] for row in room]
         torch.cuda.synchronize()
         for _ in range(max(args.warmup, 1)):
             finish(step())
