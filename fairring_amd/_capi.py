@@ -22,7 +22,7 @@ EXPORTS = (
     "frg_create", "frg_destroy", "frg_get_layout", "frg_get_streams", "frg_get_copy_streams", "frg_allreduce", "frg_allreduce_host",
     "frg_work_wait", "frg_set_wait_timeout", "frg_get_progress", "frg_get_progress2", "frg_allreduce_gathered", "frg_allreduce_compressed_gathered", "frg_reduce_pieces", "frg_work_is_completed", "frg_work_block_stream", "frg_work_release",
     "frg_synchronize", "frg_profile_mark", "frg_set_profiling", "frg_kernel_times", "frg_launch_records",
-    "frg_set_tuning", "frg_set_tile_runs",
+    "frg_set_tuning", "frg_set_tile_runs", "frg_set_mixed_loads",
     "frg_last_error", "frg_version",
 )
 
@@ -126,6 +126,7 @@ def lib():
     L.frg_launch_records.argtypes = [vp, ctypes.POINTER(LaunchRecord), i32, ctypes.POINTER(i32)]
     L.frg_set_tuning.argtypes = [i32]
     L.frg_set_tile_runs.argtypes = [i32]
+    L.frg_set_mixed_loads.argtypes = [i32]
     L.frg_last_error.restype = ctypes.c_char_p
     L.frg_version.restype = ctypes.c_char_p
     _lib = L

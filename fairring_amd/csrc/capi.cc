@@ -550,6 +550,12 @@ int frg_set_tile_runs(int log2_tiles) {
   return FRG_OK;
 }
 
+int frg_set_mixed_loads(int mode) {
+  if (mode < -1 || mode > 1) return fail(FRG_ERR_INVALID, "mode must be -1, 0 or 1");
+  frg::setMixedLoads(mode);
+  return FRG_OK;
+}
+
 const char* frg_last_error(void) { return frg::lastError(); }
 
 const char* frg_version(void) { return "0.3"; }

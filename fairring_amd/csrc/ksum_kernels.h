@@ -38,6 +38,12 @@ struct ReduceArgs {
   // pipeline starts the rounds where the output reaches a 4 MiB boundary of its
   // allocation.
   int64_t lead_bytes = -1;
+  // The whole tiles in the form that mixes the loads of a lane's two vectors
+  // (sums of 2, 4 or 8 contributions without a carry, no scale or the multiply
+  // by 1/K; ignored elsewhere): for an operation of bucket size, whose
+  // contributions tend to be allocations of their own that all start their
+  // allocation. Same result either way.
+  bool mixed_loads = false;
   // Optional timing events (created with timing enabled) that receive the
   // begin and end timestamps of this launch.
   hipEvent_t startEvent = nullptr;
@@ -163,6 +169,10 @@ void setTuning(int blocksPerCu);
 // default: 256 KiB; 0: tile = block index). For measurements.
 void setXcdChunkShift(int shift);
 int xcdChunkShift();
+// Which launches take the mixed form of the main loop: -1 (default) those whose
+// ReduceArgs ask for it, 0 none, 1 every launch that has the form. For
+// measurements and tests.
+void setMixedLoads(int mode);
 
 // Compute units of a device (cached).
 int computeUnits(int device);

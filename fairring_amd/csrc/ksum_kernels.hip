@@ -36,6 +36,14 @@ namespace {
 // log2 of the tiles in a row that the blocks of one XCD take (0: every eighth tile).
 int gXcdChunkShift = 6;
 
+// Which launches take the mixed form of the main loop (reduceTileMixed): -1 those
+// whose ReduceArgs ask for it, 0 none, 1 every launch that has the form.
+int gMixedLoads = -1;
+
+bool wantsMixedLoads(const ReduceArgs& a) {
+  return gMixedLoads < 0 ? a.mixed_loads : gMixedLoads > 0;
+}
+
 // Loads N contributions [k0, k0+N) at (base + lane), then folds them into acc
 // in index order. `first` makes contribution k0 initialise acc instead. With a
 // pre-scale (`pre` = FRG_SCALE_PRE_MUL / FRG_SCALE_PRE_DIV) every term is
@@ -184,6 +192,71 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
   stStream(TR::pack(acc), o);
 }
 
+// A lane's two vectors of a tile (kUnroll = 2; they lie 2 KiB apart) reduced
+// together, with the loads of both mixed: a first batch of KT loads takes the
+// lower half of the contributions at the first vector and the upper half at
+// the second, a second batch, issued once the first has landed, the rest. So
+// the loads a wave has in flight at any one time do not all sit at the same
+// position within 4 KiB. That matters when the contributions do: a bucket's
+// tensors that are allocations of their own all start their allocation, and
+// run through memory in step. The fold of each vector is still contribution 0
+// to KT-1 in order; all loads come before both stores, so an output that is one
+// of the contributions is read before it is written, as in reduceOne.
+template <typename TR, int KT, int SC>
+__device__ __forceinline__ void reduceTileMixed(typename TR::elem_t* out, const Ptrs<KT>& in,
+                                                float scale, int64_t elemBase, unsigned int tid) {
+  static_assert(kUnroll == 2 && KT >= 2 && KT % 2 == 0, "two vectors per lane, halves of KT");
+  using vec_t = typename TR::vec_t;
+  using elem_t = typename TR::elem_t;
+  using acc_t = typename TR::acc_t;
+  constexpr int H = KT / 2;
+  const unsigned int laneBytes[2] = {tid * static_cast<unsigned int>(sizeof(vec_t)),
+                                     (tid + kBlock) * static_cast<unsigned int>(sizeof(vec_t))};
+  auto ld = [&](int k, int u) {
+    const char* p = reinterpret_cast<const char*>(static_cast<const elem_t*>(in.p[k]) + elemBase);
+    const vec_t v = ldStream(reinterpret_cast<const vec_t*>(p + laneBytes[u]));
+    asm volatile("" ::: "memory");  // the loads stay in the order written
+    return v;
+  };
+  vec_t v0[KT], v1[KT];  // the lane's first and second vector of every contribution
+#pragma unroll
+  for (int k = 0; k < H; ++k) v0[k] = ld(k, 0);
+#pragma unroll
+  for (int k = H; k < KT; ++k) v1[k] = ld(k, 1);
+  // The second batch only when the first has landed: KT loads per wave in
+  // flight, as in the loop that takes one vector after the other (with all 2 KT
+  // issued at once the 8-way fp32 sum lost 1.5 to 2 %).
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int k = 0; k < H; ++k) {
+    v0[H + k] = ld(H + k, 0);
+    v1[k] = ld(k, 1);
+  }
+  const acc_t sc = static_cast<acc_t>(scale);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    acc_t acc[TR::kLanes];
+#pragma unroll
+    for (int k = 0; k < KT; ++k) {
+      acc_t f[TR::kLanes];
+      TR::unpack(u == 0 ? v0[k] : v1[k], f);
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = k == 0 ? f[j] : combine<FRG_SUM>(acc[j], f[j]);
+    }
+    if constexpr (TR::kFloating && SC == FRG_SCALE_MUL) {
+#pragma unroll
+      for (int j = 0; j < TR::kLanes; ++j) acc[j] = acc[j] * sc;
+    }
+    stStream(TR::pack(acc),
+             reinterpret_cast<vec_t*>(reinterpret_cast<char*>(out + elemBase) + laneBytes[u]));
+  }
+}
+
+// Whether a variant of the body kernel has the mixed form of its main loop.
+template <typename TR, int OP, int KT, int SC>
+constexpr bool kHasMixedLoads = OP == FRG_SUM && KT >= 2 && KT % 2 == 0 && kUnroll == 2 &&
+                                (SC == FRG_SCALE_NONE || SC == FRG_SCALE_MUL);
+
 // Body kernel. The slice is [head scalars][nvec vectors][tail scalars], where
 // `head` brings every pointer to a 16-byte boundary. The first `lead` vectors
 // are dealt in pieces of their own, so that the tiles start on a 4 KiB
@@ -197,7 +270,9 @@ __device__ __forceinline__ void reduceOne(typename TR::elem_t* out,
 // blocks on CUs round-robin, so spreading the remainder over twice as many
 // blocks in half-size pieces evens out the work per CU, and the launch does not
 // end on a few CUs finishing a whole extra tile.
-template <typename TRV, typename TRS, int OP, int KT, int SC>
+// MIXED: the whole tiles go through reduceTileMixed (a variant of its own, so
+// that neither form carries the other's code).
+template <typename TRV, typename TRS, int OP, int KT, int SC, bool MIXED = false>
 __global__ void __launch_bounds__(kBlock)
     ksumKernel(typename TRV::elem_t* out, Ptrs<KT> in, int K,
                const typename TRV::elem_t* carrySrc,
@@ -236,6 +311,8 @@ __global__ void __launch_bounds__(kBlock)
         reduceOne<TRV, OP, KT, SC>(out, in, K, carrySrc, scaleMode, scale, accFlags, elemBase,
                                    threadIdx.x + u * kBlock);
       }
+    } else if constexpr (MIXED) {
+      reduceTileMixed<TRV, KT, SC>(out, in, scale, elemBase, threadIdx.x);
     } else {
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
@@ -346,20 +423,26 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
       !a.carry ? nullptr
                : static_cast<const elem_t*>(a.carry_src != nullptr ? a.carry_src : a.out);
   const int accFlags = (a.carry && a.carry_acc ? kCarryIsAcc : 0) | (a.out_acc ? kOutIsAcc : 0);
-  if (a.startEvent != nullptr || a.stopEvent != nullptr) {
-    // Timed launch: the events take the dispatch's own begin/end timestamps.
-    hipExtLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
-                          dim3(kBlock), 0, stream, a.startEvent, a.stopEvent, 0,
-                          static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                          carrySrc, a.scale_mode, a.scale, accFlags, head, lead, nvec, tail, roundTiles, pieces,
-                          chunkShift);
-  } else {
-    hipLaunchKernelGGL((ksumKernel<TRV, TRS, OP, KT, SC>), dim3(static_cast<unsigned>(grid)),
-                       dim3(kBlock), 0, stream,
-                       static_cast<typename TRV::elem_t*>(a.out), tab, a.K,
-                       carrySrc, a.scale_mode, a.scale, accFlags, head, lead, nvec, tail, roundTiles, pieces,
-                       chunkShift);
+  auto launch = [&](auto kernel) {
+    if (a.startEvent != nullptr || a.stopEvent != nullptr) {
+      // Timed launch: the events take the dispatch's own begin/end timestamps.
+      hipExtLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, stream,
+                            a.startEvent, a.stopEvent, 0, static_cast<typename TRV::elem_t*>(a.out),
+                            tab, a.K, carrySrc, a.scale_mode, a.scale, accFlags, head, lead, nvec,
+                            tail, roundTiles, pieces, chunkShift);
+    } else {
+      hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0, stream,
+                         static_cast<typename TRV::elem_t*>(a.out), tab, a.K, carrySrc,
+                         a.scale_mode, a.scale, accFlags, head, lead, nvec, tail, roundTiles, pieces,
+                         chunkShift);
+    }
+  };
+  bool mixed = false;
+  if constexpr (kHasMixedLoads<TRV, OP, KT, SC>) mixed = wantsMixedLoads(a);
+  if constexpr (kHasMixedLoads<TRV, OP, KT, SC>) {
+    if (mixed) launch(&ksumKernel<TRV, TRS, OP, KT, SC, true>);
   }
+  if (!mixed) launch(&ksumKernel<TRV, TRS, OP, KT, SC, false>);
   return hipGetLastError();
 }
 
@@ -673,6 +756,7 @@ bool isFloating(int dtype) {
 void setTuning(int blocksPerCu) { gBlocksPerCu = blocksPerCu > 0 ? blocksPerCu : 0; }
 
 void setXcdChunkShift(int shift) { gXcdChunkShift = shift >= 0 && shift <= 12 ? shift : 0; }
+void setMixedLoads(int mode) { gMixedLoads = mode < 0 ? -1 : (mode > 0 ? 1 : 0); }
 int xcdChunkShift() { return gXcdChunkShift; }
 
 int launchSegmented(const SegmentedArgs& a, hipStream_t stream, std::string* err) {

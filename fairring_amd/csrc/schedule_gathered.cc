@@ -170,6 +170,7 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
       a.scale_mode = req.scaleMode;
       a.scale = req.scale;
       a.blocks_per_cu = 4;
+      a.mixed_loads = true;  // a bucket's tensors, allocations of their own: see runResident
       launch(a, s);
       continue;
     }

@@ -515,6 +515,20 @@ FRG_API int frg_set_tuning(int blocks_per_cu);
  * For measurements. */
 FRG_API int frg_set_tile_runs(int log2_tiles);
 
+/* Launch-shape knob of the reduction kernel: which launches run the form of
+ * the main loop that mixes the loads of a lane's two 16-byte vectors of a tile
+ * (half of the contributions at the first vector together with the other half
+ * at the second, 2 KiB further on, then the rest), so that the loads in flight
+ * do not all sit at the same position within 4 KiB. -1, the default: the
+ * launches of operations of bucket size (frg_allreduce* of up to 8 launches),
+ * whose contributions tend to be allocations of their own that all start
+ * their allocation and run through memory in step (8-way fp32, 25 MiB buckets
+ * allocated one by one: +1.8 %; a whole gradient of 5.5 GB per contribution:
+ * -1.4 %, hence the rule). 0: no launch. 1: every launch that has the form
+ * (sums of 2, 4 or 8 fp32 / bf16 / fp16 contributions, no scale or the
+ * multiply by 1/K). Results do not depend on it. For measurements. */
+FRG_API int frg_set_mixed_loads(int mode);
+
 /* Message of the last failure on the calling thread (or of the failed work). */
 FRG_API const char* frg_last_error(void);
 
@@ -522,8 +536,8 @@ FRG_API const char* frg_last_error(void);
  * frg_reduce_slice_static added (and frg_progress grew in place, which 0.3
  * takes back). 0.3: frg_progress has its four fields of 0.1 again and
  * frg_get_progress2 carries the later counters with the caller's struct size;
- * frg_allreduce_gathered, frg_allreduce_compressed_gathered, frg_reduce_pieces
- * and frg_set_tile_runs added. */
+ * frg_allreduce_gathered, frg_allreduce_compressed_gathered, frg_reduce_pieces,
+ * frg_set_tile_runs and frg_set_mixed_loads added. */
 FRG_API const char* frg_version(void);
 
 #ifdef __cplusplus

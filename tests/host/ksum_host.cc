@@ -40,6 +40,7 @@ bool isFloating(int dtype) {
 void setTuning(int) {}
 
 void setXcdChunkShift(int) {}
+void setMixedLoads(int) {}
 
 int computeUnits(int) { return 4; }  // what the stand-in runtime reports
 

@@ -1348,3 +1348,62 @@ def test_results_do_not_depend_on_the_tile_runs():
                 assert_bits_equal(bf16_bits(ob), wantb, "bf16 n=%d runs=%d" % (n, runs))
     finally:
         _capi.lib().frg_set_tile_runs(6)
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
+def test_results_do_not_depend_on_the_mixed_loads(kind):
+    # The form of the main loop that mixes the loads of a lane's two vectors (by default for
+    # operations of bucket size only) against the plain form, forced on and off for every
+    # launch: 2, 4 and 8 contributions (the variants that have it) and 3 (which has not), no
+    # scale and x1/K, off-boundary starts, in place into each contribution in turn (all loads
+    # come before both stores), one launch and the pipeline with a bucket and a long tensor.
+    _print_case("mixed loads", kind)
+    from fairring_amd import _capi
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[kind]
+    rng = np.random.default_rng(67)
+
+    def values(k, n):
+        x = (rng.standard_normal((k, n)) * 0.01).astype(np.float32)
+        if kind == "f32":
+            return x
+        if kind == "bf16":
+            return oracle.np_f32_to_bf16_rne(x).reshape(k, n)
+        return x.astype(np.float16).view(np.uint16)
+
+    def gpu(a, skew):
+        t = torch.from_numpy(np.ascontiguousarray(a))
+        if kind != "f32":
+            t = t.view(torch.int16).view(tdt)
+        buf = torch.empty(a.size + 16, dtype=tdt, device=DEV)
+        buf[skew:skew + a.size].copy_(t)
+        return buf[skew:skew + a.size]
+
+    def host(t):
+        return t.cpu().numpy() if kind == "f32" else t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    dev = fa.DeviceFairring(0, slice_size_in_bytes=25 * MiB, max_memory_allocated_in_bytes=50 * MiB)
+    try:
+        for k in (8, 4, 2, 3):
+            for n, skew in ((3 * 1024 * 1024 + 77, 0), (25 * MiB // 4, 1), (40 * MiB + 5, 0)):
+                x = values(k, n)
+                for mode, omode, sc in ((fa.SCALE_NONE, oracle.SCALE_NONE, 1.0),
+                                        (fa.SCALE_MUL, oracle.SCALE_MUL, 1.0 / k)):
+                    want = oracle.reduce(kind, list(x), "sum", omode, sc)
+                    for mixed in (1, 0, -1):
+                        _capi.check(_capi.lib().frg_set_mixed_loads(mixed))
+                        xs = [gpu(r, skew) for r in x]
+                        out = torch.zeros(n + 16, dtype=tdt, device=DEV)[skew:skew + n]
+                        fa.reduce_slice(out, xs, scale_mode=mode, scale=sc)
+                        torch.cuda.synchronize()
+                        what = "%s k=%d n=%d mixed=%d" % (kind, k, n, mixed)
+                        assert_bits_equal(host(out), want, what, half=kind == "f16")
+                        out.zero_()
+                        dev.allreduce(out, xs, scale_mode=mode, scale=sc).wait()
+                        assert_bits_equal(host(out), want, what + " pipeline", half=kind == "f16")
+                        j = int(rng.integers(0, k))       # in place into contribution j
+                        dev.allreduce(xs[j], xs, scale_mode=mode, scale=sc).wait()
+                        assert_bits_equal(host(xs[j]), want, what + " in place", half=kind == "f16")
+    finally:
+        _capi.lib().frg_set_mixed_loads(-1)
+        dev.close()
+
