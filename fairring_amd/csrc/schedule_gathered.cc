@@ -170,7 +170,7 @@ std::vector<hipStream_t> Context::runGathered(const Request& req,
       a.scale_mode = req.scaleMode;
       a.scale = req.scale;
       a.blocks_per_cu = 4;
-      a.mixed_loads = true;  // a bucket's tensors, allocations of their own: see runResident
+      a.mixed_loads = closelySpaced(one.contribs, total);  // see runResident
       launch(a, s);
       continue;
     }

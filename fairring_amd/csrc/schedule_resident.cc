@@ -199,6 +199,13 @@ std::vector<hipStream_t> Context::runResident(const Request& req,
     orderAfterConflicts(spans, targets);
   }
 
+  // Tensors that lie close to one another (a bucket's, allocated one by one)
+  // run through memory in step: their launches mix the loads of a lane's two
+  // vectors (8-way fp32, 48 buckets of 25 MiB: 6,45x GB/s against 6,37x). The
+  // tensors of a whole gradient, gigabytes apart, do better without (-1.4 %).
+  const bool mixedLoads =
+      total <= kMaxContribsPerLaunch && closelySpaced(req.contribs.data(), total);
+
   for (const auto& range : ranges) {
     const int64_t off = range.first;
     const int64_t len = range.second;
@@ -253,13 +260,7 @@ std::vector<hipStream_t> Context::runResident(const Request& req,
       a.carry = k0 > 0;
       a.blocks_per_cu = range.blocksPerCu;
       a.lead_bytes = range.leadBytes;
-      // An operation of bucket size: its tensors tend to be allocations of their
-      // own that all start their allocation (8-way fp32, 48 buckets of 25 MiB
-      // allocated one by one: 6,49x GB/s with the mixed loads against 6,37x; the
-      // buckets of one flat gradient handed over one at a time: no difference;
-      // a whole gradient, or buckets joined into a run: 1 to 1.4 % slower, and
-      // those are not `oneStream`).
-      a.mixed_loads = oneStream;
+      a.mixed_loads = mixedLoads;
       launch(a, s);
     }
     lastIdx = si;
