@@ -39,8 +39,8 @@ struct ReduceArgs {
   // allocation.
   int64_t lead_bytes = -1;
   // The whole tiles in the form that mixes the loads of a lane's two vectors
-  // (sums of 2, 4 or 8 contributions without a carry, no scale or the multiply
-  // by 1/K; ignored elsewhere): for contributions that lie close to one
+  // (sums of 2, 4 or 8 contributions without a carry; no scale, the multiply
+  // by 1/K or every term times 1/K; ignored elsewhere): for contributions that lie close to one
   // another (closelySpaced() below), which run through memory in step. Same
   // result either way.
   bool mixed_loads = false;

@@ -240,6 +240,11 @@ __device__ __forceinline__ void reduceTileMixed(typename TR::elem_t* out, const 
     for (int k = 0; k < KT; ++k) {
       acc_t f[TR::kLanes];
       TR::unpack(u == 0 ? v0[k] : v1[k], f);
+      if constexpr (TR::kFloating && SC == kPreMul) {
+        // every term scaled and rounded to the storage type first, as in foldChunk
+#pragma unroll
+        for (int j = 0; j < TR::kLanes; ++j) f[j] = TR::roundStorage(f[j] * sc);
+      }
 #pragma unroll
       for (int j = 0; j < TR::kLanes; ++j) acc[j] = k == 0 ? f[j] : combine<FRG_SUM>(acc[j], f[j]);
     }
@@ -255,7 +260,8 @@ __device__ __forceinline__ void reduceTileMixed(typename TR::elem_t* out, const 
 // Whether a variant of the body kernel has the mixed form of its main loop.
 template <typename TR, int OP, int KT, int SC>
 constexpr bool kHasMixedLoads = OP == FRG_SUM && KT >= 2 && KT % 2 == 0 && kUnroll == 2 &&
-                                (SC == FRG_SCALE_NONE || SC == FRG_SCALE_MUL);
+                                (SC == FRG_SCALE_NONE || SC == FRG_SCALE_MUL ||
+                                 (SC == kPreMul && TR::kFloating));
 
 // Body kernel. The slice is [head scalars][nvec vectors][tail scalars], where
 // `head` brings every pointer to a 16-byte boundary. The first `lead` vectors
@@ -438,7 +444,7 @@ hipError_t launchVariant(const ReduceArgs& a, int64_t head, int64_t nvec,
     }
   };
   bool mixed = false;
-  if constexpr (kHasMixedLoads<TRV, OP, KT, SC>) mixed = wantsMixedLoads(a);
+  if constexpr (kHasMixedLoads<TRV, OP, KT, SC>) mixed = wantsMixedLoads(a) && !a.carry;
   if constexpr (kHasMixedLoads<TRV, OP, KT, SC>) {
     if (mixed) launch(&ksumKernel<TRV, TRS, OP, KT, SC, true>);
   }

@@ -526,8 +526,9 @@ FRG_API int frg_set_tile_runs(int log2_tiles);
  * memory in step (8-way fp32: tensors 64 MiB apart +4.5 %, 512 MiB apart +2 %,
  * 1 GiB apart -3.5 %, the 5.5 GB tensors of a whole gradient -1.4 %, hence
  * the rule). 0: no launch. 1: every launch that has the form
- * (sums of 2, 4 or 8 fp32 / bf16 / fp16 contributions, no scale or the
- * multiply by 1/K). Results do not depend on it. For measurements. */
+ * (sums of 2, 4 or 8 fp32 / bf16 / fp16 contributions; no scale, the multiply
+ * by 1/K, or every term times 1/K). Results do not depend on it. For
+ * measurements. */
 FRG_API int frg_set_mixed_loads(int mode);
 
 /* Message of the last failure on the calling thread (or of the failed work). */

@@ -1353,10 +1353,11 @@ def test_results_do_not_depend_on_the_tile_runs():
 @pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
 def test_results_do_not_depend_on_the_mixed_loads(kind):
     # The form of the main loop that mixes the loads of a lane's two vectors (by default for
-    # operations of bucket size only) against the plain form, forced on and off for every
-    # launch: 2, 4 and 8 contributions (the variants that have it) and 3 (which has not), no
-    # scale and x1/K, off-boundary starts, in place into each contribution in turn (all loads
-    # come before both stores), one launch and the pipeline with a bucket and a long tensor.
+    # contributions that lie close together) against the plain form, forced on and off for
+    # every launch: 2, 4 and 8 contributions (the variants that have it) and 3 (which has not),
+    # no scale, x1/K and every term x1/K, off-boundary starts, in place into each contribution in
+    # turn (all loads come before both stores), one launch and the pipeline with a bucket and a
+    # long tensor.
     _print_case("mixed loads", kind)
     from fairring_amd import _capi
     tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[kind]
@@ -1387,7 +1388,9 @@ def test_results_do_not_depend_on_the_mixed_loads(kind):
             for n, skew in ((3 * 1024 * 1024 + 77, 0), (25 * MiB // 4, 1), (40 * MiB + 5, 0)):
                 x = values(k, n)
                 for mode, omode, sc in ((fa.SCALE_NONE, oracle.SCALE_NONE, 1.0),
-                                        (fa.SCALE_MUL, oracle.SCALE_MUL, 1.0 / k)):
+                                        (fa.SCALE_MUL, oracle.SCALE_MUL, 1.0 / k),
+                                        (fa.SCALE_PRE_MUL, oracle.SCALE_PRE_MUL,
+                                         float(np.float32(1) / np.float32(k)))):
                     want = oracle.reduce(kind, list(x), "sum", omode, sc)
                     for mixed in (1, 0, -1):
                         _capi.check(_capi.lib().frg_set_mixed_loads(mixed))
