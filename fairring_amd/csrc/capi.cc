@@ -149,6 +149,9 @@ int frg_reduce_slice(void* out, const void* const* contribs, int K, int64_t n, i
   a.scale_mode = scale_mode;
   a.scale = scale;
   a.carry = carry != 0;
+  // the pipeline's rule: tensors that lie close together take the mixed loads
+  a.mixed_loads = contribs != nullptr && K >= 1 && K <= frg::kMaxContribsPerLaunch &&
+                  frg::closelySpaced(contribs, K);
   std::string err;
   const int rc = frg::launchReduce(a, static_cast<hipStream_t>(stream), &err);
   if (rc != FRG_OK) return fail(rc, err);

@@ -520,12 +520,12 @@ FRG_API int frg_set_tile_runs(int log2_tiles);
  * (half of the contributions at the first vector together with the other half
  * at the second, 2 KiB further on, then the rest), so that the loads in flight
  * do not all sit at the same position within 4 KiB. -1, the default: the
- * launches of frg_allreduce* operations whose contributions lie close to one
- * another in the address space (median distance between neighbours below
- * 768 MiB: a bucket's tensors, allocated one by one), which run through
- * memory in step (8-way fp32: tensors 64 MiB apart +4.5 %, 512 MiB apart +2 %,
- * 1 GiB apart -3.5 %, the 5.5 GB tensors of a whole gradient -1.4 %, hence
- * the rule). 0: no launch. 1: every launch that has the form
+ * launches of frg_allreduce* and frg_reduce_slice whose contributions lie
+ * close to one another in the address space (median distance between
+ * neighbours below 768 MiB: a bucket's tensors, allocated one by one), which
+ * run through memory in step (8-way fp32: tensors 64 MiB apart +4.5 %, 512 MiB
+ * apart +2 %, 1 GiB apart -3.5 %, the 5.5 GB tensors of a whole gradient
+ * -1.4 %, hence the rule). 0: no launch. 1: every launch that has the form
  * (sums of 2, 4 or 8 fp32 / bf16 / fp16 contributions; no scale, the multiply
  * by 1/K, or every term times 1/K). Results do not depend on it. For
  * measurements. */
