@@ -6,6 +6,8 @@
 // folded in.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstring>
 #include <vector>
 
@@ -174,6 +176,10 @@ bool rawPiecesVectorize(const void* out, int, const void* const*, int, int, cons
 
 int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err);
 
+// Launches that asked for the mixed loads (the tests read it).
+std::atomic<long long> gMixedLoadLaunches{0};
+long long mixedLoadLaunches() { return gMixedLoadLaunches.load(); }
+
 // The segmented launch: every piece as a unit of work of its own, in order (the
 // packing into launches and the cuts on tiles are the pipeline's and are what is
 // under test; the real kernel's limits are checked here as it checks them).
@@ -225,6 +231,7 @@ int launchReduce(const ReduceArgs& a, hipStream_t stream, std::string* err) {
                    a.scale,
                    a.carry};
   for (int k = 0; k < a.K; ++k) j->in.push_back(static_cast<const float*>(a.contribs[k]));
+  if (a.mixed_loads) gMixedLoadLaunches.fetch_add(1);
   if (a.startEvent) hipEventRecord(a.startEvent, stream);
   fake_hip_enqueue(stream, &runJob, j);
   if (a.stopEvent) hipEventRecord(a.stopEvent, stream);

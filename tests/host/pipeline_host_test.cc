@@ -17,8 +17,13 @@
 #include <thread>
 #include <vector>
 
+#include "../../fairring_amd/csrc/ksum_kernels.h"
 #include "../../fairring_amd/csrc/layout.h"
 #include "../../include/fairring_hip.h"
+
+namespace frg {
+long long mixedLoadLaunches();  // of the stand-in for the kernels
+}
 
 // The default launch shapes, pinned: 48 MiB up to 2 contributions; 3 contributions
 // 12.5 MiB with the kernel's own grid, 20 MiB from 100 MiB per contribution; from 4
@@ -1115,6 +1120,53 @@ std::vector<hipStream_t> streamsOf(frg_ctx* ctx) {
   return v;
 }
 
+// Which launches are asked to mix the loads of a lane's two vectors: those of
+// operations whose contributions lie close to one another.
+void scenarioMixedLoadsRule() {
+  auto at = [](uint64_t a) { return reinterpret_cast<const void*>(a); };
+  const uint64_t MiBs = 1ull << 20, base = 0x7f0000000000ull;
+  {
+    const void* p[8];
+    for (int k = 0; k < 8; ++k) p[k] = at(base + k * 26 * MiBs);
+    CHECK(frg::closelySpaced(p, 8));  // a bucket's tensors, allocated one by one
+    for (int k = 0; k < 8; ++k) p[k] = at(base + k * 5480000000ull);
+    CHECK(!frg::closelySpaced(p, 8));  // the tensors of a whole gradient
+    for (int k = 1; k < 8; ++k) p[k] = at(base + k * 26 * MiBs);
+    p[0] = at(base + 40000 * MiBs);
+    CHECK(frg::closelySpaced(p, 8));  // the bucket far from its peers' copies, those side by side
+    p[3] = p[0];
+    CHECK(frg::closelySpaced(p, 8));  // an address twice (in place) counts once
+    CHECK(!frg::closelySpaced(p, 1));
+    const void* two[2] = {at(base), at(base + 512 * MiBs)};
+    CHECK(frg::closelySpaced(two, 2));
+    two[1] = at(base + 1024 * MiBs);
+    CHECK(!frg::closelySpaced(two, 2));
+    const void* same[2] = {at(base), at(base)};
+    CHECK(!frg::closelySpaced(same, 2));
+  }
+  // through the pipeline: host buffers lie megabytes apart
+  frg_options o = {};
+  o.max_memory_allocated_in_bytes = 2 << 20;
+  o.slice_size_in_bytes = 1 << 20;
+  frg_ctx* ctx = nullptr;
+  CHECK(frg_create(0, &o, &ctx) == FRG_OK);
+  const int64_t n = 300000;
+  std::vector<std::vector<float>> x(4, std::vector<float>(n, 1.0f));
+  std::vector<float> out(n, 0.0f);
+  const void* t[4] = {x[0].data(), x[1].data(), x[2].data(), x[3].data()};
+  const long long before = frg::mixedLoadLaunches();
+  frg_work* w = nullptr;
+  CHECK(frg_allreduce(ctx, out.data(), t, 4, n, FRG_F32, FRG_SUM, FRG_SCALE_NONE, 1.0f, nullptr,
+                      nullptr, nullptr, &w) == FRG_OK);
+  CHECK(frg_work_wait(w) == FRG_OK);
+  frg_work_release(w);
+  frg_progress pr = {};
+  CHECK(frg_get_progress(ctx, &pr) == FRG_OK);
+  CHECK(frg::mixedLoadLaunches() - before >= 1);
+  for (int64_t i = 0; i < n; i += 9973) CHECK(out[static_cast<size_t>(i)] == 4.0f);
+  CHECK(frg_destroy(ctx) == FRG_OK);
+}
+
 void scenarioStreamsAreReused() {
   std::puts("contexts created one after the other run on the same streams");
   frg_ctx* a = makeCtx(8192, 4096, 2, 0);
@@ -1656,6 +1708,7 @@ void runAll() {
       {"the null stream remembers its waits", scenarioNullStreamRemembersItsWaits},
       {"small operations on the caller's stream", scenarioSmallOperationsOnTheCallersStream},
       {"producer ordering", scenarioProducerOrdering},
+      {"mixed loads rule", scenarioMixedLoadsRule},
       {"streams are reused", scenarioStreamsAreReused},
       {"order between operations", scenarioOrderBetweenOperations},
       {"random dependent operations", scenarioRandomDependentOperations},
